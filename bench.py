@@ -1,0 +1,225 @@
+#!/usr/bin/env python3
+"""Benchmark of the Kronecker-matrix multiplication hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c1|c2|c3|c4|c5] [--tune] [--no-cpu]
+
+One "step" is one call of the C-ABI entry point (sgemkm / dgemkm / sgekmm / sgemkmStridedBatched) on a
+synthetic problem whose operands are already resident in HBM.  The default workload is c2, the
+configuration the headline metric is quoted on: sgemkm, X 1024 x 65536, four 16x16 factors.
+Prints ONE JSON line: GFLOP/s with FastKron's FLOP count (2*M*sum_i Kin_i*Q_i), the roofline of the
+dominant kernel measured with HIP events on the library's stream, and a CPU baseline (the oracle's
+vectorised OpenMP port) timed on the host cores in the same run.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0            # MI355X HBM3E
+FP64_PEAK_TFLOPS = 78.6          # MI355X fp64 (vector = matrix)
+
+# name: (call, M, Ps, Qs, dtype, alpha, beta, batch, bound)
+CONFIGS = {
+    "c1": ("sgemkm", 1024, [8] * 5, [8] * 5, "f32", 1.0, 0.0, 1, "hbm"),
+    "c2": ("sgemkm", 1024, [16] * 4, [16] * 4, "f32", 1.0, 0.0, 1, "hbm"),
+    "c3": ("dgemkm", 256, [64] * 3, [64] * 3, "f64", 1.0, 0.0, 1, "mfma"),
+    "c4": ("sgekmm", 2048, [4] * 6, [4] * 6, "f32", 1.5, 0.5, 1, "hbm"),
+    "c5": ("sgemkmStridedBatched", 512, [32] * 3, [16] * 3, "f32", 1.0, 1.0, 8, "hbm"),
+}
+
+
+def flop_count(M, Ps, Qs, batch):
+    kk, ops = int(np.prod(Ps)), 0
+    for p, q in zip(reversed(Ps), reversed(Qs)):
+        kk = kk // p * q
+        ops += kk * p
+    return 2 * M * ops * batch
+
+
+def compulsory_bytes(M, Ps, Qs, batch, esize, beta):
+    """Read X once, write Z once, read Y once when beta != 0, read the factors."""
+    K, L = int(np.prod(Ps)), int(np.prod(Qs))
+    b = M * K + M * L + (M * L if beta != 0 else 0)
+    return (b * batch + batch * sum(p * q for p, q in zip(Ps, Qs))) * esize
+
+
+class HipEvents:
+    """hipEvent timing on an explicit stream (the one handed to fastKronInitHIP)."""
+
+    def __init__(self):
+        self.hip = ctypes.CDLL("libamdhip64.so.7")
+        self.hip.hipEventElapsedTime.argtypes = [ctypes.POINTER(ctypes.c_float), ctypes.c_void_p, ctypes.c_void_p]
+        self.hip.hipEventRecord.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
+        self.hip.hipEventSynchronize.argtypes = [ctypes.c_void_p]
+
+    def create(self):
+        e = ctypes.c_void_p()
+        assert self.hip.hipEventCreate(ctypes.byref(e)) == 0
+        return e
+
+    def record(self, e, stream):
+        assert self.hip.hipEventRecord(e, stream) == 0
+
+    def elapsed_ms(self, e0, e1):
+        assert self.hip.hipEventSynchronize(e1) == 0
+        ms = ctypes.c_float()
+        assert self.hip.hipEventElapsedTime(ctypes.byref(ms), e0, e1) == 0
+        return ms.value
+
+
+def cpu_baseline(M, Ps, Qs, dt, alpha, beta, batch, budget_s):
+    """The oracle's OpenMP port on a bounded sample of the same workload: at most 256 rows of one
+    batch, repeated until about `budget_s` seconds of CPU work have been spent."""
+    from oracle import kron_oracle as ko
+    rows = min(M, 256)
+    rng = np.random.default_rng(0)
+    K, L = int(np.prod(Ps)), int(np.prod(Qs))
+    X = rng.uniform(-1, 1, size=(rows, K)).astype(dt)
+    Fs = [rng.uniform(-1, 1, size=(p, q)).astype(dt) for p, q in zip(Ps, Qs)]
+    Y = rng.uniform(-1, 1, size=(rows, L)).astype(dt) if beta != 0 else None
+    out = np.empty(rows * L, dtype=dt)
+    ko.sliced_multiply_fast(rows, Ps, Qs, X, Fs, alpha, beta, Y, out=out)       # warm-up, page in
+    best, spent, reps = float("inf"), 0.0, 0
+    while spent < budget_s and reps < 200:
+        t0 = time.perf_counter()
+        ko.sliced_multiply_fast(rows, Ps, Qs, X, Fs, alpha, beta, Y, out=out)
+        dtm = time.perf_counter() - t0
+        best = min(best, dtm)
+        spent += dtm
+        reps += 1
+    cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    gflops = flop_count(rows, Ps, Qs, 1) / best / 1e9
+    return {"value": round(gflops, 2), "unit": "GFLOP/s", "cores": cores, "kind": "port",
+            "sample": f"{rows} of {M * batch} rows, MKM form of the same factors, best of {reps} runs "
+                      f"({spent:.1f} s of CPU work)"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--config", default="c2", choices=sorted(CONFIGS))
+    ap.add_argument("--tune", action="store_true", help="time candidate launch plans first (excluded from timing)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-seconds", type=float, default=10.0)
+    ap.add_argument("--sets", type=int, default=2, help="operand sets rotated between steps")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU only (no multi-GPU path exists); use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import fastkron_amd
+    from fastkron_amd import capi
+
+    call, M, Ps, Qs, dts, alpha, beta, batch, bound = CONFIGS[args.config]
+    dt = np.float32 if dts == "f32" else np.float64
+    tdt = torch.float32 if dts == "f32" else torch.float64
+    esize = 4 if dts == "f32" else 8
+    K, L = int(np.prod(Ps)), int(np.prod(Qs))
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    stream = torch.cuda.current_stream()
+    fk = fastkron_amd.FastKron(stream=stream, tune=args.tune)
+    ye, te = fk.sizes(M, Ps, Qs)
+
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(0xFA57C0DE)
+
+    def uniform(n):
+        return torch.rand(n, generator=gen, device=dev, dtype=tdt) * 2 - 1
+
+    sets = []
+    for _ in range(args.sets):
+        X = uniform(batch * M * K)
+        Fs = [uniform(batch * p * q) for p, q in zip(Ps, Qs)]
+        Y = uniform(batch * M * L) if beta != 0 else None
+        Z = torch.empty(batch * ye, device=dev, dtype=tdt)
+        sets.append((X, Fs, Y, Z))
+    t1 = torch.empty(batch * te, device=dev, dtype=tdt)
+    t2 = torch.empty(batch * te, device=dev, dtype=tdt)
+
+    def step(i):
+        X, Fs, Y, Z = sets[i % len(sets)]
+        if call == "sgemkmStridedBatched":
+            e = fk.xgemkm_strided_batched(M, Ps, Qs, X, M * K, Fs, [p * q for p, q in zip(Ps, Qs)], Z, M * L, batch,
+                                          alpha, beta, Y, M * L, t1, t2)
+        elif call == "sgekmm":
+            e = fk.xgekmm(M, Ps, Qs, X, Fs, Z, alpha, beta, Y, t1, t2)
+        else:
+            e = fk.xgemkm(M, Ps, Qs, X, Fs, Z, alpha, beta, Y, t1, t2)
+        if e != capi.SUCCESS:
+            raise RuntimeError(f"{call} failed with fastKronError {e}")
+
+    for i in range(max(args.warmup, 1)):
+        step(i)
+    torch.cuda.synchronize()
+
+    ev = HipEvents()
+    sp = ctypes.c_void_p(stream.cuda_stream)
+    e0, e1 = ev.create(), ev.create()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ev.record(e0, sp)
+    for i in range(args.steps):
+        step(i)
+    ev.record(e1, sp)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    gpu_ms = ev.elapsed_ms(e0, e1)
+
+    ms_per_step = wall * 1e3 / args.steps
+    flop = flop_count(M, Ps, Qs, batch)
+    value = flop / (wall / args.steps) / 1e9
+
+    # Roofline of the dominant kernel.  The unit of work is "one factor applied to one row"; the
+    # algorithmic bytes of a unit are the call's compulsory bytes / (rows * factors), so the launches
+    # of one call add up to exactly the compulsory bytes.  Every launch of a call runs the same
+    # kernel family, hence: average launch duration = event time / launches, bytes per launch =
+    # compulsory bytes / launches.
+    plan = fk.last_plan()
+    launches = len(plan)
+    kernel_ms = gpu_ms / args.steps / launches
+    cbytes = compulsory_bytes(M, Ps, Qs, batch, esize, beta)
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "traffic.json")
+    if os.path.exists(tpath):
+        traffic = json.load(open(tpath)).get(args.config, {}).get("traffic_bytes_per_launch")
+    if bound == "hbm":
+        achieved = cbytes / launches / (kernel_ms * 1e-3) / 1e9
+        roof = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic}
+    else:
+        achieved = flop / launches / (kernel_ms * 1e-3) / 1e12
+        roof = {"bound": "mfma", "achieved": round(achieved, 2), "peak": FP64_PEAK_TFLOPS, "unit": "TFLOP/s",
+                "frac": round(achieved / FP64_PEAK_TFLOPS, 4), "traffic": traffic}
+    roof["kernel"] = sorted(set(k for _, _, k in plan))
+    roof["launches_per_step"] = launches
+    roof["kernel_ms"] = round(kernel_ms, 5)
+
+    out = {
+        "metric": "GeMKM/GeKMM GFLOP/s on 1 MI355X (FastKron FLOP count 2*M*sum Kin_i*Q_i)",
+        "value": round(value, 1), "unit": "GFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": dts, "data": "synthetic",
+        "config": {"workload": f"{args.config}: {call} M={M} factors={len(Ps)}x({Ps[0]}x{Qs[0]}) K={K} L={L} "
+                               f"alpha={alpha} beta={beta} batch={batch}, uniform[-1,1], seed 0xFA57C0DE",
+                   "operand_sets_rotated": args.sets, "tuned": bool(args.tune)},
+        "roofline": roof,
+        "gpu_ms_per_step_events": round(gpu_ms / args.steps, 5),
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(M, Ps, Qs, dt, alpha, beta, batch, args.cpu_seconds)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

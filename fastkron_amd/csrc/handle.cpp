@@ -1,0 +1,245 @@
+#include "handle.h"
+
+#include <algorithm>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+
+namespace fk {
+
+static int logLevel() {
+  static int lvl = -1;
+  if (lvl < 0) {
+    const char* e = getenv("FASTKRON_LOG");          // reference src/env/env.cpp:57-65
+    lvl = 0;
+    if (e && (!strcmp(e, "INFO") || !strcmp(e, "info"))) lvl = 1;
+    if (e && (!strcmp(e, "DEBUG") || !strcmp(e, "debug"))) lvl = 2;
+  }
+  return lvl;
+}
+
+Handle::Handle(uint32_t backends) : backends_(backends) {
+  dbPath_ = KernelDB::defaultPath();
+  if (!dbPath_.empty()) db_.loadFile(dbPath_);
+}
+
+Handle::~Handle() {}
+
+void Handle::setTunedDB(const char* path) {
+  dbPath_ = path ? path : "";
+  if (!dbPath_.empty()) db_.loadFile(dbPath_);
+}
+
+fastKronError Handle::ensureDevice() {
+  if (dev_.valid) return fastKronSuccess;
+  int d = 0;
+  if (hipGetDevice(&d) != hipSuccess) return fastKronBackendNotAvailable;
+  hipDeviceProp_t prop;
+  if (hipGetDeviceProperties(&prop, d) != hipSuccess) return fastKronBackendNotAvailable;
+  dev_.device = d;
+  dev_.cus = prop.multiProcessorCount;
+  dev_.ldsPerBlock = (int)prop.sharedMemPerBlock;
+  dev_.waveSize = prop.warpSize;
+  dev_.clockKHz = prop.clockRate;
+  strncpy(dev_.arch, prop.gcnArchName, sizeof(dev_.arch) - 1);
+  dev_.valid = true;
+  if (logLevel() >= 1)
+    printf("[fastkron] device %d %s: %d CUs, %d B LDS per workgroup, wave %d, %d kHz\n", d, dev_.arch,
+           dev_.cus, dev_.ldsPerBlock, dev_.waveSize, dev_.clockKHz);
+  return fastKronSuccess;
+}
+
+fastKronError Handle::initHIP(void* ptrToStream) {
+  if (!hasBackend(fastKronBackend_HIP)) return fastKronBackendNotAvailable;
+  stream_ = ptrToStream ? *(hipStream_t*)ptrToStream : nullptr;
+  hipInit_ = true;
+  return ensureDevice();
+}
+
+fastKronError Handle::setStream(fastKronBackend backend, void* ptrToStream) {
+  if (!ptrToStream) return fastKronInvalidArgument;                    // reference handle.cpp:94
+  if (!hasBackend(backend)) return fastKronBackendNotAvailable;        // reference handle.cpp:95
+  if (backend != fastKronBackend_HIP) return fastKronBackendNotAvailable;
+  stream_ = *(hipStream_t*)ptrToStream;
+  return fastKronSuccess;
+}
+
+// Columns of every step's output, widths[i] for the step of factor i.
+static void stepWidths(uint32_t N, const uint32_t* Ps, const uint32_t* Qs, uint64_t* widths) {
+  uint64_t w = 1;
+  for (uint32_t i = 0; i < N; i++) w *= Ps[i];
+  for (int i = (int)N - 1; i >= 0; i--) { w = (w / Ps[i]) * Qs[i]; widths[i] = w; }
+}
+
+// reference src/handle/handle.cpp:305-342,375-388: the temporary holds the widest step output
+// (X itself is not counted), except for N == 1 where it is max(K, L) columns.
+fastKronError Handle::sizes(uint32_t M, uint32_t N, const uint32_t* Ps, const uint32_t* Qs,
+                            size_t* yElems, size_t* tmpElems) {
+  if (!yElems || !tmpElems) return fastKronInvalidArgument;
+  if (N == 0 || N > kMaxFactors || !Ps || !Qs) return fastKronInvalidKMMProblem;
+  uint64_t K = 1, L = 1;
+  for (uint32_t i = 0; i < N; i++) { K *= Ps[i]; L *= Qs[i]; }
+  *yElems = (size_t)M * L;
+  if (N == 1) { *tmpElems = (size_t)M * std::max(K, L); return fastKronSuccess; }
+  uint64_t w[kMaxFactors];
+  stepWidths(N, Ps, Qs, w);
+  *tmpElems = (size_t)M * *std::max_element(w, w + N);
+  return fastKronSuccess;
+}
+
+// reference src/handle/handle.cpp:390-408
+fastKronError Handle::sizesForward(uint32_t M, uint32_t N, const uint32_t* Ps, const uint32_t* Qs,
+                                   size_t* yElems, size_t* interElems) {
+  if (!yElems || !interElems) return fastKronInvalidArgument;
+  if (N == 0 || N > kMaxFactors || !Ps || !Qs) return fastKronInvalidKMMProblem;
+  uint64_t w[kMaxFactors];
+  stepWidths(N, Ps, Qs, w);
+  for (uint32_t i = 1; i < N; i++) interElems[i - 1] = (size_t)M * w[i];
+  *yElems = (size_t)M * w[0];
+  return fastKronSuccess;
+}
+
+fastKronError Handle::xgemm(KronProblem p, fastKronBackend backend, void* temp1, void* temp2) {
+  // argument checks in the order of reference src/handle/handle.cpp:116-122
+  if (!p.forward) {
+    if (p.Z == nullptr || temp1 == nullptr || !hasBackend(backend)) return fastKronInvalidArgument;
+    if (p.Z == p.Y && temp2 == nullptr) return fastKronInvalidArgument;
+  } else {
+    if (p.Z == nullptr || !hasBackend(backend)) return fastKronInvalidArgument;
+  }
+  if (backend != fastKronBackend_HIP) return fastKronInvalidArgument;
+  if (p.N == 0 || p.N > kMaxFactors || p.M == 0 || p.batch == 0) return fastKronInvalidKMMProblem;
+  for (uint32_t i = 0; i < p.N; i++)
+    if (p.P[i] == 0 || p.Q[i] == 0 || p.F[i] == nullptr) return fastKronInvalidKMMProblem;
+  if (p.X == nullptr) return fastKronInvalidArgument;
+  if (p.forward && p.N > 1)
+    for (uint32_t i = 0; i + 1 < p.N; i++) if (!p.inter[i]) return fastKronInvalidArgument;
+
+  // A KMM with a single column is the MKM of the same vector with transposed factors
+  // (reference src/handle/handle.cpp:134-138).
+  if (p.mm == MMType::KMM && p.M == 1) {
+    p.mm = MMType::MKM;
+    p.opF = (p.opF == fastKronOp_N) ? fastKronOp_T : fastKronOp_N;
+    p.opX = fastKronOp_N;
+  }
+
+  fastKronError e = ensureDevice();
+  if (e != fastKronSuccess) return e;
+
+  Plan plan;
+  const std::string key = p.str();
+  bool have = false;
+  if (!p.forward) have = db_.lookupTuned(key, &plan);
+  if (!have && canTune() && !p.forward) {
+    e = tune(p, &plan);
+    if (e != fastKronSuccess) return e;
+    have = true;
+  }
+  if (!have) {
+    const std::string ck = key + (p.forward ? "_fwd" : "") + (useFusion() ? "" : "_nofuse");
+    auto it = planCache_.find(ck);
+    if (it != planCache_.end()) plan = it->second;
+    else {
+      plan = db_.selectOnline(p, dev_, useFusion());
+      planCache_[ck] = plan;
+      if (logLevel() >= 1) {
+        printf("[fastkron] %s ->", key.c_str());
+        for (auto& s : plan) printf(" [%u,%u] %s", s.lo, s.hi, db_.kernels()[s.kernel].name.c_str());
+        printf("\n");
+      }
+    }
+  }
+  lastPlan_ = key;
+  for (auto& s : plan)
+    lastPlan_ += ";" + std::to_string(s.lo) + "-" + std::to_string(s.hi) + ":" + db_.kernels()[s.kernel].name;
+  return execute(p, plan, temp1, temp2);
+}
+
+// Everything of a launch's arguments that follows from the problem and the factor range; the caller
+// fills in the input/output buffers.
+StepArgs makeStepArgs(const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool last) {
+  StepArgs a{};
+  a.nf = hi - lo + 1;
+  a.M = p.M; a.batch = p.batch;
+  a.Kin = p.colsBefore(hi);
+  a.Kout = p.colsAfter(lo);
+  for (uint32_t j = 0; j < a.nf && j < kMaxFused; j++) {
+    const uint32_t fi = hi - j;
+    a.f[j] = p.F[fi]; a.f_batch[j] = p.strideF[fi];
+    a.p[j] = p.P[fi]; a.q[j] = p.Q[fi];
+    // Storage of op(F): MKM factors are P x Q, KMM factors are Q x P; opF = T stores the transpose
+    // (reference tests/testBase.h:264-268,295-299).
+    const bool pMajor = (p.mm == MMType::MKM) == (p.opF == fastKronOp_N);
+    a.f_sp[j] = pMajor ? (int64_t)p.Q[fi] : 1;
+    a.f_sq[j] = pMajor ? 1 : (int64_t)p.P[fi];
+  }
+  const bool rowMajor = (p.mm == MMType::MKM);      // rows contiguous along the columns
+  auto setLd = [&](int64_t& ldm, int64_t& ldc, uint64_t cols, bool transposed) {
+    const bool rm = transposed ? !rowMajor : rowMajor;
+    if (rm) { ldm = (int64_t)cols; ldc = 1; } else { ldm = 1; ldc = (int64_t)p.M; }
+  };
+  setLd(a.in_ldm, a.in_ldc, a.Kin, first && p.opX == fastKronOp_T);
+  setLd(a.out_ldm, a.out_ldc, a.Kout, false);
+  if (last) {
+    a.epilogue = 1; a.alpha = p.alpha; a.beta = p.beta;
+    a.y = (p.beta != 0.0) ? p.Y : nullptr;          // beta is skipped when Y is null, reference kernel.h:158-159
+    a.y_batch = p.strideY;
+    setLd(a.y_ldm, a.y_ldc, p.L(), false);
+  }
+  return a;
+}
+
+fastKronError Handle::execute(const KronProblem& p, const Plan& plan, void* temp1, void* temp2) {
+  const size_t n = plan.size();
+  if (n == 0) return fastKronKernelNotFound;
+  const uint64_t L = p.L();
+
+  // Ping-pong plan of reference src/kmm/kmmalgo.cpp:82-110: launch l < n-1 writes tmps[l % 2]; when
+  // only one temporary is given, Z is the other one, placed so that the last intermediate is not Z.
+  void* tmps[2] = {temp1, temp2};
+  bool zIsTmp[2] = {false, false};
+  if (!p.forward && n > 1 && temp2 == nullptr) {
+    if (n % 2 == 1) { tmps[1] = temp1; tmps[0] = p.Z; zIsTmp[0] = true; }
+    else            { tmps[1] = p.Z; zIsTmp[1] = true; }
+    if (n == 2) { tmps[1] = nullptr; zIsTmp[1] = false; }     // a 2-launch plan never touches the second one
+  }
+
+  const void* in = p.X;
+  uint64_t inBatch = p.strideX;
+  for (size_t l = 0; l < n; l++) {
+    const PlanStep& s = plan[l];
+    const KernelInfo& k = db_.kernels()[s.kernel];
+    const bool first = (l == 0), last = (l + 1 == n);
+    if (s.hi - s.lo + 1 > kMaxFused) return fastKronKernelNotFound;
+    StepArgs a = makeStepArgs(p, s.lo, s.hi, first, last);
+    a.in = in; a.in_batch = inBatch;
+    if (last) {
+      a.out = p.Z; a.out_batch = p.strideZ;
+    } else if (p.forward) {
+      a.out = p.inter[s.lo - 1];
+      a.out_batch = p.haveStrideInter ? p.strideInter[s.lo - 1] : (uint64_t)p.M * a.Kout;
+    } else {
+      const int t = (int)(l % 2);
+      a.out = tmps[t];
+      a.out_batch = (uint64_t)p.M * a.Kout;
+      if (zIsTmp[t]) {
+        // Z doubles as scratch: the intermediate has to fit the per-batch Z region.
+        if (a.Kout > L || (p.batch > 1 && p.strideZ < (uint64_t)p.M * L)) return fastKronInvalidArgument;
+        if (p.batch > 1) a.out_batch = p.strideZ;
+      }
+      if (a.out == nullptr) return fastKronInvalidArgument;
+    }
+    if (logLevel() >= 2)
+      printf("[fastkron]   launch %zu: factors [%u,%u] Kin=%llu Kout=%llu kernel %s\n", l, s.lo, s.hi,
+             (unsigned long long)a.Kin, (unsigned long long)a.Kout, k.name.c_str());
+    hipError_t he = k.launch(k, a, stream_);
+    if (he != hipSuccess) {
+      fprintf(stderr, "[fastkron] launch of %s failed: %s\n", k.name.c_str(), hipGetErrorString(he));
+      return fastKronInvalidArgument;                 // reference cuda_kernel_db.cu:296-301
+    }
+    in = a.out; inBatch = a.out_batch;
+  }
+  return fastKronSuccess;
+}
+
+}  // namespace fk

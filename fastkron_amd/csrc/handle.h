@@ -1,0 +1,66 @@
+// The object behind fastKronHandle: backends, options, the HIP stream, the gfx950 kernel database and
+// the tuner.  Role of reference src/handle/handle.{h,cpp} (FastKronHandle, xgemm, gekmmSizes).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <string>
+#include <unordered_map>
+#include "../../include/fastkron.h"
+#include "kernel_db.h"
+#include "problem.h"
+
+namespace fk {
+
+struct BufferPlan {          // where each launch reads and writes
+  const void* in;  void* out;
+  uint64_t in_batch, out_batch;
+};
+
+StepArgs makeStepArgs(const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool last);
+
+class Handle {
+ public:
+  explicit Handle(uint32_t backends);
+  ~Handle();
+
+  bool hasBackend(uint32_t b) const { return (backends_ & b) == b; }
+  void setOptions(uint32_t o) { options_ = o; }
+  bool canTune() const { return (options_ & fastKronOptionsTune) != 0; }
+  bool useFusion() const { return (options_ & fastKronOptionsUseFusion) != 0; }
+
+  fastKronError initHIP(void* ptrToStream);
+  fastKronError setStream(fastKronBackend backend, void* ptrToStream);
+
+  static fastKronError sizes(uint32_t M, uint32_t N, const uint32_t* Ps, const uint32_t* Qs,
+                             size_t* yElems, size_t* tmpElems);
+  static fastKronError sizesForward(uint32_t M, uint32_t N, const uint32_t* Ps, const uint32_t* Qs,
+                                    size_t* yElems, size_t* interElems);
+
+  // Entry point of every gemkm/gekmm/forward call (reference src/handle/handle.cpp:114-286).
+  fastKronError xgemm(KronProblem p, fastKronBackend backend, void* temp1, void* temp2);
+
+  // Runs `plan` on the stream; temps may be null when the plan has a single launch.
+  fastKronError execute(const KronProblem& p, const Plan& plan, void* temp1, void* temp2);
+  fastKronError tune(const KronProblem& p, Plan* best);
+
+  const std::string& lastPlan() const { return lastPlan_; }
+  void setTunedDB(const char* path);
+
+  KernelDB& db() { return db_; }
+  const DeviceInfo& device() const { return dev_; }
+  hipStream_t stream() const { return stream_; }
+
+ private:
+  fastKronError ensureDevice();
+
+  uint32_t backends_;
+  uint32_t options_ = fastKronOptionsNone;
+  hipStream_t stream_ = nullptr;
+  bool hipInit_ = false;
+  DeviceInfo dev_;
+  KernelDB db_;
+  std::unordered_map<std::string, Plan> planCache_;   // online selections, per problem string
+  std::string dbPath_;
+  std::string lastPlan_;
+};
+
+}  // namespace fk

@@ -1,0 +1,146 @@
+#include "kernel_db.h"
+
+#include <cstdio>
+#include <cstdlib>
+#include <fstream>
+#include <sstream>
+
+#include "kernels/launch.h"
+
+namespace fk {
+
+std::string KronProblem::str() const {
+  std::ostringstream o;
+  auto facs = [&]() {
+    if (sameShapes(0, N - 1)) o << P[0] << "x" << Q[0] << "^" << N;
+    else for (uint32_t i = 0; i < N; i++) { o << P[i] << "x" << Q[i]; if (i + 1 < N) o << "(x)"; }
+  };
+  if (mm == MMType::MKM) { o << M << "x" << K() << "*("; facs(); o << ")"; }
+  else                   { o << "("; facs(); o << ")*" << K() << "x" << M; }
+  o << "_" << (opX == 2 ? "T" : "N") << (opF == 2 ? "T" : "N") << "_" << (dt == DType::F32 ? "f" : "d");
+  if (strided) o << "_stridedBatched_" << batch;
+  return o.str();
+}
+
+static bool genericCanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, uint32_t hi, bool, bool,
+                          const DeviceInfo&) {
+  return lo == hi && k.dt == p.dt;
+}
+static hipError_t genericLaunch(const KernelInfo& k, const StepArgs& a, hipStream_t s) {
+  return launchGenericStep(a, k.dt, s);
+}
+
+void registerGenericKernels(std::vector<KernelInfo>& out) {
+  for (DType dt : {DType::F32, DType::F64}) {
+    KernelInfo k{};
+    k.name = std::string("gekmm_hip_gfx950_256_") + (dt == DType::F32 ? "f" : "d") + "_generic_1";
+    k.dt = dt; k.P = 0; k.Q = 0; k.fused = 1; k.tileM = 0; k.tileK = 0; k.threads = 256; k.variant = 0;
+    k.canRun = genericCanRun; k.launch = genericLaunch;
+    out.push_back(k);
+  }
+}
+
+KernelDB::KernelDB() {
+  registerGenericKernels(kernels_);
+}
+
+int KernelDB::findByName(const std::string& name) const {
+  for (size_t i = 0; i < kernels_.size(); i++) if (kernels_[i].name == name) return (int)i;
+  return -1;
+}
+
+int KernelDB::genericKernel(DType dt) const {
+  for (size_t i = 0; i < kernels_.size(); i++)
+    if (kernels_[i].P == 0 && kernels_[i].dt == dt) return (int)i;
+  return -1;
+}
+
+std::vector<int> KernelDB::candidates(const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool last,
+                                      const DeviceInfo& dev) const {
+  std::vector<int> r;
+  for (size_t i = 0; i < kernels_.size(); i++)
+    if (kernels_[i].canRun(kernels_[i], p, lo, hi, first, last, dev)) r.push_back((int)i);
+  return r;
+}
+
+Plan KernelDB::selectOnline(const KronProblem& p, const DeviceInfo& dev, bool allowFusion) const {
+  Plan plan;
+  int hi = (int)p.N - 1;
+  while (hi >= 0) {
+    int bestLo = hi, bestK = genericKernel(p.dt);
+    if (!p.forward) {
+      const uint32_t maxDepth = allowFusion ? kMaxFused : 1;
+      for (int lo = (hi + 1 >= (int)maxDepth) ? hi + 1 - (int)maxDepth : 0; lo <= hi; lo++) {
+        auto c = candidates(p, (uint32_t)lo, (uint32_t)hi, hi == (int)p.N - 1, lo == 0, dev);
+        int pick = -1;
+        for (int k : c) if (kernels_[k].P != 0) { pick = k; break; }   // first registered = preferred
+        if (pick >= 0) { bestLo = lo; bestK = pick; break; }           // deepest fusion wins
+      }
+    }
+    plan.push_back(PlanStep{(uint32_t)bestLo, (uint32_t)hi, bestK});
+    hi = bestLo - 1;
+  }
+  return plan;
+}
+
+bool KernelDB::lookupTuned(const std::string& key, Plan* plan) const {
+  auto it = tuned_.find(key);
+  if (it == tuned_.end()) return false;
+  Plan pl;
+  for (auto& s : it->second.steps) {
+    int k = findByName(s.second);
+    if (k < 0) return false;
+    pl.push_back(PlanStep{s.first.first, s.first.second, k});
+  }
+  *plan = pl;
+  return true;
+}
+
+void KernelDB::storeTuned(const std::string& key, const Plan& plan, float ms) {
+  Tuned t;
+  t.ms = ms;
+  for (auto& s : plan) t.steps.push_back({{s.lo, s.hi}, kernels_[s.kernel].name});
+  tuned_[key] = t;
+}
+
+// File format, one problem per line:
+//   <problem string> <ms> <nsteps> {<lo> <hi> <kernel name>}...
+bool KernelDB::loadFile(const std::string& path) {
+  std::ifstream f(path);
+  if (!f) return false;
+  std::string line;
+  while (std::getline(f, line)) {
+    if (line.empty() || line[0] == '#') continue;
+    std::istringstream is(line);
+    std::string key; float ms; size_t n;
+    if (!(is >> key >> ms >> n)) continue;
+    Tuned t; t.ms = ms;
+    bool ok = true;
+    for (size_t i = 0; i < n; i++) {
+      uint32_t lo, hi; std::string name;
+      if (!(is >> lo >> hi >> name)) { ok = false; break; }
+      t.steps.push_back({{lo, hi}, name});
+    }
+    if (ok) tuned_[key] = t;
+  }
+  return true;
+}
+
+bool KernelDB::saveFile(const std::string& path) const {
+  std::ofstream f(path);
+  if (!f) return false;
+  f << "# fastkron gfx950 tuned launch plans: problem ms nsteps {lo hi kernel}\n";
+  for (auto& kv : tuned_) {
+    f << kv.first << " " << kv.second.ms << " " << kv.second.steps.size();
+    for (auto& s : kv.second.steps) f << " " << s.first.first << " " << s.first.second << " " << s.second;
+    f << "\n";
+  }
+  return (bool)f;
+}
+
+std::string KernelDB::defaultPath() {
+  if (const char* e = getenv("FASTKRON_TUNED_DB")) return e;
+  return "";
+}
+
+}  // namespace fk

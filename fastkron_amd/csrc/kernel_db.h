@@ -1,0 +1,77 @@
+// Registry of compiled gfx950 kernels, launch-plan selection and the persisted tuning database.
+//
+// Role of reference src/kernel_db/kernel_db.{h,cpp} (abstract database + online selection,
+// :152-290) with a gfx950 subclass in place of the reference's CUDA one (cuda_kernel_db.cu); unlike
+// the reference, whose tuner keeps results only in memory (src/autotuner/autotuner.h:101-116), tuned
+// plans are written to a text file and reloaded by later processes.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <map>
+#include <string>
+#include <vector>
+#include "problem.h"
+
+namespace fk {
+
+struct DeviceInfo {
+  int  device = -1;
+  int  cus = 256;
+  int  ldsPerBlock = 65536;      // bytes a workgroup may allocate
+  int  waveSize = 64;
+  int  clockKHz = 2400000;
+  char arch[64] = "gfx950";
+  bool valid = false;
+};
+
+struct KernelInfo;
+using CanRunFn = bool (*)(const KernelInfo&, const KronProblem&, uint32_t lo, uint32_t hi,
+                          bool firstLaunch, bool lastLaunch, const DeviceInfo&);
+using LaunchFn = hipError_t (*)(const KernelInfo&, const StepArgs&, hipStream_t);
+
+// One compiled kernel variant.  `name` follows the reference kernel-string grammar
+// (src/kernels/kmmkernel.cpp:128-136 with the backend/arch prefix of src/kernels/gpu_kmmkernel.cu:3-8).
+struct KernelInfo {
+  std::string name;
+  DType    dt;
+  uint32_t P, Q;          // 0: any factor shape
+  uint32_t fused;         // factors applied per launch
+  uint32_t tileM, tileK;  // rows and input columns per workgroup (0: not tiled that way)
+  uint32_t threads;
+  uint32_t variant;       // kernel-family specific
+  CanRunFn canRun;
+  LaunchFn launch;
+};
+
+struct PlanStep { uint32_t lo, hi; int kernel; };   // factors [lo, hi], hi applied first
+using Plan = std::vector<PlanStep>;
+
+class KernelDB {
+ public:
+  KernelDB();
+  const std::vector<KernelInfo>& kernels() const { return kernels_; }
+  int findByName(const std::string& name) const;
+  int genericKernel(DType dt) const;
+
+  // Online selection (no timing): greedy over the chain, deepest fusion first.
+  Plan selectOnline(const KronProblem& p, const DeviceInfo& dev, bool allowFusion) const;
+  // All kernels able to run factors [lo, hi] as one launch.
+  std::vector<int> candidates(const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool last,
+                              const DeviceInfo& dev) const;
+
+  // Tuned plans, keyed by the problem string.
+  bool lookupTuned(const std::string& key, Plan* plan) const;
+  void storeTuned(const std::string& key, const Plan& plan, float ms);
+  bool loadFile(const std::string& path);
+  bool saveFile(const std::string& path) const;
+  static std::string defaultPath();
+
+ private:
+  std::vector<KernelInfo> kernels_;
+  struct Tuned { std::vector<std::pair<std::pair<uint32_t, uint32_t>, std::string>> steps; float ms; };
+  std::map<std::string, Tuned> tuned_;
+};
+
+// Filled in by each kernel family's translation unit.
+void registerGenericKernels(std::vector<KernelInfo>& out);
+
+}  // namespace fk

@@ -1,0 +1,69 @@
+"""Helpers for the GPU parity tests: seeded inputs, a call through the C-ABI library, the oracle's
+answer for the same buffers."""
+import numpy as np
+
+from oracle import kron_oracle as ko
+
+TOL = {np.float32: 1e-5, np.float64: 1e-12}        # normwise bounds stated for fp32 / fp64 results
+
+
+def seeded(seed, shape, dt, integer=False):
+    rng = np.random.default_rng(seed)
+    if integer:                                      # the reference's own tests fill with rand() % 3 + 1
+        return rng.integers(1, 4, size=shape).astype(dt)
+    return rng.uniform(-1.0, 1.0, size=shape).astype(dt)
+
+
+def normwise(a, b):
+    a = np.asarray(a, np.float64).reshape(-1)
+    b = np.asarray(b, np.float64).reshape(-1)
+    s = np.max(np.abs(b))
+    return float(np.max(np.abs(a - b)) / (s if s > 0 else 1.0))
+
+
+def make_case(mm, M, Ps, Qs, dt, seed=0, opX=ko.OP_N, opFs=ko.OP_N, batch=1, with_y=True, integer=False,
+              share_f=False, share_y=False):
+    """Flat host buffers laid out as the C API expects, batches included."""
+    K, L = int(np.prod(Ps)), int(np.prod(Qs))
+    X = seeded(seed, (batch, M * K), dt, integer)
+    Fs = [seeded(seed + 1 + i, (1 if share_f else batch, p * q), dt, integer) for i, (p, q) in enumerate(zip(Ps, Qs))]
+    Y = seeded(seed + 100, (1 if share_y else batch, M * L), dt, integer) if with_y else None
+    return X, Fs, Y
+
+
+def oracle_answer(mm, M, Ps, Qs, X, Fs, Y, alpha, beta, opX=ko.OP_N, opFs=ko.OP_N, batch=1,
+                  share_f=False, share_y=False, keep_intermediates=False):
+    K, L = int(np.prod(Ps)), int(np.prod(Qs))
+    return ko.sliced_multiply(mm, M, Ps, Qs, X, Fs, alpha=alpha, beta=beta, Y=Y, opX=opX, opFs=opFs, batch=batch,
+                              strideX=M * K, strideF=[0 if share_f else p * q for p, q in zip(Ps, Qs)],
+                              strideZ=M * L, strideY=0 if share_y else M * L,
+                              keep_intermediates=keep_intermediates)
+
+
+def run_gpu(fk, mm, M, Ps, Qs, X, Fs, Y, alpha, beta, opX=ko.OP_N, opFs=ko.OP_N, batch=1,
+            share_f=False, share_y=False, use_temp2=True, strided=None, poison=True):
+    """Calls the library on device copies of the host buffers; returns Z as numpy and the error code."""
+    import torch
+    from fastkron_amd import capi
+    dev = "cuda:0"
+    K, L = int(np.prod(Ps)), int(np.prod(Qs))
+    tX = torch.from_numpy(X).to(dev)
+    tFs = [torch.from_numpy(f).to(dev) for f in Fs]
+    tY = torch.from_numpy(Y).to(dev) if Y is not None else None
+    ye, te = fk.sizes(M, Ps, Qs)
+    assert ye == M * L
+    tdt = tX.dtype
+    fill = float("nan") if poison else 0.0
+    Z = torch.full((batch * max(ye, te if not use_temp2 else ye),), fill, dtype=tdt, device=dev)
+    t1 = torch.full((batch * te,), fill, dtype=tdt, device=dev)
+    t2 = torch.full((batch * te,), fill, dtype=tdt, device=dev) if use_temp2 else None
+    strided = (batch > 1) if strided is None else strided
+    if strided:
+        fn = fk.xgemkm_strided_batched if mm == ko.MKM else fk.xgekmm_strided_batched
+        e = fn(M, Ps, Qs, tX, M * K, tFs, [0 if share_f else p * q for p, q in zip(Ps, Qs)], Z, M * L, batch,
+               alpha, beta, tY, 0 if share_y else M * L, t1, t2, opX, opFs)
+    else:
+        fn = fk.xgemkm if mm == ko.MKM else fk.xgekmm
+        e = fn(M, Ps, Qs, tX, tFs, Z, alpha, beta, tY, t1, t2, opX, opFs)
+    torch.cuda.synchronize()
+    return Z[: batch * M * L].cpu().numpy(), e

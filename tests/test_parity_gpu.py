@@ -1,0 +1,159 @@
+"""GPU parity: every call goes through the C-ABI library and is compared with the CPU oracle on the
+same seeded buffers.  Bounds: normwise max|Z - Zref| / max|Zref| <= 1e-5 (fp32), 1e-12 (fp64); integer-valued
+inputs additionally use the reference harness's element-wise rule (reference tests/testBase.h:136-146)."""
+import numpy as np
+import pytest
+
+from oracle import kron_oracle as ko
+from tests.gpu_util import TOL, make_case, normwise, oracle_answer, run_gpu
+from tests.kron_ref import eq_val
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def fk():
+    import fastkron_amd
+    h = fastkron_amd.FastKron()
+    yield h
+    h.close()
+
+
+def check(fk, mm, M, Ps, Qs, dt, alpha=1.0, beta=0.0, seed=0, **kw):
+    run_kw = {k: kw.pop(k) for k in ("use_temp2", "strided") if k in kw}
+    integer = kw.get("integer", False)
+    X, Fs, Y = make_case(mm, M, Ps, Qs, dt, seed=seed, with_y=(beta != 0), **kw)
+    kw.pop("integer", None)
+    want = oracle_answer(mm, M, Ps, Qs, X, Fs, Y, alpha, beta, **kw)
+    got, e = run_gpu(fk, mm, M, Ps, Qs, X, Fs, Y, alpha, beta, **kw, **run_kw)
+    assert e == 0, f"fastKronError {e}"
+    assert not np.isnan(got).any()
+    err = normwise(got, want)
+    assert err <= TOL[dt], f"normwise error {err:.3e}"
+    if integer:
+        assert eq_val(got, want)
+
+
+# shape matrix of reference tests/src/general-tests-NN.cpp:52-100 (square, non-square, distinct), sized so
+# that the oracle answers in seconds
+SQUARE = [(16, [p] * n) for p, n in [(1, 4), (2, 8), (3, 5), (4, 6), (5, 4), (6, 3), (8, 4), (12, 3), (16, 3),
+                                     (24, 2), (31, 2), (32, 3), (50, 2), (55, 2), (62, 2), (64, 2), (127, 2),
+                                     (128, 2), (129, 1), (255, 1), (297, 1), (512, 1)]]
+NONSQUARE = [(16, [1, 1, 1], [4, 4, 4]), (16, [5, 5, 5], [1, 1, 1]), (16, [2] * 5, [4] * 5),
+             (16, [31, 31], [63, 63]), (16, [63, 63], [31, 31]), (8, [297], [127]), (8, [127], [297]),
+             (16, [2, 5, 6], [3, 2, 4]), (16, [14, 19], [15, 13]), (4, [8, 8], [32, 32]), (4, [32, 32], [8, 8])]
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+@pytest.mark.parametrize("M,Ps", SQUARE)
+def test_mkm_square(fk, M, Ps, dt):
+    check(fk, ko.MKM, M, Ps, Ps, dt, alpha=2.0, beta=1.0, integer=(max(Ps) ** len(Ps) < 4096))
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+@pytest.mark.parametrize("M,Ps,Qs", NONSQUARE)
+def test_mkm_nonsquare(fk, M, Ps, Qs, dt):
+    check(fk, ko.MKM, M, Ps, Qs, dt, alpha=2.0, beta=1.0)
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+@pytest.mark.parametrize("M", [1, 3, 16, 20])
+@pytest.mark.parametrize("Ps,Qs", [([4] * 4, [4] * 4), ([8, 8, 8], [8, 8, 8]), ([2, 5, 6], [3, 2, 4]),
+                                   ([32, 32], [16, 16]), ([31], [63])])
+def test_kmm(fk, M, Ps, Qs, dt):
+    check(fk, ko.KMM, M, Ps, Qs, dt, alpha=2.0, beta=1.0)
+
+
+@pytest.mark.parametrize("mm", [ko.MKM, ko.KMM])
+@pytest.mark.parametrize("opX,opFs", [(ko.OP_T, ko.OP_T), (ko.OP_T, ko.OP_N), (ko.OP_N, ko.OP_T)])
+@pytest.mark.parametrize("M,Ps,Qs", [(16, [8, 8, 8], [8, 8, 8]), (13, [2, 5, 6], [3, 2, 4]), (17, [31], [63]),
+                                     (1, [4, 4, 4], [4, 4, 4])])
+def test_transposed_operands(fk, mm, opX, opFs, M, Ps, Qs):
+    """reference tests/src/general-tests-TT.cpp:36-83"""
+    check(fk, mm, M, Ps, Qs, np.float32, alpha=2.0, beta=1.0, opX=opX, opFs=opFs)
+    check(fk, mm, M, Ps, Qs, np.float64, alpha=2.0, beta=1.0, opX=opX, opFs=opFs)
+
+
+@pytest.mark.parametrize("mm", [ko.MKM, ko.KMM])
+@pytest.mark.parametrize("share_f,share_y", [(False, False), (True, False), (True, True)])
+@pytest.mark.parametrize("M,Ps,Qs", [(16, [32] * 3, [16] * 3), (8, [32, 32], [64, 64]), (5, [3, 4], [2, 5])])
+def test_strided_batched(fk, mm, share_f, share_y, M, Ps, Qs):
+    """batch combinations of reference tests/src/general-tests-NN.cpp:94-100"""
+    check(fk, mm, M, Ps, Qs, np.float32, alpha=1.0, beta=1.0, batch=3, share_f=share_f, share_y=share_y)
+    check(fk, mm, M, Ps, Qs, np.float64, alpha=1.0, beta=1.0, batch=2, share_f=share_f, share_y=share_y)
+
+
+@pytest.mark.parametrize("mm", [ko.MKM, ko.KMM])
+@pytest.mark.parametrize("Ps,Qs", [([4, 4, 4], [4, 4, 4]), ([4] * 4, [4] * 4), ([8, 8], [8, 8]), ([2] * 5, [3] * 5)])
+def test_single_temporary_uses_z_as_scratch(fk, mm, Ps, Qs):
+    check(fk, mm, 8, Ps, Qs, np.float32, alpha=1.5, beta=0.5, use_temp2=False)
+
+
+def test_single_temporary_with_z_smaller_than_an_intermediate_is_rejected(fk):
+    """A shrinking chain needs both temporaries (include/fastkron.h: temp2 is required when Z is smaller
+    than the temporary); with one, the call must fail instead of writing past Z."""
+    fk.set_options(fusion=False)
+    try:
+        X, Fs, _ = make_case(ko.MKM, 4, [16] * 3, [2] * 3, np.float32, with_y=False)
+        _, e = run_gpu(fk, ko.MKM, 4, [16] * 3, [2] * 3, X, Fs, None, 1.0, 0.0, use_temp2=False)
+        assert e == 4
+    finally:
+        fk.set_options(fusion=True)
+
+
+def test_alpha_beta_and_null_y(fk):
+    check(fk, ko.MKM, 8, [8, 8], [8, 8], np.float32, alpha=-0.75, beta=0.0)
+    check(fk, ko.MKM, 8, [8, 8], [8, 8], np.float64, alpha=0.0, beta=3.0)
+    # beta != 0 with Y == NULL: the beta term is skipped, as in the reference kernels
+    X, Fs, _ = make_case(ko.MKM, 4, [4, 4], [4, 4], np.float32, with_y=False)
+    want = oracle_answer(ko.MKM, 4, [4, 4], [4, 4], X, Fs, None, 2.0, 0.0)
+    got, e = run_gpu(fk, ko.MKM, 4, [4, 4], [4, 4], X, Fs, None, 2.0, 5.0)
+    assert e == 0 and normwise(got, want) <= 1e-5
+
+
+@pytest.mark.parametrize("mm,name", [(ko.MKM, "mkm"), (ko.KMM, "kmm")])
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_forward_keeps_every_intermediate(fk, mm, name, dt):
+    import torch
+    M, Ps, Qs = 6, [4, 3, 5], [2, 4, 3]
+    X, Fs, _ = make_case(mm, M, Ps, Qs, dt, with_y=False)
+    Zw, Iw = oracle_answer(mm, M, Ps, Qs, X, Fs, None, 1.0, 0.0, keep_intermediates=True)
+    ye, sizes = fk.sizes_forward(M, Ps, Qs)
+    dev = "cuda:0"
+    tX = torch.from_numpy(X).to(dev)
+    tFs = [torch.from_numpy(f).to(dev) for f in Fs]
+    Z = torch.full((ye,), float("nan"), dtype=tX.dtype, device=dev)
+    inters = [torch.full((s,), float("nan"), dtype=tX.dtype, device=dev) for s in sizes]
+    e = fk.xforward(name, M, Ps, Qs, tX, tFs, Z, inters)
+    torch.cuda.synchronize()
+    assert e == 0
+    assert normwise(Z.cpu().numpy(), Zw) <= TOL[dt]
+    for got, want in zip(inters, Iw):
+        assert normwise(got.cpu().numpy(), want) <= TOL[dt]
+
+
+# ---- the five benchmark configurations at a row count the oracle finishes quickly ----
+BENCH = [
+    ("c1", ko.MKM, 16, [8] * 5, [8] * 5, np.float32, 1.0, 0.0, 1),
+    ("c2", ko.MKM, 8, [16] * 4, [16] * 4, np.float32, 1.0, 0.0, 1),
+    ("c3", ko.MKM, 2, [64] * 3, [64] * 3, np.float64, 1.0, 0.0, 1),
+    ("c4", ko.KMM, 64, [4] * 6, [4] * 6, np.float32, 1.5, 0.5, 1),
+    ("c5", ko.MKM, 8, [32] * 3, [16] * 3, np.float32, 1.0, 1.0, 8),
+]
+
+
+@pytest.mark.parametrize("name,mm,M,Ps,Qs,dt,alpha,beta,batch", BENCH, ids=[b[0] for b in BENCH])
+def test_benchmark_configurations_reduced_rows(fk, name, mm, M, Ps, Qs, dt, alpha, beta, batch):
+    check(fk, mm, M, Ps, Qs, dt, alpha=alpha, beta=beta, batch=batch, seed=7)
+
+
+@pytest.mark.parametrize("tune", [False, True])
+def test_tuned_and_online_plans_agree(tune):
+    import fastkron_amd
+    h = fastkron_amd.FastKron(tune=tune)
+    try:
+        check(h, ko.MKM, 32, [8] * 4, [8] * 4, np.float32, alpha=1.0, beta=0.0, seed=3)
+        check(h, ko.MKM, 16, [16] * 3, [16] * 3, np.float32, alpha=2.0, beta=1.0, seed=4)
+        check(h, ko.KMM, 32, [4] * 5, [4] * 5, np.float64, alpha=2.0, beta=1.0, seed=5)
+    finally:
+        h.close()
