@@ -87,7 +87,7 @@ def cpu_baseline(M, Ps, Qs, dt, alpha, beta, batch, budget_s):
     out = np.empty(rows * L, dtype=dt)
     ko.sliced_multiply_fast(rows, Ps, Qs, X, Fs, alpha, beta, Y, out=out)       # warm-up, page in
     best, spent, reps = float("inf"), 0.0, 0
-    while spent < budget_s and reps < 200:
+    while spent < budget_s and reps < 100000:
         t0 = time.perf_counter()
         ko.sliced_multiply_fast(rows, Ps, Qs, X, Fs, alpha, beta, Y, out=out)
         dtm = time.perf_counter() - t0

@@ -40,6 +40,13 @@ def load():
     global _lib
     if _lib is not None:
         return _lib
+    try:
+        # PyTorch bundles its own libamdhip64.so.7; importing it first makes the dynamic loader bind
+        # libFastKron.so to that same runtime, so the process holds exactly one HIP runtime and
+        # torch's allocations and streams are valid inside the library.
+        import torch  # noqa: F401
+    except ImportError:
+        pass
     if not os.path.exists(LIB_PATH):
         raise RuntimeError(
             f"{LIB_PATH} is missing: build it with fastkron_amd/csrc/build.sh (or __graft_entry__.build())")
