@@ -149,6 +149,15 @@ fastKronError Handle::xgemm(KronProblem p, fastKronBackend backend, void* temp1,
       }
     }
   }
+  // Kernel-specific requirements on the actual buffers (alignment, strides): when the chosen plan
+  // cannot run on them, fall back to one generic launch per factor.
+  e = execute(p, plan, temp1, temp2, true);
+  if (e == fastKronKernelNotFound) {
+    plan.clear();
+    for (int i = (int)p.N - 1; i >= 0; i--) plan.push_back(PlanStep{(uint32_t)i, (uint32_t)i, db_.genericKernel(p.dt)});
+  } else if (e != fastKronSuccess) {
+    return e;
+  }
   lastPlan_ = key;
   for (auto& s : plan)
     lastPlan_ += ";" + std::to_string(s.lo) + "-" + std::to_string(s.hi) + ":" + db_.kernels()[s.kernel].name;
@@ -189,7 +198,9 @@ StepArgs makeStepArgs(const KronProblem& p, uint32_t lo, uint32_t hi, bool first
   return a;
 }
 
-fastKronError Handle::execute(const KronProblem& p, const Plan& plan, void* temp1, void* temp2) {
+// With dryRun the launches are only validated (kernel-specific checks on the concrete buffers);
+// fastKronKernelNotFound then means "this plan cannot run on these buffers".
+fastKronError Handle::execute(const KronProblem& p, const Plan& plan, void* temp1, void* temp2, bool dryRun) {
   const size_t n = plan.size();
   if (n == 0) return fastKronKernelNotFound;
   const uint64_t L = p.L();
@@ -232,6 +243,11 @@ fastKronError Handle::execute(const KronProblem& p, const Plan& plan, void* temp
     if (logLevel() >= 2)
       printf("[fastkron]   launch %zu: factors [%u,%u] Kin=%llu Kout=%llu kernel %s\n", l, s.lo, s.hi,
              (unsigned long long)a.Kin, (unsigned long long)a.Kout, k.name.c_str());
+    if (dryRun) {
+      if (k.check && !k.check(k, a)) return fastKronKernelNotFound;
+      in = a.out; inBatch = a.out_batch;
+      continue;
+    }
     hipError_t he = k.launch(k, a, stream_);
     if (he != hipSuccess) {
       fprintf(stderr, "[fastkron] launch of %s failed: %s\n", k.name.c_str(), hipGetErrorString(he));

@@ -39,7 +39,7 @@ class Handle {
   fastKronError xgemm(KronProblem p, fastKronBackend backend, void* temp1, void* temp2);
 
   // Runs `plan` on the stream; temps may be null when the plan has a single launch.
-  fastKronError execute(const KronProblem& p, const Plan& plan, void* temp1, void* temp2);
+  fastKronError execute(const KronProblem& p, const Plan& plan, void* temp1, void* temp2, bool dryRun = false);
   fastKronError tune(const KronProblem& p, Plan* best);
 
   const std::string& lastPlan() const { return lastPlan_; }

@@ -35,12 +35,34 @@ void registerGenericKernels(std::vector<KernelInfo>& out) {
     KernelInfo k{};
     k.name = std::string("gekmm_hip_gfx950_256_") + (dt == DType::F32 ? "f" : "d") + "_generic_1";
     k.dt = dt; k.P = 0; k.Q = 0; k.fused = 1; k.tileM = 0; k.tileK = 0; k.threads = 256; k.variant = 0;
-    k.canRun = genericCanRun; k.launch = genericLaunch;
+    k.canRun = genericCanRun; k.launch = genericLaunch; k.check = nullptr;
     out.push_back(k);
   }
 }
 
+// ---- whole-row kernel for four fused 16x16 fp32 factors ----
+static bool row16CanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
+                        const DeviceInfo& dev) {
+  if (p.dt != DType::F32 || p.mm != MMType::MKM || hi - lo + 1 != 4 || p.forward) return false;
+  for (uint32_t i = lo; i <= hi; i++) if (p.P[i] != 16 || p.Q[i] != 16) return false;
+  if (p.colsBefore(hi) != 65536) return false;
+  if (first && p.opX == 2) return false;
+  return dev.ldsPerBlock >= 131072 && k.dt == p.dt;
+}
+static hipError_t row16Launch(const KernelInfo&, const StepArgs& a, hipStream_t s) { return launchRow16x4(a, s); }
+static bool row16Check(const KernelInfo&, const StepArgs& a) { return row16x4Supported(a); }
+
+void registerRowKernels(std::vector<KernelInfo>& out) {
+  KernelInfo k{};
+  // grammar: <mm>_<backend>_<arch>_<threads>_<type>_<PxQ>_<TilePxTileQ>_<fused>_<TileMxTileK>_<regs>_<ops>_<batch>_<p2p>_<opt>
+  k.name = "mkm_hip_gfx950_1024_f_16x16_16x16_4_1x65536_mfma16x16x4_NN_strided_0_3";
+  k.dt = DType::F32; k.P = 16; k.Q = 16; k.fused = 4; k.tileM = 1; k.tileK = 65536; k.threads = 1024; k.variant = 0;
+  k.canRun = row16CanRun; k.launch = row16Launch; k.check = row16Check;
+  out.push_back(k);
+}
+
 KernelDB::KernelDB() {
+  registerRowKernels(kernels_);
   registerGenericKernels(kernels_);
 }
 

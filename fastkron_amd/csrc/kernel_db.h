@@ -27,6 +27,8 @@ struct KernelInfo;
 using CanRunFn = bool (*)(const KernelInfo&, const KronProblem&, uint32_t lo, uint32_t hi,
                           bool firstLaunch, bool lastLaunch, const DeviceInfo&);
 using LaunchFn = hipError_t (*)(const KernelInfo&, const StepArgs&, hipStream_t);
+// Final check on the concrete launch arguments (pointer alignment, strides); null = always fine.
+using CheckFn  = bool (*)(const KernelInfo&, const StepArgs&);
 
 // One compiled kernel variant.  `name` follows the reference kernel-string grammar
 // (src/kernels/kmmkernel.cpp:128-136 with the backend/arch prefix of src/kernels/gpu_kmmkernel.cu:3-8).
@@ -40,6 +42,7 @@ struct KernelInfo {
   uint32_t variant;       // kernel-family specific
   CanRunFn canRun;
   LaunchFn launch;
+  CheckFn  check;
 };
 
 struct PlanStep { uint32_t lo, hi; int kernel; };   // factors [lo, hi], hi applied first
@@ -73,5 +76,6 @@ class KernelDB {
 
 // Filled in by each kernel family's translation unit.
 void registerGenericKernels(std::vector<KernelInfo>& out);
+void registerRowKernels(std::vector<KernelInfo>& out);
 
 }  // namespace fk

@@ -8,4 +8,8 @@ namespace fk {
 // Any shape, one factor per launch.
 hipError_t launchGenericStep(const StepArgs& a, DType dt, hipStream_t stream);
 
+// Four fused 16x16 fp32 factors on rows of exactly 16^4 columns, one workgroup per row.
+bool row16x4Supported(const StepArgs& a);
+hipError_t launchRow16x4(const StepArgs& a, hipStream_t stream);
+
 }  // namespace fk

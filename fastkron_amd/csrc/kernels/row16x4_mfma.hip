@@ -1,0 +1,200 @@
+// Whole-row kernel for four fused 16x16 fp32 factors (row length 16^4 = 65536, e.g. sgemkm
+// 1024 x 65536 with 16x16^4): one workgroup of 16 wave64s owns one row, keeps it in VGPRs
+// (64 per lane) and touches HBM exactly once for the read and once for the write.
+//
+//   Z[q1,q2,q3,q4] = alpha * sum_{k1..k4} X[k1,k2,k3,k4] F1[k1,q1] F2[k2,q2] F3[k3,q3] F4[k4,q4] (+ beta*Y)
+//
+// The reference cannot fuse this shape in one launch (its tile must fit 48 KB of shared memory,
+// reference src/gen_tuner_kernels.py:10,366; it runs 2 launches of 2 fused factors each).  Here the
+// row (256 KB) does not fit the 160 KB LDS either, so the LDS is only the exchange buffer:
+//
+//   stage 1  contract k3 then k4 with V_MFMA_F32_16X16X4_F32, chained in registers: the first
+//            product leaves D[i][j] in register i%4 of lane 16*(i/4)+j, which is exactly the A-operand
+//            layout (lane 16*k+i) of a second product that contracts the *row* index i of the first;
+//            the factor operand of the second product is loaded with its rows permuted (4*k + r)
+//            to match.  No data movement between the two steps.
+//   exch. 1  transpose (k1,k2) <-> (q3,q4) through LDS, in two halves of 128 KB, XOR-swizzled so that
+//            both the ds_write_b32 and the ds_read_b32 side hit 64 distinct banks.
+//   stage 2  contract k1 then k2 the same way.
+//   exch. 2  bring the result to the store layout (lane = 4 consecutive columns, 1 KB per wave store),
+//            again in two swizzled halves; ds_read_b128 on the way out.
+//
+// Algorithmic traffic: 4*65536 bytes read + 4*65536 bytes written per row (+ Y when beta != 0).
+#include <hip/hip_runtime.h>
+#include "../problem.h"
+#include "launch.h"
+
+namespace fk {
+
+typedef float f4 __attribute__((ext_vector_type(4)));
+
+#define MFMA16(a, b, c) __builtin_amdgcn_mfma_f32_16x16x4f32((a), (b), (c), 0, 0, 0)
+
+constexpr int kRowLen = 65536;
+constexpr int kLdsWords = 32768;           // 128 KB: one half of a row
+
+template <bool HAS_Y>
+__global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a) {
+  extern __shared__ float lds[];
+  const int tid = threadIdx.x;
+  const int l = tid & 63, w = tid >> 6;
+  const int i = l & 15, kb = l >> 4;
+  const uint32_t m = blockIdx.x, b = blockIdx.y;
+
+  const float* X = (const float*)a.in + (size_t)b * a.in_batch + (size_t)m * a.in_ldm;
+  float* Z = (float*)a.out + (size_t)b * a.out_batch + (size_t)m * a.out_ldm;
+
+  // Factor operands (B side of every product).  a.f[0] is the last factor (F4) ... a.f[3] the first (F1).
+  // First product of a chain: B_c[k][j] = F[4c + k][j]; second product: B_r[k][j] = F[4k + r][j].
+  float FA[4], FB[4], FC[4], FD[4];
+  {
+    const float* F4p = (const float*)a.f[0] + (size_t)b * a.f_batch[0];
+    const float* F3p = (const float*)a.f[1] + (size_t)b * a.f_batch[1];
+    const float* F2p = (const float*)a.f[2] + (size_t)b * a.f_batch[2];
+    const float* F1p = (const float*)a.f[3] + (size_t)b * a.f_batch[3];
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+      FA[c] = F3p[(int64_t)(4 * c + kb) * a.f_sp[1] + (int64_t)i * a.f_sq[1]];
+      FB[c] = F4p[(int64_t)(4 * kb + c) * a.f_sp[0] + (int64_t)i * a.f_sq[0]];
+      FC[c] = F1p[(int64_t)(4 * c + kb) * a.f_sp[3] + (int64_t)i * a.f_sq[3]];
+      FD[c] = F2p[(int64_t)(4 * kb + c) * a.f_sp[2] + (int64_t)i * a.f_sq[2]];
+    }
+  }
+
+  // ---- load: wave w reads the 16 KB of k1 = w; x[t][c] = X[k1=w][k2=t][k3=4c+kb][k4=i] ----
+  float x[16][4];
+  {
+    const float* xp = X + w * 4096 + l;
+#pragma unroll
+    for (int t = 0; t < 16; t++)
+#pragma unroll
+      for (int c = 0; c < 4; c++) x[t][c] = xp[t * 256 + c * 64];
+  }
+
+  // ---- stage 1: contract k3 (first product) and k4 (second product) ----
+#pragma unroll
+  for (int t = 0; t < 16; t++) {
+    f4 d = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int c = 0; c < 4; c++) d = MFMA16(x[t][c], FA[c], d);
+    f4 e = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int r = 0; r < 4; r++) e = MFMA16(d[r], FB[r], e);
+#pragma unroll
+    for (int r = 0; r < 4; r++) x[t][r] = e[r];       // = Y[k1=w][k2=t][q3=4kb+r][q4=i]
+  }
+
+  // ---- exchange 1: rows (q3,q4), columns (k1,k2); half h holds the rows with bit 1 of q3 == h ----
+  float z[16][4];
+#pragma unroll
+  for (int h = 0; h < 2; h++) {
+    if (h) __syncthreads();
+#pragma unroll
+    for (int t = 0; t < 16; t++)
+#pragma unroll
+      for (int rr = 0; rr < 2; rr++) {
+        const int row = (kb * 2 + rr) * 16 + i;
+        lds[row * 256 + ((w * 16 + t) ^ l)] = x[t][2 * h + rr];
+      }
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < 16; u++) {
+      if (((u >> 1) & 1) != h) continue;
+      const int row = ((u >> 2) * 2 + (u & 1)) * 16 + w;
+      const int swz = w + 16 * (u >> 2);
+#pragma unroll
+      for (int c = 0; c < 4; c++) z[u][c] = lds[row * 256 + ((c * 64 + l) ^ swz)];   // Y[k1=4c+kb][k2=i][q3=u][q4=w]
+    }
+  }
+  __syncthreads();
+
+  // ---- stage 2: contract k1 (first product) and k2 (second product) ----
+#pragma unroll
+  for (int u = 0; u < 16; u++) {
+    f4 d = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int c = 0; c < 4; c++) d = MFMA16(z[u][c], FC[c], d);
+    f4 e = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int r = 0; r < 4; r++) e = MFMA16(d[r], FD[r], e);
+#pragma unroll
+    for (int r = 0; r < 4; r++) z[u][r] = e[r];       // = Z[q1=4kb+r][q2=i][q3=u][q4=w]
+  }
+
+  // ---- exchange 2: rows (q1,q2), columns (q3,q4); half h holds the rows with bit 1 of q1 == h.
+  //      Reader: wave w owns q2 = w, lane owns columns 4l .. 4l+3, register index is q1. ----
+  f4 o[16];
+#pragma unroll
+  for (int h = 0; h < 2; h++) {
+    if (h) __syncthreads();
+#pragma unroll
+    for (int u = 0; u < 16; u++)
+#pragma unroll
+      for (int rr = 0; rr < 2; rr++) {
+        const int row = (kb * 2 + rr) * 16 + i;
+        lds[row * 256 + ((u * 16 + w) ^ (i * 4) ^ kb)] = z[u][2 * h + rr];
+      }
+    __syncthreads();
+#pragma unroll
+    for (int q1hi = 0; q1hi < 4; q1hi++)
+#pragma unroll
+      for (int rr = 0; rr < 2; rr++) {
+        const int row = (q1hi * 2 + rr) * 16 + w;
+        const f4 v = *(const f4*)&lds[row * 256 + ((l * 4) ^ (w * 4))];
+        f4 p;                                           // word e of v is column 4l + (e ^ q1hi)
+        p[0] = v[0 ^ q1hi]; p[1] = v[1 ^ q1hi]; p[2] = v[2 ^ q1hi]; p[3] = v[3 ^ q1hi];
+        o[4 * q1hi + 2 * h + rr] = p;
+      }
+  }
+
+  // ---- epilogue and store: every wave-level store covers 1 KB of contiguous columns ----
+  const float alpha = (float)a.alpha, beta = (float)a.beta;
+  const float* Y = HAS_Y ? (const float*)a.y + (size_t)b * a.y_batch + (size_t)m * a.y_ldm : nullptr;
+#pragma unroll
+  for (int q1 = 0; q1 < 16; q1++) {
+    const int col = q1 * 4096 + w * 256 + l * 4;
+    f4 v = o[q1];
+    if (a.epilogue) {
+      v = v * alpha;
+      if (HAS_Y) {
+        const f4 yv = *(const f4*)(Y + col);
+        v = v + yv * beta;
+      }
+    }
+    *(f4*)(Z + col) = v;
+  }
+}
+
+bool row16x4Supported(const StepArgs& a) {
+  if (a.nf != 4 || a.Kin != (uint64_t)kRowLen || a.Kout != (uint64_t)kRowLen) return false;
+  for (int j = 0; j < 4; j++) if (a.p[j] != 16 || a.q[j] != 16) return false;
+  if (a.in_ldc != 1 || a.out_ldc != 1) return false;
+  if (a.y && a.y_ldc != 1) return false;
+  // 16-byte aligned rows for the vector stores / Y loads
+  if (((uintptr_t)a.out & 15) || (a.out_ldm & 3) || (a.out_batch & 3)) return false;
+  if (a.y && (((uintptr_t)a.y & 15) || (a.y_ldm & 3) || (a.y_batch & 3))) return false;
+  return a.batch <= 65535;
+}
+
+hipError_t launchRow16x4(const StepArgs& a, hipStream_t stream) {
+  if (!row16x4Supported(a)) return hipErrorInvalidValue;
+  static bool attrSet = false;
+  const size_t ldsBytes = kLdsWords * sizeof(float);
+  if (!attrSet) {
+    hipError_t e = hipFuncSetAttribute((const void*)kron_row16x4_kernel<true>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes);
+    if (e != hipSuccess) return e;
+    e = hipFuncSetAttribute((const void*)kron_row16x4_kernel<false>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes);
+    if (e != hipSuccess) return e;
+    attrSet = true;
+  }
+  dim3 grid(a.M, a.batch), block(1024);
+  if (a.y && a.epilogue)
+    hipLaunchKernelGGL(kron_row16x4_kernel<true>, grid, block, ldsBytes, stream, a);
+  else
+    hipLaunchKernelGGL(kron_row16x4_kernel<false>, grid, block, ldsBytes, stream, a);
+  return hipGetLastError();
+}
+
+}  // namespace fk

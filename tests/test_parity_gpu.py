@@ -157,3 +157,18 @@ def test_tuned_and_online_plans_agree(tune):
         check(h, ko.KMM, 32, [4] * 5, [4] * 5, np.float64, alpha=2.0, beta=1.0, seed=5)
     finally:
         h.close()
+
+
+def test_whole_row_kernel_for_four_16x16_factors(fk):
+    """16x16^4 fp32 rows run as ONE launch of the register-resident row kernel, with and without Y,
+    batched, and with transposed factors (handled by the factor strides)."""
+    check(fk, ko.MKM, 5, [16] * 4, [16] * 4, np.float32, alpha=1.0, beta=0.0, seed=11)
+    plan = fk.last_plan()
+    assert len(plan) == 1 and "1x65536" in plan[0][2], plan
+    check(fk, ko.MKM, 3, [16] * 4, [16] * 4, np.float32, alpha=-1.5, beta=0.75, seed=12)
+    check(fk, ko.MKM, 2, [16] * 4, [16] * 4, np.float32, alpha=2.0, beta=1.0, seed=13, batch=3)
+    check(fk, ko.MKM, 2, [16] * 4, [16] * 4, np.float32, alpha=2.0, beta=1.0, seed=14, opFs=ko.OP_T)
+    assert len(fk.last_plan()) == 1
+    check(fk, ko.MKM, 2, [16] * 4, [16] * 4, np.float32, alpha=1.0, beta=0.0, seed=15, integer=True)
+    # five factors: the last four are fused by the row kernel only when the row is exactly 16^4 long
+    check(fk, ko.MKM, 2, [2] + [16] * 4, [2] + [16] * 4, np.float32, alpha=1.0, beta=0.5, seed=16)
