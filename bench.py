@@ -111,6 +111,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
     ap.add_argument("--sets", type=int, default=2, help="operand sets rotated between steps")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run 4 plain device copies of 256 MiB (a known-size kernel for scaling rocprof counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU only (no multi-GPU path exists); use --gpus 1", file=sys.stderr)
@@ -158,6 +160,13 @@ def main():
             e = fk.xgemkm(M, Ps, Qs, X, Fs, Z, alpha, beta, Y, t1, t2)
         if e != capi.SUCCESS:
             raise RuntimeError(f"{call} failed with fastKronError {e}")
+
+    if args.calibrate_copy:
+        src = torch.empty(64 * 1024 * 1024, device=dev, dtype=torch.float32).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(4):
+            dst.copy_(src)                    # reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
 
     for i in range(max(args.warmup, 1)):
         step(i)

@@ -7,7 +7,7 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libFastKron.so")
+LIB_PATH = os.environ.get("FASTKRON_LIB", os.path.join(_HERE, "lib", "libFastKron.so"))
 
 # enum values of include/fastkron.h
 OP_N, OP_T = 1, 2

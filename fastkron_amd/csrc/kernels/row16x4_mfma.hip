@@ -21,6 +21,8 @@
 //
 // Algorithmic traffic: 4*65536 bytes read + 4*65536 bytes written per row (+ Y when beta != 0).
 #include <hip/hip_runtime.h>
+#include <cstdio>
+#include <cstdlib>
 #include "../problem.h"
 #include "launch.h"
 
@@ -30,16 +32,45 @@ typedef float f4 __attribute__((ext_vector_type(4)));
 
 #define MFMA16(a, b, c) __builtin_amdgcn_mfma_f32_16x16x4f32((a), (b), (c), 0, 0, 0)
 
+#ifdef FK_ROW_TIMING
+// Experiment-only build: phase time stamps (s_memtime) of wave 0 of every workgroup.
+__device__ unsigned long long g_rowTiming[1024 * 8];
+#define FK_STAMP(k) do { if (tid == 0 && blockIdx.x < 1024) g_rowTiming[blockIdx.x * 8 + (k)] = __builtin_readcyclecounter(); } while (0)
+extern "C" void fkDebugReadRowTiming(unsigned long long* out) {
+  (void)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_rowTiming), sizeof(unsigned long long) * 1024 * 8);
+}
+#else
+#define FK_STAMP(k)
+#endif
+
 constexpr int kRowLen = 65536;
 constexpr int kLdsWords = 32768;           // 128 KB: one half of a row
 
 template <bool HAS_Y>
-__global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a) {
+__global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a, const uint32_t firstWave,
+                                                               const uint32_t groups, const uint32_t delayCycles) {
   extern __shared__ float lds[];
   const int tid = threadIdx.x;
+  // One workgroup fills a CU, so every CU alternates between an HBM phase (load, store) and an
+  // on-chip phase (MFMA, LDS exchange).  Workgroups that start together stay in lockstep and leave
+  // HBM idle during the on-chip phases; delaying a part of the first wave of workgroups by a fraction
+  // of the row period interleaves the phases of different CUs.  Later workgroups inherit the offset.
+  if (groups > 1) {
+    const uint32_t wg = blockIdx.x + blockIdx.y * gridDim.x;
+    const uint32_t g = (wg >> 3) % groups;   // workgroups go round-robin over the 8 XCDs: keep every group on every XCD
+    if (wg < firstWave && g != 0) {
+      const uint64_t t0 = __builtin_readcyclecounter();
+      const uint64_t wait = (uint64_t)g * delayCycles;
+      while (__builtin_readcyclecounter() - t0 < wait) __builtin_amdgcn_s_sleep(16);
+    }
+  }
   const int l = tid & 63, w = tid >> 6;
   const int i = l & 15, kb = l >> 4;
   const uint32_t m = blockIdx.x, b = blockIdx.y;
+  FK_STAMP(0);
+#ifdef FK_ROW_TIMING
+  if (tid == 0 && blockIdx.x < 1024) g_rowTiming[blockIdx.x * 8 + 6] = wall_clock64();
+#endif
 
   const float* X = (const float*)a.in + (size_t)b * a.in_batch + (size_t)m * a.in_ldm;
   float* Z = (float*)a.out + (size_t)b * a.out_batch + (size_t)m * a.out_ldm;
@@ -84,6 +115,7 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a)
     for (int r = 0; r < 4; r++) x[t][r] = e[r];       // = Y[k1=w][k2=t][q3=4kb+r][q4=i]
   }
 
+  FK_STAMP(1);
   // ---- exchange 1: rows (q3,q4), columns (k1,k2); half h holds the rows with bit 1 of q3 == h ----
   float z[16][4];
 #pragma unroll
@@ -107,6 +139,7 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a)
     }
   }
   __syncthreads();
+  FK_STAMP(2);
 
   // ---- stage 2: contract k1 (first product) and k2 (second product) ----
 #pragma unroll
@@ -121,6 +154,7 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a)
     for (int r = 0; r < 4; r++) z[u][r] = e[r];       // = Z[q1=4kb+r][q2=i][q3=u][q4=w]
   }
 
+  FK_STAMP(3);
   // ---- exchange 2: rows (q1,q2), columns (q3,q4); half h holds the rows with bit 1 of q1 == h.
   //      Reader: wave w owns q2 = w, lane owns columns 4l .. 4l+3, register index is q1. ----
   f4 o[16];
@@ -147,6 +181,7 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a)
       }
   }
 
+  FK_STAMP(4);
   // ---- epilogue and store: every wave-level store covers 1 KB of contiguous columns ----
   const float alpha = (float)a.alpha, beta = (float)a.beta;
   const float* Y = HAS_Y ? (const float*)a.y + (size_t)b * a.y_batch + (size_t)m * a.y_ldm : nullptr;
@@ -163,6 +198,10 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a)
     }
     *(f4*)(Z + col) = v;
   }
+  FK_STAMP(5);
+#ifdef FK_ROW_TIMING
+  if (tid == 0 && blockIdx.x < 1024) g_rowTiming[blockIdx.x * 8 + 7] = wall_clock64();
+#endif
 }
 
 bool row16x4Supported(const StepArgs& a) {
@@ -190,10 +229,24 @@ hipError_t launchRow16x4(const StepArgs& a, hipStream_t stream) {
     attrSet = true;
   }
   dim3 grid(a.M, a.batch), block(1024);
+  static int cus = 0;
+  static uint32_t groups = 2, delay = 1100;            // delay in s_memtime ticks (100 MHz): 11 us
+  if (!cus) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) cus = prop.multiProcessorCount;
+    else cus = 256;
+    if (const char* e = getenv("FASTKRON_ROW_STAGGER")) {   // "<groups>,<ticks>" for experiments
+      unsigned g = 0, d = 0;
+      if (sscanf(e, "%u,%u", &g, &d) == 2) { groups = g; delay = d; }
+    }
+  }
+  const uint32_t firstWave = (uint32_t)cus;
+  const uint32_t g = ((uint64_t)a.M * a.batch > (uint64_t)cus) ? groups : 1;   // a single wave of rows gains nothing
   if (a.y && a.epilogue)
-    hipLaunchKernelGGL(kron_row16x4_kernel<true>, grid, block, ldsBytes, stream, a);
+    hipLaunchKernelGGL(kron_row16x4_kernel<true>, grid, block, ldsBytes, stream, a, firstWave, g, delay);
   else
-    hipLaunchKernelGGL(kron_row16x4_kernel<false>, grid, block, ldsBytes, stream, a);
+    hipLaunchKernelGGL(kron_row16x4_kernel<false>, grid, block, ldsBytes, stream, a, firstWave, g, delay);
   return hipGetLastError();
 }
 
