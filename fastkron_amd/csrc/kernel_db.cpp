@@ -52,6 +52,18 @@ static bool row16CanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, 
 static hipError_t row16Launch(const KernelInfo&, const StepArgs& a, hipStream_t s) { return launchRow16x4(a, s); }
 static bool row16Check(const KernelInfo&, const StepArgs& a) { return row16x4Supported(a); }
 
+// ---- whole-row kernel for five fused 8x8 fp32 factors ----
+static bool row8CanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
+                       const DeviceInfo& dev) {
+  if (p.dt != DType::F32 || p.mm != MMType::MKM || hi - lo + 1 != 5 || p.forward) return false;
+  for (uint32_t i = lo; i <= hi; i++) if (p.P[i] != 8 || p.Q[i] != 8) return false;
+  if (p.colsBefore(hi) != 32768) return false;
+  if (first && p.opX == 2) return false;
+  return dev.ldsPerBlock >= 67000 && k.dt == p.dt;
+}
+static hipError_t row8Launch(const KernelInfo&, const StepArgs& a, hipStream_t s) { return launchRow8x5(a, s); }
+static bool row8Check(const KernelInfo&, const StepArgs& a) { return row8x5Supported(a); }
+
 void registerRowKernels(std::vector<KernelInfo>& out) {
   KernelInfo k{};
   // grammar: <mm>_<backend>_<arch>_<threads>_<type>_<PxQ>_<TilePxTileQ>_<fused>_<TileMxTileK>_<regs>_<ops>_<batch>_<p2p>_<opt>
@@ -59,6 +71,12 @@ void registerRowKernels(std::vector<KernelInfo>& out) {
   k.dt = DType::F32; k.P = 16; k.Q = 16; k.fused = 4; k.tileM = 1; k.tileK = 65536; k.threads = 1024; k.variant = 0;
   k.canRun = row16CanRun; k.launch = row16Launch; k.check = row16Check;
   out.push_back(k);
+
+  KernelInfo k8{};
+  k8.name = "mkm_hip_gfx950_512_f_8x8_8x8_5_1x32768_mfma4x4x1_NN_strided_0_3";
+  k8.dt = DType::F32; k8.P = 8; k8.Q = 8; k8.fused = 5; k8.tileM = 1; k8.tileK = 32768; k8.threads = 512; k8.variant = 0;
+  k8.canRun = row8CanRun; k8.launch = row8Launch; k8.check = row8Check;
+  out.push_back(k8);
 }
 
 KernelDB::KernelDB() {

@@ -172,3 +172,15 @@ def test_whole_row_kernel_for_four_16x16_factors(fk):
     check(fk, ko.MKM, 2, [16] * 4, [16] * 4, np.float32, alpha=1.0, beta=0.0, seed=15, integer=True)
     # five factors: the last four are fused by the row kernel only when the row is exactly 16^4 long
     check(fk, ko.MKM, 2, [2] + [16] * 4, [2] + [16] * 4, np.float32, alpha=1.0, beta=0.5, seed=16)
+
+
+def test_whole_row_kernel_for_five_8x8_factors(fk):
+    """8x8^5 fp32 rows run as ONE launch of the register-resident 4x4x1-MFMA row kernel."""
+    check(fk, ko.MKM, 5, [8] * 5, [8] * 5, np.float32, alpha=1.0, beta=0.0, seed=21)
+    plan = fk.last_plan()
+    assert len(plan) == 1 and "1x32768" in plan[0][2], plan
+    check(fk, ko.MKM, 3, [8] * 5, [8] * 5, np.float32, alpha=-1.5, beta=0.75, seed=22)
+    check(fk, ko.MKM, 2, [8] * 5, [8] * 5, np.float32, alpha=2.0, beta=1.0, seed=23, batch=3)
+    check(fk, ko.MKM, 2, [8] * 5, [8] * 5, np.float32, alpha=2.0, beta=1.0, seed=24, opFs=ko.OP_T)
+    check(fk, ko.MKM, 2, [8] * 5, [8] * 5, np.float32, alpha=1.0, beta=0.0, seed=25, integer=True)
+    check(fk, ko.MKM, 2, [3] + [8] * 5, [2] + [8] * 5, np.float32, alpha=1.0, beta=0.5, seed=26)
