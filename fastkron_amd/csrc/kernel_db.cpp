@@ -64,6 +64,18 @@ static bool row8CanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, u
 static hipError_t row8Launch(const KernelInfo&, const StepArgs& a, hipStream_t s) { return launchRow8x5(a, s); }
 static bool row8Check(const KernelInfo&, const StepArgs& a) { return row8x5Supported(a); }
 
+// ---- whole-row kernel for three fused 32x16 fp32 factors ----
+static bool row32CanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
+                        const DeviceInfo&) {
+  if (p.dt != DType::F32 || p.mm != MMType::MKM || hi - lo + 1 != 3 || p.forward) return false;
+  for (uint32_t i = lo; i <= hi; i++) if (p.P[i] != 32 || p.Q[i] != 16) return false;
+  if (p.colsBefore(hi) != 32768) return false;
+  if (first && p.opX == 2) return false;
+  return k.dt == p.dt;
+}
+static hipError_t row32Launch(const KernelInfo&, const StepArgs& a, hipStream_t s) { return launchRow32x16x3(a, s); }
+static bool row32Check(const KernelInfo&, const StepArgs& a) { return row32x16x3Supported(a); }
+
 void registerRowKernels(std::vector<KernelInfo>& out) {
   KernelInfo k{};
   // grammar: <mm>_<backend>_<arch>_<threads>_<type>_<PxQ>_<TilePxTileQ>_<fused>_<TileMxTileK>_<regs>_<ops>_<batch>_<p2p>_<opt>
@@ -77,6 +89,12 @@ void registerRowKernels(std::vector<KernelInfo>& out) {
   k8.dt = DType::F32; k8.P = 8; k8.Q = 8; k8.fused = 5; k8.tileM = 1; k8.tileK = 32768; k8.threads = 512; k8.variant = 0;
   k8.canRun = row8CanRun; k8.launch = row8Launch; k8.check = row8Check;
   out.push_back(k8);
+
+  KernelInfo k32{};
+  k32.name = "mkm_hip_gfx950_512_f_32x16_32x16_3_1x32768_mfma16x16x4_NN_strided_0_3";
+  k32.dt = DType::F32; k32.P = 32; k32.Q = 16; k32.fused = 3; k32.tileM = 1; k32.tileK = 32768; k32.threads = 512;
+  k32.variant = 0; k32.canRun = row32CanRun; k32.launch = row32Launch; k32.check = row32Check;
+  out.push_back(k32);
 }
 
 KernelDB::KernelDB() {

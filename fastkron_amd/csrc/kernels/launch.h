@@ -16,4 +16,8 @@ hipError_t launchRow16x4(const StepArgs& a, hipStream_t stream);
 bool row8x5Supported(const StepArgs& a);
 hipError_t launchRow8x5(const StepArgs& a, hipStream_t stream);
 
+// Three fused 32x16 fp32 factors on rows of exactly 32^3 columns, one workgroup per row, two per CU.
+bool row32x16x3Supported(const StepArgs& a);
+hipError_t launchRow32x16x3(const StepArgs& a, hipStream_t stream);
+
 }  // namespace fk

@@ -184,3 +184,16 @@ def test_whole_row_kernel_for_five_8x8_factors(fk):
     check(fk, ko.MKM, 2, [8] * 5, [8] * 5, np.float32, alpha=2.0, beta=1.0, seed=24, opFs=ko.OP_T)
     check(fk, ko.MKM, 2, [8] * 5, [8] * 5, np.float32, alpha=1.0, beta=0.0, seed=25, integer=True)
     check(fk, ko.MKM, 2, [3] + [8] * 5, [2] + [8] * 5, np.float32, alpha=1.0, beta=0.5, seed=26)
+
+
+def test_whole_row_kernel_for_three_32x16_factors(fk):
+    """32x16^3 fp32 rows (non-square, which the reference never fuses) run as ONE launch."""
+    check(fk, ko.MKM, 5, [32] * 3, [16] * 3, np.float32, alpha=1.0, beta=0.0, seed=31)
+    plan = fk.last_plan()
+    assert len(plan) == 1 and "32x16" in plan[0][2] and "1x32768" in plan[0][2], plan
+    check(fk, ko.MKM, 3, [32] * 3, [16] * 3, np.float32, alpha=-1.5, beta=0.75, seed=32)
+    check(fk, ko.MKM, 4, [32] * 3, [16] * 3, np.float32, alpha=1.0, beta=1.0, seed=33, batch=5)
+    check(fk, ko.MKM, 4, [32] * 3, [16] * 3, np.float32, alpha=1.0, beta=1.0, seed=34, batch=3, share_f=True)
+    check(fk, ko.MKM, 2, [32] * 3, [16] * 3, np.float32, alpha=2.0, beta=1.0, seed=35, opFs=ko.OP_T)
+    check(fk, ko.MKM, 2, [32] * 3, [16] * 3, np.float32, alpha=1.0, beta=0.0, seed=36, integer=True)
+    check(fk, ko.MKM, 2, [2] + [32] * 3, [3] + [16] * 3, np.float32, alpha=1.0, beta=0.5, seed=37)
