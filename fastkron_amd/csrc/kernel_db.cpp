@@ -76,6 +76,17 @@ static bool row32CanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, 
 static hipError_t row32Launch(const KernelInfo&, const StepArgs& a, hipStream_t s) { return launchRow32x16x3(a, s); }
 static bool row32Check(const KernelInfo&, const StepArgs& a) { return row32x16x3Supported(a); }
 
+// ---- fp64 single-factor MFMA step ----
+static bool stepF64CanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
+                          const DeviceInfo& dev) {
+  if (p.dt != DType::F64 || p.mm != MMType::MKM || lo != hi) return false;
+  if (p.P[lo] != k.P || p.Q[lo] != k.Q) return false;
+  if (first && p.opX == 2) return false;
+  return (int)((64 * (k.P + 1) + k.P * (k.Q + 1)) * 8) <= dev.ldsPerBlock;
+}
+static hipError_t stepF64Launch(const KernelInfo&, const StepArgs& a, hipStream_t s) { return launchStepMfmaF64(a, s); }
+static bool stepF64Check(const KernelInfo&, const StepArgs& a) { return stepMfmaF64Supported(a); }
+
 void registerRowKernels(std::vector<KernelInfo>& out) {
   KernelInfo k{};
   // grammar: <mm>_<backend>_<arch>_<threads>_<type>_<PxQ>_<TilePxTileQ>_<fused>_<TileMxTileK>_<regs>_<ops>_<batch>_<p2p>_<opt>
@@ -95,6 +106,16 @@ void registerRowKernels(std::vector<KernelInfo>& out) {
   k32.dt = DType::F32; k32.P = 32; k32.Q = 16; k32.fused = 3; k32.tileM = 1; k32.tileK = 32768; k32.threads = 512;
   k32.variant = 0; k32.canRun = row32CanRun; k32.launch = row32Launch; k32.check = row32Check;
   out.push_back(k32);
+
+  for (uint32_t P : {16u, 32u, 64u}) {
+    KernelInfo kd{};
+    const std::string ps = std::to_string(P);
+    kd.name = "mkm_hip_gfx950_256_d_" + ps + "x" + ps + "_" + ps + "x" + ps + "_1_1x" + std::to_string(64 * P) +
+              "_mfma16x16x4_NN_strided_0_3";
+    kd.dt = DType::F64; kd.P = P; kd.Q = P; kd.fused = 1; kd.tileM = 1; kd.tileK = 64 * P; kd.threads = 256; kd.variant = 0;
+    kd.canRun = stepF64CanRun; kd.launch = stepF64Launch; kd.check = stepF64Check;
+    out.push_back(kd);
+  }
 }
 
 KernelDB::KernelDB() {
@@ -126,8 +147,8 @@ Plan KernelDB::selectOnline(const KronProblem& p, const DeviceInfo& dev, bool al
   int hi = (int)p.N - 1;
   while (hi >= 0) {
     int bestLo = hi, bestK = genericKernel(p.dt);
-    if (!p.forward) {
-      const uint32_t maxDepth = allowFusion ? kMaxFused : 1;
+    {
+      const uint32_t maxDepth = (allowFusion && !p.forward) ? kMaxFused : 1;   // forward keeps every step's output
       for (int lo = (hi + 1 >= (int)maxDepth) ? hi + 1 - (int)maxDepth : 0; lo <= hi; lo++) {
         auto c = candidates(p, (uint32_t)lo, (uint32_t)hi, hi == (int)p.N - 1, lo == 0, dev);
         int pick = -1;

@@ -20,4 +20,8 @@ hipError_t launchRow8x5(const StepArgs& a, hipStream_t stream);
 bool row32x16x3Supported(const StepArgs& a);
 hipError_t launchRow32x16x3(const StepArgs& a, hipStream_t stream);
 
+// One fp64 step with a 16x16 / 32x32 / 64x64 factor on the fp64 matrix cores (MKM layout).
+bool stepMfmaF64Supported(const StepArgs& a);
+hipError_t launchStepMfmaF64(const StepArgs& a, hipStream_t stream);
+
 }  // namespace fk

@@ -197,3 +197,13 @@ def test_whole_row_kernel_for_three_32x16_factors(fk):
     check(fk, ko.MKM, 2, [32] * 3, [16] * 3, np.float32, alpha=2.0, beta=1.0, seed=35, opFs=ko.OP_T)
     check(fk, ko.MKM, 2, [32] * 3, [16] * 3, np.float32, alpha=1.0, beta=0.0, seed=36, integer=True)
     check(fk, ko.MKM, 2, [2] + [32] * 3, [3] + [16] * 3, np.float32, alpha=1.0, beta=0.5, seed=37)
+
+
+@pytest.mark.parametrize("M,Ps", [(3, [64]), (2, [16, 16]), (5, [32, 32]), (2, [64, 64, 64]), (7, [16] * 4), (4, [64, 16, 32])])
+def test_fp64_mfma_step_kernel(fk, M, Ps):
+    """fp64 steps with 16/32/64-wide square factors run on the fp64 matrix cores, including tiles with
+    fewer than 64 slices and mixed chains."""
+    check(fk, ko.MKM, M, Ps, Ps, np.float64, alpha=1.5, beta=0.5, seed=41)
+    assert all("mfma16x16x4" in k for _, _, k in fk.last_plan()), fk.last_plan()
+    check(fk, ko.MKM, M, Ps, Ps, np.float64, alpha=1.0, beta=0.0, seed=42, opFs=ko.OP_T)
+    check(fk, ko.MKM, M, Ps, Ps, np.float64, alpha=1.0, beta=1.0, seed=43, batch=2)
