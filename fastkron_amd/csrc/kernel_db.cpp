@@ -88,6 +88,17 @@ static bool stepF64CanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo
 static hipError_t stepF64Launch(const KernelInfo&, const StepArgs& a, hipStream_t s) { return launchStepMfmaF64(a, s); }
 static bool stepF64Check(const KernelInfo&, const StepArgs& a) { return stepMfmaF64Supported(a); }
 
+// ---- KMM-layout register kernel: NF fused PxP fp32 factors with P^NF = 64 ----
+static bool kmmRegCanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
+                         const DeviceInfo&) {
+  if (p.dt != DType::F32 || p.mm != MMType::KMM || hi - lo + 1 != k.fused || p.forward) return false;
+  for (uint32_t i = lo; i <= hi; i++) if (p.P[i] != k.P || p.Q[i] != k.Q) return false;
+  if (first && p.opX == 2) return false;
+  return p.colsBefore(hi) % 64 == 0 && p.M >= 16;
+}
+static hipError_t kmmRegLaunch(const KernelInfo&, const StepArgs& a, hipStream_t s) { return launchKmmReg(a, s); }
+static bool kmmRegCheck(const KernelInfo&, const StepArgs& a) { return kmmRegSupported(a); }
+
 void registerRowKernels(std::vector<KernelInfo>& out) {
   KernelInfo k{};
   // grammar: <mm>_<backend>_<arch>_<threads>_<type>_<PxQ>_<TilePxTileQ>_<fused>_<TileMxTileK>_<regs>_<ops>_<batch>_<p2p>_<opt>
@@ -107,6 +118,17 @@ void registerRowKernels(std::vector<KernelInfo>& out) {
   k32.dt = DType::F32; k32.P = 32; k32.Q = 16; k32.fused = 3; k32.tileM = 1; k32.tileK = 32768; k32.threads = 512;
   k32.variant = 0; k32.canRun = row32CanRun; k32.launch = row32Launch; k32.check = row32Check;
   out.push_back(k32);
+
+  for (uint32_t P : {4u, 8u}) {
+    KernelInfo kk{};
+    const std::string ps = std::to_string(P);
+    kk.fused = (P == 4) ? 3 : 2;
+    kk.name = "kmm_hip_gfx950_256_f_" + ps + "x" + ps + "_" + ps + "x" + ps + "_" + std::to_string(kk.fused) +
+              "_64x64_mfma4x4x1_NN_strided_0_3";
+    kk.dt = DType::F32; kk.P = P; kk.Q = P; kk.tileM = 64; kk.tileK = 64; kk.threads = 256; kk.variant = 0;
+    kk.canRun = kmmRegCanRun; kk.launch = kmmRegLaunch; kk.check = kmmRegCheck;
+    out.push_back(kk);
+  }
 
   for (uint32_t P : {16u, 32u, 64u}) {
     KernelInfo kd{};

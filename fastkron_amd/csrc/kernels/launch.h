@@ -24,4 +24,8 @@ hipError_t launchRow32x16x3(const StepArgs& a, hipStream_t stream);
 bool stepMfmaF64Supported(const StepArgs& a);
 hipError_t launchStepMfmaF64(const StepArgs& a, hipStream_t stream);
 
+// KMM layout, fp32: three fused 4x4 or two fused 8x8 factors held in registers, lanes along M.
+bool kmmRegSupported(const StepArgs& a);
+hipError_t launchKmmReg(const StepArgs& a, hipStream_t stream);
+
 }  // namespace fk

@@ -207,3 +207,15 @@ def test_fp64_mfma_step_kernel(fk, M, Ps):
     assert all("mfma16x16x4" in k for _, _, k in fk.last_plan()), fk.last_plan()
     check(fk, ko.MKM, M, Ps, Ps, np.float64, alpha=1.0, beta=0.0, seed=42, opFs=ko.OP_T)
     check(fk, ko.MKM, M, Ps, Ps, np.float64, alpha=1.0, beta=1.0, seed=43, batch=2)
+
+
+@pytest.mark.parametrize("M,Ps", [(64, [4] * 6), (100, [4] * 3), (16, [4] * 6), (130, [8] * 2), (64, [8] * 4),
+                                  (70, [4] * 5), (33, [8] * 3)])
+def test_kmm_register_kernel(fk, M, Ps):
+    """KMM with 4x4 / 8x8 fp32 factors: three (two) factors per launch held in registers, lanes along M,
+    including column counts that are not a multiple of 64 and chains with a generic remainder."""
+    check(fk, ko.KMM, M, Ps, Ps, np.float32, alpha=1.5, beta=0.5, seed=51)
+    assert any("mfma4x4x1" in k for _, _, k in fk.last_plan()), fk.last_plan()
+    check(fk, ko.KMM, M, Ps, Ps, np.float32, alpha=1.0, beta=0.0, seed=52, opFs=ko.OP_T)
+    check(fk, ko.KMM, M, Ps, Ps, np.float32, alpha=1.0, beta=1.0, seed=53, batch=2)
+    check(fk, ko.KMM, M, Ps, Ps, np.float32, alpha=2.0, beta=1.0, seed=54, use_temp2=False)
