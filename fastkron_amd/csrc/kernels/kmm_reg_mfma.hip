@@ -36,7 +36,8 @@ __global__ __launch_bounds__(256, 4) void kron_kmm_reg_kernel(const StepArgs a, 
   constexpr int G = KmmRegCfg<P, NF>::G;
   constexpr int QQ = P / 4;
   const int tid = threadIdx.x;
-  const int l = tid & 63, w = tid >> 6;
+  const int l = tid & 63;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);      // wave-uniform: keeps row addresses in SGPRs
   const uint32_t bt = blockIdx.y;
   const uint64_t SG = a.Kin / G;
   const uint32_t t = blockIdx.x * kKmmWaves + w;
@@ -89,18 +90,28 @@ __global__ __launch_bounds__(256, 4) void kron_kmm_reg_kernel(const StepArgs a, 
 
   if (!valid) return;
   float* out = (float*)a.out + (size_t)bt * a.out_batch + (size_t)m * a.out_ldm;
-  const float* Y = HAS_Y ? (const float*)a.y + (size_t)bt * a.y_batch + (size_t)m * a.y_ldm : nullptr;
   const float alpha = (float)a.alpha, beta = (float)a.beta;
+  if (a.epilogue) {
+    if (HAS_Y) {
+      // Every Y load is issued before the first store (on gfx9 loads and stores share one in-order
+      // counter, so a load behind a store could only be waited for together with that store); a
+      // rolling window of 16 registers keeps the loads in flight.
+      const float* Y = (const float*)a.y + (size_t)bt * a.y_batch + (size_t)m * a.y_ldm;
+      float yw[16];
 #pragma unroll
-  for (int e = 0; e < G; e++) {
-    const uint64_t col = (uint64_t)e * SG + sg;
-    float v = x[e];
-    if (a.epilogue) {
-      v *= alpha;
-      if (HAS_Y) v += beta * Y[(int64_t)col * a.y_ldc];
+      for (int e = 0; e < 16; e++) yw[e] = Y[(int64_t)((uint64_t)e * SG + sg) * a.y_ldc];
+#pragma unroll
+      for (int e = 0; e < G; e++) {
+        x[e] = alpha * x[e] + beta * yw[e & 15];
+        if (e + 16 < G) yw[e & 15] = Y[(int64_t)((uint64_t)(e + 16) * SG + sg) * a.y_ldc];
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < G; e++) x[e] *= alpha;
     }
-    out[(int64_t)col * a.out_ldc] = v;
   }
+#pragma unroll
+  for (int e = 0; e < G; e++) out[(int64_t)((uint64_t)e * SG + sg) * a.out_ldc] = x[e];
 }
 
 bool kmmRegSupported(const StepArgs& a) {

@@ -64,7 +64,8 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a,
       while (__builtin_readcyclecounter() - t0 < wait) __builtin_amdgcn_s_sleep(16);
     }
   }
-  const int l = tid & 63, w = tid >> 6;
+  const int l = tid & 63;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);      // wave-uniform: keeps row addresses in SGPRs
   const int i = l & 15, kb = l >> 4;
   const uint32_t m = blockIdx.x, b = blockIdx.y;
   FK_STAMP(0);

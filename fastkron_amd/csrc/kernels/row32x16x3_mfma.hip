@@ -31,7 +31,8 @@ template <bool HAS_Y>
 __global__ __launch_bounds__(512, 4) void kron_row32x16x3_kernel(const StepArgs a) {
   extern __shared__ float lds[];
   const int tid = threadIdx.x;
-  const int l = tid & 63, w = tid >> 6;
+  const int l = tid & 63;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);      // wave-uniform: keeps row addresses in SGPRs
   const int lo = l & 15, hi = l >> 4;
   const uint32_t m = blockIdx.x, bt = blockIdx.y;
 
@@ -42,6 +43,17 @@ __global__ __launch_bounds__(512, 4) void kron_row32x16x3_kernel(const StepArgs 
   const float* F3p = (const float*)a.f[0] + (size_t)bt * a.f_batch[0];
   const float* F2p = (const float*)a.f[1] + (size_t)bt * a.f_batch[1];
   const float* F1p = (const float*)a.f[2] + (size_t)bt * a.f_batch[2];
+
+  // Y first (8 values per lane, in the store layout): on gfx9 loads and stores share one in-order
+  // counter, so a load issued after a store could only be waited for together with that store.
+  const float* Y = HAS_Y ? (const float*)a.y + (size_t)bt * a.y_batch + (size_t)m * a.y_ldm : nullptr;
+  float yv[2][4];
+  if (HAS_Y) {
+#pragma unroll
+    for (int bq = 0; bq < 2; bq++)
+#pragma unroll
+      for (int r = 0; r < 4; r++) yv[bq][r] = Y[(4 * hi + r) * 256 + (2 * w + bq) * 16 + lo];
+  }
 
   // ---- load: x[g][h][c] = X[k1 = 4w+g][k2 = 4c+hi][k3 = 16h+lo] ----
   float x[4][2][8];
@@ -108,7 +120,6 @@ __global__ __launch_bounds__(512, 4) void kron_row32x16x3_kernel(const StepArgs 
   for (int c = 0; c < 8; c++) FC[c] = F1p[(int64_t)(4 * c + hi) * a.f_sp[2] + (int64_t)lo * a.f_sq[2]];
 
   const float alpha = (float)a.alpha, beta = (float)a.beta;
-  const float* Y = HAS_Y ? (const float*)a.y + (size_t)bt * a.y_batch + (size_t)m * a.y_ldm : nullptr;
 #pragma unroll
   for (int bq = 0; bq < 2; bq++) {
     f4 d = {0.f, 0.f, 0.f, 0.f};
@@ -122,7 +133,7 @@ __global__ __launch_bounds__(512, 4) void kron_row32x16x3_kernel(const StepArgs 
       float v = d[r];
       if (a.epilogue) {
         v *= alpha;
-        if (HAS_Y) v += beta * Y[col];
+        if (HAS_Y) v += beta * yv[bq][r];
       }
       Z[col] = v;
     }

@@ -77,7 +77,8 @@ __global__ __launch_bounds__(512, 4) void kron_row8x5_kernel(const StepArgs a) {
   extern __shared__ float lds[];
   float* fl = lds + 16384;                       // factors: fl[f*64 + p*8 + q], f = 0 is F1
   const int tid = threadIdx.x;
-  const int l = tid & 63, w = tid >> 6;
+  const int l = tid & 63;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);      // wave-uniform: keeps row addresses in SGPRs
   const uint32_t m = blockIdx.x, bt = blockIdx.y;
 
   const float* X = (const float*)a.in + (size_t)bt * a.in_batch + (size_t)m * a.in_ldm;

@@ -38,7 +38,8 @@ __global__ __launch_bounds__(256, 2) void kron_step_mfma_f64_kernel(const StepAr
   constexpr int PC = P / 4;              // products per tile and doubles per lane
   constexpr int NB = Q / 16;
   const int tid = threadIdx.x;
-  const int l = tid & 63, w = tid >> 6;
+  const int l = tid & 63;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);      // wave-uniform: keeps row addresses in SGPRs
   const int lo = l & 15, hi = l >> 4;
   const uint32_t bt = blockIdx.y;
   const uint64_t S = a.Kin / P;
@@ -92,6 +93,14 @@ __global__ __launch_bounds__(256, 2) void kron_step_mfma_f64_kernel(const StepAr
     if (s >= S) continue;
     double* out = outB + (size_t)m * a.out_ldm;
     const double* Y = HAS_Y ? YB + (size_t)m * a.y_ldm : nullptr;
+    // all Y loads of the tile before its first store (loads and stores share one in-order counter)
+    double yv[HAS_Y ? NB : 1][4];
+    if (HAS_Y) {
+#pragma unroll
+      for (int ib = 0; ib < NB; ib++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) yv[ib][r] = Y[(uint64_t)(16 * ib + 4 * r + hi) * S + s];
+    }
 #pragma unroll
     for (int ib = 0; ib < NB; ib++)
 #pragma unroll
@@ -100,7 +109,7 @@ __global__ __launch_bounds__(256, 2) void kron_step_mfma_f64_kernel(const StepAr
         double v = acc[ib][r];
         if (a.epilogue) {
           v *= alpha;
-          if (HAS_Y) v += beta * Y[col];
+          if (HAS_Y) v += beta * yv[ib][r];
         }
         out[col] = v;
       }
