@@ -110,3 +110,20 @@ def test_gemm_argument_checks_return_before_touching_a_device(handle):
     callk = lambda Z: lib.dgekmm(h, capi.BACKEND_HIP, 2, Qs, Ps, 4, fs, capi.OP_N, fake, capi.OP_N, Z,
                                  ctypes.c_double(1), ctypes.c_double(0), None, fake, None)
     assert callk(None) == capi.INVALID_ARGUMENT
+
+
+def test_extension_symbols_and_last_plan_before_any_call(handle):
+    lib, h = handle
+    for n in capi.EXT_EXPORTS:                      # include/fastkron_ext.h
+        assert hasattr(lib, n), n
+    buf = ctypes.create_string_buffer(64)
+    assert lib.fastKronGetLastPlan(h, buf, 64) == 0
+    assert lib.fastKronSetTunedDB(h, None) == capi.SUCCESS
+
+
+def test_tuned_plan_file_round_trip(tmp_path, handle):
+    """A tuned-plan file written by hand is accepted; unknown kernel names are ignored at lookup time."""
+    lib, h = handle
+    f = tmp_path / "tuned.db"
+    f.write_text("# comment\n8x64*(8x8^2)_NN_f 0.01 1 0 1 no_such_kernel\n")
+    assert lib.fastKronSetTunedDB(h, str(f).encode()) == capi.SUCCESS
