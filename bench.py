@@ -149,15 +149,19 @@ def main():
     t1 = torch.empty(batch * te, device=dev, dtype=tdt)
     t2 = torch.empty(batch * te, device=dev, dtype=tdt)
 
-    def step(i):
-        X, Fs, Y, Z = sets[i % len(sets)]
+    # the ctypes arguments of every operand set are marshalled once; a step is then one C call
+    calls = []
+    for X, Fs, Y, Z in sets:
         if call == "sgemkmStridedBatched":
-            e = fk.xgemkm_strided_batched(M, Ps, Qs, X, M * K, Fs, [p * q for p, q in zip(Ps, Qs)], Z, M * L, batch,
-                                          alpha, beta, Y, M * L, t1, t2)
+            calls.append(fk.prepared("xgemkm_strided_batched", M, Ps, Qs, X, M * K, Fs, [p * q for p, q in zip(Ps, Qs)],
+                                     Z, M * L, batch, alpha, beta, Y, M * L, t1, t2))
         elif call == "sgekmm":
-            e = fk.xgekmm(M, Ps, Qs, X, Fs, Z, alpha, beta, Y, t1, t2)
+            calls.append(fk.prepared("xgekmm", M, Ps, Qs, X, Fs, Z, alpha, beta, Y, t1, t2))
         else:
-            e = fk.xgemkm(M, Ps, Qs, X, Fs, Z, alpha, beta, Y, t1, t2)
+            calls.append(fk.prepared("xgemkm", M, Ps, Qs, X, Fs, Z, alpha, beta, Y, t1, t2))
+
+    def step(i):
+        e = calls[i % len(calls)]()
         if e != capi.SUCCESS:
             raise RuntimeError(f"{call} failed with fastKronError {e}")
 

@@ -139,6 +139,28 @@ class FastKron:
                   capi.arr_ptr([f.data_ptr() for f in Fs]), opFs, capi.arr_u64(strideF), _ptr(X), opX, strideX,
                   _ptr(Z), strideZ, sc(alpha), sc(beta), batch, _ptr(Y), strideY, _ptr(temp1), _ptr(temp2))
 
+    def prepared(self, call, *args, **kwargs):
+        """Marshal the arguments of one raw call once and return a zero-argument callable that repeats
+        it (what a C caller does when it calls the same problem in a loop).  `call` is the name of one
+        of the x* methods above, e.g. "xgemkm"."""
+        captured = {}
+        real = self.lib
+
+        class _Capture:
+            def __getattr__(_, name):
+                def grab(*a):
+                    captured["fn"], captured["args"] = getattr(real, name), a
+                    return SUCCESS
+                return grab
+
+        self.lib = _Capture()
+        try:
+            getattr(self, call)(*args, **kwargs)
+        finally:
+            self.lib = real
+        fn, a = captured["fn"], captured["args"]
+        return lambda: fn(*a)
+
     def xforward(self, mmtype, M, Ps, Qs, X, Fs, Z, inters, opX=OP_N, opFs=OP_N, backend=BACKEND_HIP):
         pre, _ = self._prefix(X.dtype)
         ip = capi.arr_ptr([t.data_ptr() for t in inters]) if inters else None

@@ -31,7 +31,7 @@ template <> struct KmmRegCfg<8, 2> { static constexpr int G = 64; };
 constexpr int kKmmWaves = 4;
 
 template <int P, int NF, bool HAS_Y>
-__global__ __launch_bounds__(256, 4) void kron_kmm_reg_kernel(const StepArgs a, const uint32_t mTiles,
+__global__ __launch_bounds__(256, HAS_Y ? 3 : 4) void kron_kmm_reg_kernel(const StepArgs a, const uint32_t mTiles,
                                                               const uint32_t totalTiles) {
   constexpr int G = KmmRegCfg<P, NF>::G;
   constexpr int QQ = P / 4;

@@ -59,9 +59,9 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a,
     const uint32_t wg = blockIdx.x + blockIdx.y * gridDim.x;
     const uint32_t g = (wg >> 3) % groups;   // workgroups go round-robin over the 8 XCDs: keep every group on every XCD
     if (wg < firstWave && g != 0) {
-      const uint64_t t0 = __builtin_readcyclecounter();
-      const uint64_t wait = (uint64_t)g * delayCycles;
-      while (__builtin_readcyclecounter() - t0 < wait) __builtin_amdgcn_s_sleep(16);
+      // pure s_sleep (64 cycles per unit): polling a clock from thousands of waves would itself load the memory path
+      const uint32_t n = (g * delayCycles) >> 12;                 // units of 64*64 cycles
+      for (uint32_t k = 0; k < n; k++) __builtin_amdgcn_s_sleep(64);
     }
   }
   const int l = tid & 63;
@@ -114,6 +114,10 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a,
     for (int r = 0; r < 4; r++) e = MFMA16(d[r], FB[r], e);
 #pragma unroll
     for (int r = 0; r < 4; r++) x[t][r] = e[r];       // = Y[k1=w][k2=t][q3=4kb+r][q4=i]
+    // half 0 of exchange 1 goes out as soon as it exists, under the products of the next blocks
+#pragma unroll
+    for (int rr = 0; rr < 2; rr++)
+      lds[((kb * 2 + rr) * 16 + i) * 256 + ((w * 16 + t) ^ l)] = e[rr];
   }
 
   FK_STAMP(1);
@@ -121,14 +125,16 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a,
   float z[16][4];
 #pragma unroll
   for (int h = 0; h < 2; h++) {
-    if (h) __syncthreads();
+    if (h) {
+      __syncthreads();
 #pragma unroll
-    for (int t = 0; t < 16; t++)
+      for (int t = 0; t < 16; t++)
 #pragma unroll
-      for (int rr = 0; rr < 2; rr++) {
-        const int row = (kb * 2 + rr) * 16 + i;
-        lds[row * 256 + ((w * 16 + t) ^ l)] = x[t][2 * h + rr];
-      }
+        for (int rr = 0; rr < 2; rr++) {
+          const int row = (kb * 2 + rr) * 16 + i;
+          lds[row * 256 + ((w * 16 + t) ^ l)] = x[t][2 + rr];
+        }
+    }
     __syncthreads();
 #pragma unroll
     for (int u = 0; u < 16; u++) {
@@ -153,6 +159,10 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a,
     for (int r = 0; r < 4; r++) e = MFMA16(d[r], FD[r], e);
 #pragma unroll
     for (int r = 0; r < 4; r++) z[u][r] = e[r];       // = Z[q1=4kb+r][q2=i][q3=u][q4=w]
+    // half 0 of exchange 2 (every wave passed the barrier after its last read of exchange 1)
+#pragma unroll
+    for (int rr = 0; rr < 2; rr++)
+      lds[((kb * 2 + rr) * 16 + i) * 256 + ((u * 16 + w) ^ (i * 4) ^ kb)] = e[rr];
   }
 
   FK_STAMP(3);
@@ -161,14 +171,16 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a,
   f4 o[16];
 #pragma unroll
   for (int h = 0; h < 2; h++) {
-    if (h) __syncthreads();
+    if (h) {
+      __syncthreads();
 #pragma unroll
-    for (int u = 0; u < 16; u++)
+      for (int u = 0; u < 16; u++)
 #pragma unroll
-      for (int rr = 0; rr < 2; rr++) {
-        const int row = (kb * 2 + rr) * 16 + i;
-        lds[row * 256 + ((u * 16 + w) ^ (i * 4) ^ kb)] = z[u][2 * h + rr];
-      }
+        for (int rr = 0; rr < 2; rr++) {
+          const int row = (kb * 2 + rr) * 16 + i;
+          lds[row * 256 + ((u * 16 + w) ^ (i * 4) ^ kb)] = z[u][2 + rr];
+        }
+    }
     __syncthreads();
 #pragma unroll
     for (int q1hi = 0; q1hi < 4; q1hi++)
@@ -231,7 +243,7 @@ hipError_t launchRow16x4(const StepArgs& a, hipStream_t stream) {
   }
   dim3 grid(a.M, a.batch), block(1024);
   static int cus = 0;
-  static uint32_t groups = 2, delay = 1100;            // delay in s_memtime ticks (100 MHz): 11 us
+  static uint32_t groups = 3, delay = 20000;           // three start groups, 20000 cycles (about 9 us) apart
   if (!cus) {
     int dev = 0;
     hipDeviceProp_t prop;

@@ -219,3 +219,82 @@ def test_kmm_register_kernel(fk, M, Ps):
     check(fk, ko.KMM, M, Ps, Ps, np.float32, alpha=1.0, beta=0.0, seed=52, opFs=ko.OP_T)
     check(fk, ko.KMM, M, Ps, Ps, np.float32, alpha=1.0, beta=1.0, seed=53, batch=2)
     check(fk, ko.KMM, M, Ps, Ps, np.float32, alpha=2.0, beta=1.0, seed=54, use_temp2=False)
+
+
+def test_misaligned_buffers_fall_back_to_the_generic_plan(fk):
+    """The 16x16^4 row kernel stores 128-bit vectors; a Z that is only 4-byte aligned must still give the
+    right answer (the library re-plans with one generic launch per factor)."""
+    import torch
+    M, Ps = 2, [16] * 4
+    K = 65536
+    X, Fs, _ = make_case(ko.MKM, M, Ps, Ps, np.float32, seed=61, with_y=False)
+    want = oracle_answer(ko.MKM, M, Ps, Ps, X, Fs, None, 1.0, 0.0)
+    dev = "cuda:0"
+    tX = torch.from_numpy(X).to(dev)
+    tFs = [torch.from_numpy(f).to(dev) for f in Fs]
+    Zbuf = torch.full((M * K + 1,), float("nan"), dtype=torch.float32, device=dev)
+    Z = Zbuf[1:]                                       # data_ptr() is 4 bytes past a 256-byte boundary
+    t1 = torch.empty(M * K, dtype=torch.float32, device=dev)
+    t2 = torch.empty(M * K, dtype=torch.float32, device=dev)
+    e = fk.xgemkm(M, Ps, Ps, tX, tFs, Z, 1.0, 0.0, None, t1, t2)
+    torch.cuda.synchronize()
+    assert e == 0
+    assert len(fk.last_plan()) == 4 and all("generic" in k for _, _, k in fk.last_plan())
+    assert normwise(Z.cpu().numpy(), want) <= 1e-5
+
+
+@pytest.mark.parametrize("mm,name", [(ko.MKM, "mkm"), (ko.KMM, "kmm")])
+def test_forward_strided_batched(fk, mm, name):
+    import ctypes
+    import torch
+    from fastkron_amd import capi
+    M, Ps, Qs, B = 5, [4, 3, 8], [2, 5, 8], 3
+    K, L = int(np.prod(Ps)), int(np.prod(Qs))
+    X, Fs, _ = make_case(mm, M, Ps, Qs, np.float64, seed=71, with_y=False, batch=B)
+    Zw, Iw = oracle_answer(mm, M, Ps, Qs, X, Fs, None, 1.0, 0.0, batch=B, keep_intermediates=True)
+    ye, sizes = fk.sizes_forward(M, Ps, Qs)
+    dev = "cuda:0"
+    tX = torch.from_numpy(X).to(dev)
+    tFs = [torch.from_numpy(f).to(dev) for f in Fs]
+    Z = torch.full((B * ye,), float("nan"), dtype=torch.float64, device=dev)
+    inters = [torch.full((B * s,), float("nan"), dtype=torch.float64, device=dev) for s in sizes]
+    lib = fk.lib
+    fp = capi.arr_ptr([f.data_ptr() for f in tFs])
+    ip = capi.arr_ptr([t.data_ptr() for t in inters])
+    sF = capi.arr_u64([p * q for p, q in zip(Ps, Qs)])
+    if mm == ko.MKM:
+        e = lib.dmkmForwardStridedBatched(fk.h, capi.BACKEND_HIP, M, len(Ps), capi.arr_u32(Ps), capi.arr_u32(Qs),
+                                          ctypes.c_void_p(tX.data_ptr()), capi.OP_N, M * K, fp, capi.OP_N, sF,
+                                          ctypes.c_void_p(Z.data_ptr()), M * L, B, ip, None)
+    else:
+        e = lib.dkmmForwardStridedBatched(fk.h, capi.BACKEND_HIP, len(Ps), capi.arr_u32(Qs), capi.arr_u32(Ps), M,
+                                          fp, capi.OP_N, sF, ctypes.c_void_p(tX.data_ptr()), capi.OP_N, M * K,
+                                          ctypes.c_void_p(Z.data_ptr()), M * L, B, ip, None)
+    torch.cuda.synchronize()
+    assert e == 0
+    assert normwise(Z.cpu().numpy(), Zw) <= 1e-12
+    for got, want in zip(inters, Iw):
+        assert normwise(got.cpu().numpy(), want) <= 1e-12
+
+
+def test_tuned_plans_persist_to_a_file(tmp_path):
+    """fastKronOptionsTune times the candidate plans once, writes the winner to the tuning file, and a
+    new handle pointed at that file uses it without tuning."""
+    import fastkron_amd
+    db = str(tmp_path / "tuned.db")
+    h = fastkron_amd.FastKron(tune=True)
+    h.set_tuned_db(db)
+    try:
+        check(h, ko.MKM, 16, [8] * 3, [8] * 3, np.float32, alpha=1.0, beta=0.0, seed=81)
+        plan = h.last_plan()
+    finally:
+        h.close()
+    text = open(db).read()
+    assert "16x512*(8x8^3)_NN_f" in text
+    h2 = fastkron_amd.FastKron(tune=False)
+    h2.set_tuned_db(db)
+    try:
+        check(h2, ko.MKM, 16, [8] * 3, [8] * 3, np.float32, alpha=1.0, beta=0.0, seed=82)
+        assert h2.last_plan() == plan
+    finally:
+        h2.close()
