@@ -43,9 +43,12 @@ void registerGenericKernels(std::vector<KernelInfo>& out) {
 // ---- whole-row kernel for four fused 16x16 fp32 factors ----
 static bool row16CanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
                         const DeviceInfo& dev) {
-  if (p.dt != DType::F32 || p.mm != MMType::MKM || hi - lo + 1 != 4 || p.forward) return false;
-  for (uint32_t i = lo; i <= hi; i++) if (p.P[i] != 16 || p.Q[i] != 16) return false;
-  if (p.colsBefore(hi) != 65536) return false;
+  const uint32_t nf = hi - lo + 1;
+  if (p.dt != DType::F32 || p.mm != MMType::MKM || nf < 2 || nf > 4 || p.forward) return false;
+  uint64_t kk = 1, rows = 1;
+  for (uint32_t i = lo; i <= hi; i++) { if (p.P[i] != 16 || p.Q[i] != 16) return false; kk *= 16; }
+  for (uint32_t i = nf; i < 4; i++) rows *= 16;
+  if (p.colsBefore(hi) != kk || p.M % rows) return false;   // the group covers whole rows, M a whole number of blocks
   if (first && p.opX == 2) return false;
   return dev.ldsPerBlock >= 131072 && k.dt == p.dt;
 }
@@ -55,9 +58,12 @@ static bool row16Check(const KernelInfo&, const StepArgs& a) { return row16x4Sup
 // ---- whole-row kernel for five fused 8x8 fp32 factors ----
 static bool row8CanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
                        const DeviceInfo& dev) {
-  if (p.dt != DType::F32 || p.mm != MMType::MKM || hi - lo + 1 != 5 || p.forward) return false;
-  for (uint32_t i = lo; i <= hi; i++) if (p.P[i] != 8 || p.Q[i] != 8) return false;
-  if (p.colsBefore(hi) != 32768) return false;
+  const uint32_t nf = hi - lo + 1;
+  if (p.dt != DType::F32 || p.mm != MMType::MKM || nf < 2 || nf > 5 || p.forward) return false;
+  uint64_t kk = 1, rows = 1;
+  for (uint32_t i = lo; i <= hi; i++) { if (p.P[i] != 8 || p.Q[i] != 8) return false; kk *= 8; }
+  for (uint32_t i = nf; i < 5; i++) rows *= 8;
+  if (p.colsBefore(hi) != kk || p.M % rows) return false;
   if (first && p.opX == 2) return false;
   return dev.ldsPerBlock >= 67000 && k.dt == p.dt;
 }

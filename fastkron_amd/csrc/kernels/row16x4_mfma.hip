@@ -73,23 +73,27 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a,
   if (tid == 0 && blockIdx.x < 1024) g_rowTiming[blockIdx.x * 8 + 6] = wall_clock64();
 #endif
 
-  const float* X = (const float*)a.in + (size_t)b * a.in_batch + (size_t)m * a.in_ldm;
-  float* Z = (float*)a.out + (size_t)b * a.out_batch + (size_t)m * a.out_ldm;
+  // m counts blocks of 65536 contiguous elements: one row for four factors, 16^(4-nf) rows otherwise
+  const float* X = (const float*)a.in + (size_t)b * a.in_batch + (size_t)m * kRowLen;
+  float* Z = (float*)a.out + (size_t)b * a.out_batch + (size_t)m * kRowLen;
 
   // Factor operands (B side of every product).  a.f[0] is the last factor (F4) ... a.f[3] the first (F1).
   // First product of a chain: B_c[k][j] = F[4c + k][j]; second product: B_r[k][j] = F[4k + r][j].
+  // With fewer than four factors the leading digits are row indices (16^(4-nf) consecutive rows form the
+  // same contiguous 65536-element block) and their factor slots hold the identity.
   float FA[4], FB[4], FC[4], FD[4];
   {
-    const float* F4p = (const float*)a.f[0] + (size_t)b * a.f_batch[0];
-    const float* F3p = (const float*)a.f[1] + (size_t)b * a.f_batch[1];
-    const float* F2p = (const float*)a.f[2] + (size_t)b * a.f_batch[2];
-    const float* F1p = (const float*)a.f[3] + (size_t)b * a.f_batch[3];
+    auto fetch = [&](int j, int p, int q) -> float {
+      if (j >= (int)a.nf) return (p == q) ? 1.f : 0.f;
+      const float* f = (const float*)a.f[j] + (size_t)b * a.f_batch[j];
+      return f[(int64_t)p * a.f_sp[j] + (int64_t)q * a.f_sq[j]];
+    };
 #pragma unroll
     for (int c = 0; c < 4; c++) {
-      FA[c] = F3p[(int64_t)(4 * c + kb) * a.f_sp[1] + (int64_t)i * a.f_sq[1]];
-      FB[c] = F4p[(int64_t)(4 * kb + c) * a.f_sp[0] + (int64_t)i * a.f_sq[0]];
-      FC[c] = F1p[(int64_t)(4 * c + kb) * a.f_sp[3] + (int64_t)i * a.f_sq[3]];
-      FD[c] = F2p[(int64_t)(4 * kb + c) * a.f_sp[2] + (int64_t)i * a.f_sq[2]];
+      FA[c] = fetch(1, 4 * c + kb, i);      // F3: first product of stage 1
+      FB[c] = fetch(0, 4 * kb + c, i);      // F4: second product of stage 1
+      FC[c] = fetch(3, 4 * c + kb, i);      // F1: first product of stage 2
+      FD[c] = fetch(2, 4 * kb + c, i);      // F2: second product of stage 2
     }
   }
 
@@ -197,7 +201,7 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a,
   FK_STAMP(4);
   // ---- epilogue and store: every wave-level store covers 1 KB of contiguous columns ----
   const float alpha = (float)a.alpha, beta = (float)a.beta;
-  const float* Y = HAS_Y ? (const float*)a.y + (size_t)b * a.y_batch + (size_t)m * a.y_ldm : nullptr;
+  const float* Y = HAS_Y ? (const float*)a.y + (size_t)b * a.y_batch + (size_t)m * kRowLen : nullptr;
 #pragma unroll
   for (int q1 = 0; q1 < 16; q1++) {
     const int col = q1 * 4096 + w * 256 + l * 4;
@@ -217,14 +221,21 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a,
 #endif
 }
 
+// Rows per workgroup: 16^(4-nf).
+static uint32_t row16Rows(const StepArgs& a) { uint32_t r = 1; for (uint32_t j = a.nf; j < 4; j++) r *= 16; return r; }
+
 bool row16x4Supported(const StepArgs& a) {
-  if (a.nf != 4 || a.Kin != (uint64_t)kRowLen || a.Kout != (uint64_t)kRowLen) return false;
-  for (int j = 0; j < 4; j++) if (a.p[j] != 16 || a.q[j] != 16) return false;
-  if (a.in_ldc != 1 || a.out_ldc != 1) return false;
-  if (a.y && a.y_ldc != 1) return false;
-  // 16-byte aligned rows for the vector stores / Y loads
-  if (((uintptr_t)a.out & 15) || (a.out_ldm & 3) || (a.out_batch & 3)) return false;
-  if (a.y && (((uintptr_t)a.y & 15) || (a.y_ldm & 3) || (a.y_batch & 3))) return false;
+  if (a.nf < 2 || a.nf > 4) return false;
+  uint64_t k = 1;
+  for (uint32_t j = 0; j < a.nf; j++) { if (a.p[j] != 16 || a.q[j] != 16) return false; k *= 16; }
+  if (a.Kin != k || a.Kout != k) return false;
+  if (a.in_ldc != 1 || a.out_ldc != 1 || (a.y && a.y_ldc != 1)) return false;
+  // the rows of a block must be contiguous, and M must be a whole number of blocks
+  if ((uint64_t)a.in_ldm != k || (uint64_t)a.out_ldm != k || (a.y && (uint64_t)a.y_ldm != k)) return false;
+  if (a.M % row16Rows(a)) return false;
+  // 16-byte aligned blocks for the vector stores / Y loads
+  if (((uintptr_t)a.out & 15) || (a.out_batch & 3)) return false;
+  if (a.y && (((uintptr_t)a.y & 15) || (a.y_batch & 3))) return false;
   return a.batch <= 65535;
 }
 
@@ -241,7 +252,7 @@ hipError_t launchRow16x4(const StepArgs& a, hipStream_t stream) {
     if (e != hipSuccess) return e;
     attrSet = true;
   }
-  dim3 grid(a.M, a.batch), block(1024);
+  dim3 grid(a.M / row16Rows(a), a.batch), block(1024);
   static int cus = 0;
   static uint32_t groups = 3, delay = 20000;           // three start groups, 20000 cycles (about 9 us) apart
   if (!cus) {
@@ -255,7 +266,7 @@ hipError_t launchRow16x4(const StepArgs& a, hipStream_t stream) {
     }
   }
   const uint32_t firstWave = (uint32_t)cus;
-  const uint32_t g = ((uint64_t)a.M * a.batch > (uint64_t)cus) ? groups : 1;   // a single wave of rows gains nothing
+  const uint32_t g = ((uint64_t)grid.x * a.batch > (uint64_t)cus) ? groups : 1;   // a single wave of rows gains nothing
   if (a.y && a.epilogue)
     hipLaunchKernelGGL(kron_row16x4_kernel<true>, grid, block, ldsBytes, stream, a, firstWave, g, delay);
   else

@@ -92,8 +92,9 @@ __global__ __launch_bounds__(512, 4) void kron_row8x5_kernel(const StepArgs a) {
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);      // wave-uniform: keeps row addresses in SGPRs
   const uint32_t m = blockIdx.x, bt = blockIdx.y;
 
-  const float* X = (const float*)a.in + (size_t)bt * a.in_batch + (size_t)m * a.in_ldm;
-  float* Z = (float*)a.out + (size_t)bt * a.out_batch + (size_t)m * a.out_ldm;
+  // m counts blocks of 32768 contiguous elements: one row for five factors, 8^(5-nf) rows otherwise
+  const float* X = (const float*)a.in + (size_t)bt * a.in_batch + (size_t)m * kRow8Len;
+  float* Z = (float*)a.out + (size_t)bt * a.out_batch + (size_t)m * kRow8Len;
 
   FK8_STAMP(0); FK8_STAMP(6);
   // ---- load: x[k1][k2] = X[k1][k2][k3 = w][(k4,k5) = l] ----
@@ -105,12 +106,18 @@ __global__ __launch_bounds__(512, 4) void kron_row8x5_kernel(const StepArgs a) {
 #pragma unroll
       for (int j = 0; j < 8; j++) x[i][j] = xp[i * 4096 + j * 512];
   }
-  // factors to LDS (a.f[0] is the last factor F5 ... a.f[4] the first, F1)
+  // factors to LDS (a.f[0] is the last factor F5 ... a.f[nf-1] the first).  With fewer than five
+  // factors the leading digits are row indices (8^(5-nf) consecutive rows form the same contiguous
+  // 32768-element block) and their factor slots hold the identity.
   if (tid < 320) {
     const int f = tid >> 6, e = tid & 63, p = e >> 3, q = e & 7;
     const int j = 4 - f;
-    const float* fp = (const float*)a.f[j] + (size_t)bt * a.f_batch[j];
-    fl[tid] = fp[(int64_t)p * a.f_sp[j] + (int64_t)q * a.f_sq[j]];
+    float v = (p == q) ? 1.f : 0.f;
+    if (j < (int)a.nf) {
+      const float* fp = (const float*)a.f[j] + (size_t)bt * a.f_batch[j];
+      v = fp[(int64_t)p * a.f_sp[j] + (int64_t)q * a.f_sq[j]];
+    }
+    fl[tid] = v;
   }
   __syncthreads();
 
@@ -196,7 +203,7 @@ __global__ __launch_bounds__(512, 4) void kron_row8x5_kernel(const StepArgs a) {
 
   // ---- epilogue and store ----
   const float alpha = (float)a.alpha, beta = (float)a.beta;
-  const float* Y = HAS_Y ? (const float*)a.y + (size_t)bt * a.y_batch + (size_t)m * a.y_ldm : nullptr;
+  const float* Y = HAS_Y ? (const float*)a.y + (size_t)bt * a.y_batch + (size_t)m * kRow8Len : nullptr;
   const int lo = (l & 31), q2b = l >> 5;
 #pragma unroll
   for (int q3 = 0; q3 < 8; q3++)
@@ -214,11 +221,18 @@ __global__ __launch_bounds__(512, 4) void kron_row8x5_kernel(const StepArgs a) {
   FK8_STAMP(5); FK8_STAMP(7);
 }
 
+// Rows per workgroup: 8^(5-nf).
+static uint32_t row8Rows(const StepArgs& a) { uint32_t r = 1; for (uint32_t j = a.nf; j < 5; j++) r *= 8; return r; }
+
 bool row8x5Supported(const StepArgs& a) {
-  if (a.nf != 5 || a.Kin != (uint64_t)kRow8Len || a.Kout != (uint64_t)kRow8Len) return false;
-  for (int j = 0; j < 5; j++) if (a.p[j] != 8 || a.q[j] != 8) return false;
-  if (a.in_ldc != 1 || a.out_ldc != 1) return false;
-  if (a.y && a.y_ldc != 1) return false;
+  if (a.nf < 2 || a.nf > 5) return false;
+  uint64_t k = 1;
+  for (uint32_t j = 0; j < a.nf; j++) { if (a.p[j] != 8 || a.q[j] != 8) return false; k *= 8; }
+  if (a.Kin != k || a.Kout != k) return false;
+  if (a.in_ldc != 1 || a.out_ldc != 1 || (a.y && a.y_ldc != 1)) return false;
+  // the rows of a block must be contiguous, and M must be a whole number of blocks
+  if ((uint64_t)a.in_ldm != k || (uint64_t)a.out_ldm != k || (a.y && (uint64_t)a.y_ldm != k)) return false;
+  if (a.M % row8Rows(a)) return false;
   return a.batch <= 65535;
 }
 
@@ -235,7 +249,7 @@ hipError_t launchRow8x5(const StepArgs& a, hipStream_t stream) {
     if (e != hipSuccess) return e;
     attrSet = true;
   }
-  dim3 grid(a.M, a.batch), block(512);
+  dim3 grid(a.M / row8Rows(a), a.batch), block(512);
   if (a.y && a.epilogue)
     hipLaunchKernelGGL(kron_row8x5_kernel<true>, grid, block, ldsBytes, stream, a);
   else

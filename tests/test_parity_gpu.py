@@ -298,3 +298,20 @@ def test_tuned_plans_persist_to_a_file(tmp_path):
         assert h2.last_plan() == plan
     finally:
         h2.close()
+
+
+@pytest.mark.parametrize("M,Ps,tag", [(8, [8] * 4, "1x32768"), (128, [8] * 3, "1x32768"), (1024, [8] * 2, "1x32768"),
+                                      (16, [16] * 3, "1x65536"), (512, [16] * 2, "1x65536"), (32, [16] * 3, "1x65536")])
+def test_row_kernels_with_fewer_factors(fk, M, Ps, tag):
+    """Shorter chains of 8x8 / 16x16 factors reuse the whole-row kernels: 8^(5-N) (16^(4-N)) consecutive rows
+    form one contiguous block and the missing leading factors are identities."""
+    check(fk, ko.MKM, M, Ps, Ps, np.float32, alpha=1.5, beta=0.5, seed=91)
+    plan = fk.last_plan()
+    assert len(plan) == 1 and tag in plan[0][2], plan
+    check(fk, ko.MKM, M, Ps, Ps, np.float32, alpha=1.0, beta=0.0, seed=92, batch=2)
+
+
+def test_row_kernels_need_whole_blocks(fk):
+    """A row count that is not a whole number of blocks takes the generic kernels instead."""
+    check(fk, ko.MKM, 12, [8] * 4, [8] * 4, np.float32, alpha=1.0, beta=0.0, seed=93)
+    assert all("generic" in k for _, _, k in fk.last_plan())
