@@ -82,17 +82,17 @@ static bool row32CanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, 
 static hipError_t row32Launch(const KernelInfo&, const StepArgs& a, hipStream_t s) { return launchRow32x16x3(a, s); }
 static bool row32Check(const KernelInfo&, const StepArgs& a) { return row32x16x3Supported(a); }
 
-// ---- fp64 single-factor MFMA step ----
+// ---- single-factor MFMA step (fp64 and fp32) ----
 static bool stepF64CanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
                           const DeviceInfo& dev) {
-  if (p.dt != DType::F64 || p.mm != MMType::MKM || lo != hi) return false;
+  if (p.dt != k.dt || p.mm != MMType::MKM || lo != hi) return false;
   if (p.P[lo] != k.P || p.Q[lo] != k.Q) return false;
   if (first && p.opX == 2) return false;
   (void)dev;
   return true;
 }
-static hipError_t stepF64Launch(const KernelInfo&, const StepArgs& a, hipStream_t s) { return launchStepMfmaF64(a, s); }
-static bool stepF64Check(const KernelInfo&, const StepArgs& a) { return stepMfmaF64Supported(a); }
+static hipError_t stepF64Launch(const KernelInfo& k, const StepArgs& a, hipStream_t s) { return launchStepMfma(a, k.dt, s); }
+static bool stepF64Check(const KernelInfo& k, const StepArgs& a) { return stepMfmaSupported(a, k.dt); }
 
 // ---- KMM-layout register kernel: NF fused PxP fp32 factors with P^NF = 64 ----
 static bool kmmRegCanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
@@ -136,12 +136,13 @@ void registerRowKernels(std::vector<KernelInfo>& out) {
     out.push_back(kk);
   }
 
+  for (DType dt : {DType::F64, DType::F32})
   for (uint32_t P : {16u, 32u, 64u}) {
     KernelInfo kd{};
     const std::string ps = std::to_string(P);
-    kd.name = "mkm_hip_gfx950_256_d_" + ps + "x" + ps + "_" + ps + "x" + ps + "_1_1x" + std::to_string(16 * P) +
+    kd.name = std::string("mkm_hip_gfx950_256_") + (dt == DType::F64 ? "d_" : "f_") + ps + "x" + ps + "_" + ps + "x" + ps + "_1_1x" + std::to_string(16 * P) +
               "_mfma16x16x4_NN_strided_0_3";
-    kd.dt = DType::F64; kd.P = P; kd.Q = P; kd.fused = 1; kd.tileM = 1; kd.tileK = 16 * P; kd.threads = 256; kd.variant = 0;
+    kd.dt = dt; kd.P = P; kd.Q = P; kd.fused = 1; kd.tileM = 1; kd.tileK = 16 * P; kd.threads = 256; kd.variant = 0;
     kd.canRun = stepF64CanRun; kd.launch = stepF64Launch; kd.check = stepF64Check;
     out.push_back(kd);
   }

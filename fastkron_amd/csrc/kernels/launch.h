@@ -20,9 +20,9 @@ hipError_t launchRow8x5(const StepArgs& a, hipStream_t stream);
 bool row32x16x3Supported(const StepArgs& a);
 hipError_t launchRow32x16x3(const StepArgs& a, hipStream_t stream);
 
-// One fp64 step with a 16x16 / 32x32 / 64x64 factor on the fp64 matrix cores (MKM layout).
-bool stepMfmaF64Supported(const StepArgs& a);
-hipError_t launchStepMfmaF64(const StepArgs& a, hipStream_t stream);
+// One step with a 16x16 / 32x32 / 64x64 factor on the matrix cores, fp64 or fp32 (MKM layout).
+bool stepMfmaSupported(const StepArgs& a, DType dt);
+hipError_t launchStepMfma(const StepArgs& a, DType dt, hipStream_t stream);
 
 // KMM layout, fp32: three fused 4x4 or two fused 8x8 factors held in registers, lanes along M.
 bool kmmRegSupported(const StepArgs& a);

@@ -1,5 +1,5 @@
-// One sliced-multiply step with a square fp64 factor (P = Q in {16, 32, 64}), MKM layout, on the
-// fp64 matrix cores (V_MFMA_F64_16X16X4_F64).  Used per factor for shapes like dgemkm 256 x 262144
+// One sliced-multiply step with a square factor (P = Q in {16, 32, 64}), MKM layout, fp64 or fp32, on the
+// matrix cores (V_MFMA_F64_16X16X4_F64 / V_MFMA_F32_16X16X4_F32).  Used per factor for shapes like dgemkm 256 x 262144
 // with 64x64^3, where every step is a real (M*Kin/P) x P x Q contraction.
 //
 //   out[m, q*S + s] = sum_p in[m, s*P + p] * F[p, q],   S = Kin / P
@@ -12,8 +12,9 @@
 //   * A operand (lane = 16*k + q): F[(P/4)*k + c][16*ib + q]; the whole factor sits in registers
 //     (128 VGPRs for 64x64) for the life of the persistent wave, so the loop reads nothing but X;
 //   * the next tile's loads are issued before the current tile's products (register double buffer);
-//   * accumulator layout (register q/4, lane 16*(q%4) + slice): each quarter wave stores 16
-//     consecutive doubles (one 128-byte line) straight into the shuffled layout out[q*S + s].
+//   * accumulator layout (fp64: register q/4, lane 16*(q%4) + slice; fp32: register q%4, lane
+//     16*(q/4) + slice): each quarter wave stores 16 consecutive elements (a 128-byte line in fp64)
+//     straight into the shuffled layout out[q*S + s].
 // alpha / beta*Y are applied in the same store when this is the launch that writes Z.
 //
 // Role of the reference's CUDA kernel for large factors (reference src/kernels/cuda/kernel.cuh:53-224,
@@ -27,16 +28,36 @@
 namespace fk {
 
 typedef double d4 __attribute__((ext_vector_type(4)));
+typedef float f4 __attribute__((ext_vector_type(4)));
 
-#define MFMA16D(a, b, c) __builtin_amdgcn_mfma_f64_16x16x4f64((a), (b), (c), 0, 0, 0)
+template <typename T> struct Mfma16;
+template <> struct Mfma16<double> {
+  using Acc = d4;
+  static __device__ __forceinline__ Acc mma(double a, double b, Acc c) {
+    return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0);
+  }
+  // row index (0..15) of accumulator register r in the lane group hi = lane >> 4
+  static __device__ __forceinline__ int row(int r, int hi) { return 4 * r + hi; }
+};
+template <> struct Mfma16<float> {
+  using Acc = f4;
+  static __device__ __forceinline__ Acc mma(float a, float b, Acc c) {
+    return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ int row(int r, int hi) { return 4 * hi + r; }
+};
 
-constexpr int kF64Waves = 4;             // waves per workgroup
+constexpr int kStepWaves = 4;            // waves per workgroup
 
-template <int P, int Q, bool HAS_Y>
-__global__ __launch_bounds__(256, 2) void kron_step_mfma_f64_kernel(const StepArgs a, const uint32_t tilesPerRow,
-                                                                    const uint32_t totalTiles) {
-  constexpr int PC = P / 4;              // products per tile and doubles per lane
+template <typename T, int P, int Q, bool HAS_Y>
+__global__ __launch_bounds__(256, 2) void kron_step_mfma_kernel(const StepArgs a, const uint32_t tilesPerRow,
+                                                                const uint32_t totalTiles) {
+  using M16 = Mfma16<T>;
+  using Acc = typename M16::Acc;
+  constexpr int PC = P / 4;              // products per tile and elements per lane
   constexpr int NB = Q / 16;
+  constexpr int VE = 16 / sizeof(T);     // elements per 128-bit load
+  typedef T VT __attribute__((ext_vector_type(VE)));
   const int tid = threadIdx.x;
   const int l = tid & 63;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);      // wave-uniform: keeps row addresses in SGPRs
@@ -44,69 +65,70 @@ __global__ __launch_bounds__(256, 2) void kron_step_mfma_f64_kernel(const StepAr
   const uint32_t bt = blockIdx.y;
   const uint64_t S = a.Kin / P;
 
-  const double* inB = (const double*)a.in + (size_t)bt * a.in_batch;
-  double* outB = (double*)a.out + (size_t)bt * a.out_batch;
-  const double* F = (const double*)a.f[0] + (size_t)bt * a.f_batch[0];
-  const double* YB = HAS_Y ? (const double*)a.y + (size_t)bt * a.y_batch : nullptr;
+  const T* inB = (const T*)a.in + (size_t)bt * a.in_batch;
+  T* outB = (T*)a.out + (size_t)bt * a.out_batch;
+  const T* F = (const T*)a.f[0] + (size_t)bt * a.f_batch[0];
+  const T* YB = HAS_Y ? (const T*)a.y + (size_t)bt * a.y_batch : nullptr;
 
   // the whole factor as A operands, resident in registers: fa[c][ib] = F[PC*hi + c][16*ib + lo]
-  double fa[PC][NB];
+  T fa[PC][NB];
 #pragma unroll
   for (int c = 0; c < PC; c++)
 #pragma unroll
     for (int ib = 0; ib < NB; ib++)
       fa[c][ib] = F[(int64_t)(PC * hi + c) * a.f_sp[0] + (int64_t)(16 * ib + lo) * a.f_sq[0]];
 
-  const double alpha = a.alpha, beta = a.beta;
-  const uint32_t waveId = blockIdx.x * kF64Waves + w, nWaves = gridDim.x * kF64Waves;
+  const T alpha = (T)a.alpha, beta = (T)a.beta;
+  const uint32_t waveId = blockIdx.x * kStepWaves + w, nWaves = gridDim.x * kStepWaves;
 
-  auto loadTile = [&](uint32_t t, double (&x)[PC]) {
+  auto loadTile = [&](uint32_t t, T (&x)[PC]) {
     const uint32_t m = t / tilesPerRow;
     const uint64_t s0 = (uint64_t)(t % tilesPerRow) * 16;
     const uint64_t s = (s0 + lo < S) ? s0 + lo : s0;
-    const double* xp = inB + (size_t)m * a.in_ldm + s * P + PC * hi;
+    const T* xp = inB + (size_t)m * a.in_ldm + s * P + PC * hi;
 #pragma unroll
-    for (int c = 0; c < PC; c += 2) {
-      const double2 v = *(const double2*)(xp + c);
-      x[c] = v.x; x[c + 1] = v.y;
+    for (int c = 0; c < PC; c += VE) {
+      const VT v = *(const VT*)(xp + c);
+#pragma unroll
+      for (int e = 0; e < VE; e++) x[c + e] = v[e];
     }
   };
 
-  double xn[PC];
+  T xn[PC];
   if (waveId < totalTiles) loadTile(waveId, xn);
   for (uint32_t t = waveId; t < totalTiles; t += nWaves) {
-    double x[PC];
+    T x[PC];
 #pragma unroll
     for (int c = 0; c < PC; c++) x[c] = xn[c];
     if (t + nWaves < totalTiles) loadTile(t + nWaves, xn);       // next tile streams in under the products
 
-    d4 acc[NB];
+    Acc acc[NB];
 #pragma unroll
-    for (int ib = 0; ib < NB; ib++) acc[ib] = (d4){0.0, 0.0, 0.0, 0.0};
+    for (int ib = 0; ib < NB; ib++) acc[ib] = (Acc){0, 0, 0, 0};
 #pragma unroll
     for (int c = 0; c < PC; c++)
 #pragma unroll
-      for (int ib = 0; ib < NB; ib++) acc[ib] = MFMA16D(fa[c][ib], x[c], acc[ib]);
+      for (int ib = 0; ib < NB; ib++) acc[ib] = M16::mma(fa[c][ib], x[c], acc[ib]);
 
     const uint32_t m = t / tilesPerRow;
     const uint64_t s = (uint64_t)(t % tilesPerRow) * 16 + lo;
     if (s >= S) continue;
-    double* out = outB + (size_t)m * a.out_ldm;
-    const double* Y = HAS_Y ? YB + (size_t)m * a.y_ldm : nullptr;
+    T* out = outB + (size_t)m * a.out_ldm;
+    const T* Y = HAS_Y ? YB + (size_t)m * a.y_ldm : nullptr;
     // all Y loads of the tile before its first store (loads and stores share one in-order counter)
-    double yv[HAS_Y ? NB : 1][4];
+    T yv[HAS_Y ? NB : 1][4];
     if (HAS_Y) {
 #pragma unroll
       for (int ib = 0; ib < NB; ib++)
 #pragma unroll
-        for (int r = 0; r < 4; r++) yv[ib][r] = Y[(uint64_t)(16 * ib + 4 * r + hi) * S + s];
+        for (int r = 0; r < 4; r++) yv[ib][r] = Y[(uint64_t)(16 * ib + M16::row(r, hi)) * S + s];
     }
 #pragma unroll
     for (int ib = 0; ib < NB; ib++)
 #pragma unroll
       for (int r = 0; r < 4; r++) {
-        const uint64_t col = (uint64_t)(16 * ib + 4 * r + hi) * S + s;
-        double v = acc[ib][r];
+        const uint64_t col = (uint64_t)(16 * ib + M16::row(r, hi)) * S + s;
+        T v = acc[ib][r];
         if (a.epilogue) {
           v *= alpha;
           if (HAS_Y) v += beta * yv[ib][r];
@@ -116,25 +138,25 @@ __global__ __launch_bounds__(256, 2) void kron_step_mfma_f64_kernel(const StepAr
   }
 }
 
-bool stepMfmaF64Supported(const StepArgs& a) {
+bool stepMfmaSupported(const StepArgs& a, DType dt) {
   if (a.nf != 1) return false;
   const uint32_t P = a.p[0], Q = a.q[0];
   if (!((P == 64 && Q == 64) || (P == 32 && Q == 32) || (P == 16 && Q == 16))) return false;
   if (a.in_ldc != 1 || a.out_ldc != 1 || (a.y && a.y_ldc != 1)) return false;
   if (a.Kin % P) return false;
   // 16-byte alignment of every slice for the 128-bit loads
-  if (((uintptr_t)a.in & 15) || (a.in_ldm & 1) || (a.in_batch & 1)) return false;
+  const uint64_t vmask = 16 / dtypeSize(dt) - 1;
+  if (((uintptr_t)a.in & 15) || ((uint64_t)a.in_ldm & vmask) || (a.in_batch & vmask)) return false;
   const uint64_t S = a.Kin / P;
   const uint64_t tiles = (S + 15) / 16;
   return tiles * a.M < (1ull << 31) && a.batch <= 65535;
 }
 
-template <int P, int Q>
-static hipError_t launchStepMfmaF64T(const StepArgs& a, hipStream_t stream) {
+template <typename T, int P, int Q>
+static hipError_t launchStepMfmaT(const StepArgs& a, hipStream_t stream) {
   const uint64_t S = a.Kin / P;
   const uint32_t tilesPerRow = (uint32_t)((S + 15) / 16);
   const uint32_t totalTiles = tilesPerRow * a.M;
-  const size_t ldsBytes = 0;
   static int cus = 0;
   if (!cus) {
     int dev = 0;
@@ -144,22 +166,30 @@ static hipError_t launchStepMfmaF64T(const StepArgs& a, hipStream_t stream) {
   }
   // persistent workgroups: 2 per CU (8 waves, 2 per SIMD at up to 256 VGPRs), fewer when there is not enough work
   uint32_t wgs = (uint32_t)cus * 2;
-  const uint32_t need = (totalTiles + kF64Waves - 1) / kF64Waves;
+  const uint32_t need = (totalTiles + kStepWaves - 1) / kStepWaves;
   if (wgs > need) wgs = need;
   dim3 grid(wgs, a.batch), block(256);
   if (a.y && a.epilogue)
-    hipLaunchKernelGGL((kron_step_mfma_f64_kernel<P, Q, true>), grid, block, ldsBytes, stream, a, tilesPerRow, totalTiles);
+    hipLaunchKernelGGL((kron_step_mfma_kernel<T, P, Q, true>), grid, block, 0, stream, a, tilesPerRow, totalTiles);
   else
-    hipLaunchKernelGGL((kron_step_mfma_f64_kernel<P, Q, false>), grid, block, ldsBytes, stream, a, tilesPerRow, totalTiles);
+    hipLaunchKernelGGL((kron_step_mfma_kernel<T, P, Q, false>), grid, block, 0, stream, a, tilesPerRow, totalTiles);
   return hipGetLastError();
 }
 
-hipError_t launchStepMfmaF64(const StepArgs& a, hipStream_t stream) {
-  if (!stepMfmaF64Supported(a)) return hipErrorInvalidValue;
-  switch (a.p[0]) {
-    case 16:  return launchStepMfmaF64T<16, 16>(a, stream);
-    case 32:  return launchStepMfmaF64T<32, 32>(a, stream);
-    case 64:  return launchStepMfmaF64T<64, 64>(a, stream);
+hipError_t launchStepMfma(const StepArgs& a, DType dt, hipStream_t stream) {
+  if (!stepMfmaSupported(a, dt)) return hipErrorInvalidValue;
+  if (dt == DType::F64) {
+    switch (a.p[0]) {
+      case 16: return launchStepMfmaT<double, 16, 16>(a, stream);
+      case 32: return launchStepMfmaT<double, 32, 32>(a, stream);
+      case 64: return launchStepMfmaT<double, 64, 64>(a, stream);
+    }
+  } else {
+    switch (a.p[0]) {
+      case 16: return launchStepMfmaT<float, 16, 16>(a, stream);
+      case 32: return launchStepMfmaT<float, 32, 32>(a, stream);
+      case 64: return launchStepMfmaT<float, 64, 64>(a, stream);
+    }
   }
   return hipErrorInvalidValue;
 }

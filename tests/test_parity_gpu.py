@@ -200,13 +200,14 @@ def test_whole_row_kernel_for_three_32x16_factors(fk):
 
 
 @pytest.mark.parametrize("M,Ps", [(3, [64]), (2, [16, 16]), (5, [32, 32]), (2, [64, 64, 64]), (7, [16] * 4), (4, [64, 16, 32])])
-def test_fp64_mfma_step_kernel(fk, M, Ps):
-    """fp64 steps with 16/32/64-wide square factors run on the fp64 matrix cores, including tiles with
-    fewer than 64 slices and mixed chains."""
-    check(fk, ko.MKM, M, Ps, Ps, np.float64, alpha=1.5, beta=0.5, seed=41)
+@pytest.mark.parametrize("dt", [np.float64, np.float32])
+def test_mfma_step_kernel(fk, M, Ps, dt):
+    """Steps with 16/32/64-wide square factors run on the matrix cores (fp64 and fp32), including tiles
+    with fewer than 16 slices and mixed chains."""
+    check(fk, ko.MKM, M, Ps, Ps, dt, alpha=1.5, beta=0.5, seed=41)
     assert all("mfma16x16x4" in k for _, _, k in fk.last_plan()), fk.last_plan()
-    check(fk, ko.MKM, M, Ps, Ps, np.float64, alpha=1.0, beta=0.0, seed=42, opFs=ko.OP_T)
-    check(fk, ko.MKM, M, Ps, Ps, np.float64, alpha=1.0, beta=1.0, seed=43, batch=2)
+    check(fk, ko.MKM, M, Ps, Ps, dt, alpha=1.0, beta=0.0, seed=42, opFs=ko.OP_T)
+    check(fk, ko.MKM, M, Ps, Ps, dt, alpha=1.0, beta=1.0, seed=43, batch=2)
 
 
 @pytest.mark.parametrize("M,Ps", [(64, [4] * 6), (100, [4] * 3), (16, [4] * 6), (130, [8] * 2), (64, [8] * 4),
