@@ -137,7 +137,7 @@ void registerRowKernels(std::vector<KernelInfo>& out) {
   }
 
   for (DType dt : {DType::F64, DType::F32})
-  for (uint32_t P : {16u, 32u, 64u}) {
+  for (uint32_t P : {16u, 32u, 64u, 128u}) {
     KernelInfo kd{};
     const std::string ps = std::to_string(P);
     kd.name = std::string("mkm_hip_gfx950_256_") + (dt == DType::F64 ? "d_" : "f_") + ps + "x" + ps + "_" + ps + "x" + ps + "_1_1x" + std::to_string(16 * P) +

@@ -1,4 +1,4 @@
-// One sliced-multiply step with a square factor (P = Q in {16, 32, 64}), MKM layout, fp64 or fp32, on the
+// One sliced-multiply step with a square factor (P = Q in {16, 32, 64, 128}), MKM layout, fp64 or fp32, on the
 // matrix cores (V_MFMA_F64_16X16X4_F64 / V_MFMA_F32_16X16X4_F32).  Used per factor for shapes like dgemkm 256 x 262144
 // with 64x64^3, where every step is a real (M*Kin/P) x P x Q contraction.
 //
@@ -49,13 +49,15 @@ template <> struct Mfma16<float> {
 
 constexpr int kStepWaves = 4;            // waves per workgroup
 
-template <typename T, int P, int Q, bool HAS_Y>
+// QS > 1 splits the Q output columns of a tile over QS wave tasks (each keeps only its Q/QS columns of
+// the factor in registers); used for 128x128, whose factor does not fit the register file of one wave.
+template <typename T, int P, int Q, int QS, bool HAS_Y>
 __global__ __launch_bounds__(256, 2) void kron_step_mfma_kernel(const StepArgs a, const uint32_t tilesPerRow,
                                                                 const uint32_t totalTiles) {
   using M16 = Mfma16<T>;
   using Acc = typename M16::Acc;
   constexpr int PC = P / 4;              // products per tile and elements per lane
-  constexpr int NB = Q / 16;
+  constexpr int NB = Q / 16 / QS;        // 16-column blocks per wave task
   constexpr int VE = 16 / sizeof(T);     // elements per 128-bit load
   typedef T VT __attribute__((ext_vector_type(VE)));
   const int tid = threadIdx.x;
@@ -70,16 +72,24 @@ __global__ __launch_bounds__(256, 2) void kron_step_mfma_kernel(const StepArgs a
   const T* F = (const T*)a.f[0] + (size_t)bt * a.f_batch[0];
   const T* YB = HAS_Y ? (const T*)a.y + (size_t)bt * a.y_batch : nullptr;
 
-  // the whole factor as A operands, resident in registers: fa[c][ib] = F[PC*hi + c][16*ib + lo]
+  const T alpha = (T)a.alpha, beta = (T)a.beta;
+  // wave tasks: the QS column parts of a tile go to QS different waves, a wave keeps its part for life
+  // Workgroups are dispatched round-robin over the 8 XCDs (each with its own L2): renumber them so that
+  // consecutive ids, which share tiles when QS > kStepWaves and walk neighbouring tiles otherwise, sit on
+  // one XCD.
+  const uint32_t wg = (gridDim.x % 8 == 0) ? (blockIdx.x % 8) * (gridDim.x / 8) + blockIdx.x / 8 : blockIdx.x;
+  const uint32_t gw = wg * kStepWaves + w;
+  const uint32_t qpart = gw % QS, q0 = qpart * (Q / QS);
+  const uint32_t waveId = gw / QS, nWaves = (gridDim.x * kStepWaves) / QS;
+
+  // the factor columns of this wave as A operands, resident in registers:
+  // fa[c][ib] = F[PC*hi + c][q0 + 16*ib + lo]
   T fa[PC][NB];
 #pragma unroll
   for (int c = 0; c < PC; c++)
 #pragma unroll
     for (int ib = 0; ib < NB; ib++)
-      fa[c][ib] = F[(int64_t)(PC * hi + c) * a.f_sp[0] + (int64_t)(16 * ib + lo) * a.f_sq[0]];
-
-  const T alpha = (T)a.alpha, beta = (T)a.beta;
-  const uint32_t waveId = blockIdx.x * kStepWaves + w, nWaves = gridDim.x * kStepWaves;
+      fa[c][ib] = F[(int64_t)(PC * hi + c) * a.f_sp[0] + (int64_t)(q0 + 16 * ib + lo) * a.f_sq[0]];
 
   auto loadTile = [&](uint32_t t, T (&x)[PC]) {
     const uint32_t m = t / tilesPerRow;
@@ -121,13 +131,13 @@ __global__ __launch_bounds__(256, 2) void kron_step_mfma_kernel(const StepArgs a
 #pragma unroll
       for (int ib = 0; ib < NB; ib++)
 #pragma unroll
-        for (int r = 0; r < 4; r++) yv[ib][r] = Y[(uint64_t)(16 * ib + M16::row(r, hi)) * S + s];
+        for (int r = 0; r < 4; r++) yv[ib][r] = Y[(uint64_t)(q0 + 16 * ib + M16::row(r, hi)) * S + s];
     }
 #pragma unroll
     for (int ib = 0; ib < NB; ib++)
 #pragma unroll
       for (int r = 0; r < 4; r++) {
-        const uint64_t col = (uint64_t)(16 * ib + M16::row(r, hi)) * S + s;
+        const uint64_t col = (uint64_t)(q0 + 16 * ib + M16::row(r, hi)) * S + s;
         T v = acc[ib][r];
         if (a.epilogue) {
           v *= alpha;
@@ -141,7 +151,7 @@ __global__ __launch_bounds__(256, 2) void kron_step_mfma_kernel(const StepArgs a
 bool stepMfmaSupported(const StepArgs& a, DType dt) {
   if (a.nf != 1) return false;
   const uint32_t P = a.p[0], Q = a.q[0];
-  if (!((P == 64 && Q == 64) || (P == 32 && Q == 32) || (P == 16 && Q == 16))) return false;
+  if (!((P == 128 && Q == 128) || (P == 64 && Q == 64) || (P == 32 && Q == 32) || (P == 16 && Q == 16))) return false;
   if (a.in_ldc != 1 || a.out_ldc != 1 || (a.y && a.y_ldc != 1)) return false;
   if (a.Kin % P) return false;
   // 16-byte alignment of every slice for the 128-bit loads
@@ -152,7 +162,7 @@ bool stepMfmaSupported(const StepArgs& a, DType dt) {
   return tiles * a.M < (1ull << 31) && a.batch <= 65535;
 }
 
-template <typename T, int P, int Q>
+template <typename T, int P, int Q, int QS>
 static hipError_t launchStepMfmaT(const StepArgs& a, hipStream_t stream) {
   const uint64_t S = a.Kin / P;
   const uint32_t tilesPerRow = (uint32_t)((S + 15) / 16);
@@ -166,13 +176,16 @@ static hipError_t launchStepMfmaT(const StepArgs& a, hipStream_t stream) {
   }
   // persistent workgroups: 2 per CU (8 waves, 2 per SIMD at up to 256 VGPRs), fewer when there is not enough work
   uint32_t wgs = (uint32_t)cus * 2;
-  const uint32_t need = (totalTiles + kStepWaves - 1) / kStepWaves;
+  const uint32_t need = (totalTiles * QS + kStepWaves - 1) / kStepWaves;
   if (wgs > need) wgs = need;
+  static_assert(kStepWaves % QS == 0 || QS % kStepWaves == 0, "wave tasks must tile the workgroups");
+  if (QS > kStepWaves) wgs = (wgs + QS / kStepWaves - 1) / (QS / kStepWaves) * (QS / kStepWaves);
+  if (wgs >= 64) wgs = wgs / 8 * 8;      // a multiple of the XCD count keeps the renumbering on
   dim3 grid(wgs, a.batch), block(256);
   if (a.y && a.epilogue)
-    hipLaunchKernelGGL((kron_step_mfma_kernel<T, P, Q, true>), grid, block, 0, stream, a, tilesPerRow, totalTiles);
+    hipLaunchKernelGGL((kron_step_mfma_kernel<T, P, Q, QS, true>), grid, block, 0, stream, a, tilesPerRow, totalTiles);
   else
-    hipLaunchKernelGGL((kron_step_mfma_kernel<T, P, Q, false>), grid, block, 0, stream, a, tilesPerRow, totalTiles);
+    hipLaunchKernelGGL((kron_step_mfma_kernel<T, P, Q, QS, false>), grid, block, 0, stream, a, tilesPerRow, totalTiles);
   return hipGetLastError();
 }
 
@@ -180,15 +193,17 @@ hipError_t launchStepMfma(const StepArgs& a, DType dt, hipStream_t stream) {
   if (!stepMfmaSupported(a, dt)) return hipErrorInvalidValue;
   if (dt == DType::F64) {
     switch (a.p[0]) {
-      case 16: return launchStepMfmaT<double, 16, 16>(a, stream);
-      case 32: return launchStepMfmaT<double, 32, 32>(a, stream);
-      case 64: return launchStepMfmaT<double, 64, 64>(a, stream);
+      case 16:  return launchStepMfmaT<double, 16, 16, 1>(a, stream);
+      case 32:  return launchStepMfmaT<double, 32, 32, 1>(a, stream);
+      case 64:  return launchStepMfmaT<double, 64, 64, 1>(a, stream);
+      case 128: return launchStepMfmaT<double, 128, 128, 8>(a, stream);
     }
   } else {
     switch (a.p[0]) {
-      case 16: return launchStepMfmaT<float, 16, 16>(a, stream);
-      case 32: return launchStepMfmaT<float, 32, 32>(a, stream);
-      case 64: return launchStepMfmaT<float, 64, 64>(a, stream);
+      case 16:  return launchStepMfmaT<float, 16, 16, 1>(a, stream);
+      case 32:  return launchStepMfmaT<float, 32, 32, 1>(a, stream);
+      case 64:  return launchStepMfmaT<float, 64, 64, 1>(a, stream);
+      case 128: return launchStepMfmaT<float, 128, 128, 2>(a, stream);
     }
   }
   return hipErrorInvalidValue;

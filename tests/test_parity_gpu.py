@@ -199,7 +199,8 @@ def test_whole_row_kernel_for_three_32x16_factors(fk):
     check(fk, ko.MKM, 2, [2] + [32] * 3, [3] + [16] * 3, np.float32, alpha=1.0, beta=0.5, seed=37)
 
 
-@pytest.mark.parametrize("M,Ps", [(3, [64]), (2, [16, 16]), (5, [32, 32]), (2, [64, 64, 64]), (7, [16] * 4), (4, [64, 16, 32])])
+@pytest.mark.parametrize("M,Ps", [(3, [64]), (2, [16, 16]), (5, [32, 32]), (2, [64, 64, 64]), (7, [16] * 4), (4, [64, 16, 32]),
+                                  (5, [128]), (3, [128, 128]), (40, [128, 64])])
 @pytest.mark.parametrize("dt", [np.float64, np.float32])
 def test_mfma_step_kernel(fk, M, Ps, dt):
     """Steps with 16/32/64-wide square factors run on the matrix cores (fp64 and fp32), including tiles
