@@ -130,6 +130,10 @@ fastKronError Handle::xgemm(KronProblem p, fastKronBackend backend, void* temp1,
   const std::string key = p.str();
   bool have = false;
   if (!p.forward) have = db_.lookupTuned(key, &plan);
+  if (!have && !canTune() && useFusion()) {
+    e = trySplitLeadingTrailing(p, temp1, temp2);
+    if (e != fastKronKernelNotFound) return e;
+  }
   if (!have && canTune() && !p.forward) {
     e = tune(p, &plan);
     if (e != fastKronSuccess) return e;
@@ -162,6 +166,73 @@ fastKronError Handle::xgemm(KronProblem p, fastKronBackend backend, void* temp1,
   for (auto& s : plan)
     lastPlan_ += ";" + std::to_string(s.lo) + "-" + std::to_string(s.hi) + ":" + db_.kernels()[s.kernel].name;
   return execute(p, plan, temp1, temp2);
+}
+
+// X (F_0 x ... x F_{N-1}) = first apply the trailing factors B = F_g x ... x F_{N-1} to every contiguous
+// block of prod(P_g..) columns (an MKM problem on M * K_A "virtual rows", K_A = prod of the leading P), then
+// apply the leading factors A = F_0 x ... x F_{g-1} across the blocks: for every row that is a KMM problem
+// on a K_A x T matrix whose T columns are contiguous.  Two or three launches instead of N.  The layout
+// between the two parts is [row][k_A][q_B] (digits in place), which only these two sub-problems see.
+fastKronError Handle::trySplitLeadingTrailing(const KronProblem& p, void* temp1, void* temp2) {
+  if (p.mm != MMType::MKM || p.dt != DType::F32 || p.forward || p.opX != fastKronOp_N) return fastKronKernelNotFound;
+  if (!temp1 || !temp2 || p.N < 3) return fastKronKernelNotFound;
+  // trailing run of identical 8x8 (at most 5) or 16x16 (at most 4) factors
+  const uint32_t tp = p.P[p.N - 1];
+  if ((tp != 8 && tp != 16) || p.Q[p.N - 1] != tp) return fastKronKernelNotFound;
+  const uint32_t maxT = (tp == 8) ? 5 : 4;
+  uint32_t nT = 0;
+  while (nT < maxT && nT < p.N && p.P[p.N - 1 - nT] == tp && p.Q[p.N - 1 - nT] == tp) nT++;
+  if (nT != maxT || nT == p.N) return fastKronKernelNotFound;      // shorter chains are whole-row problems already
+  const uint32_t g = p.N - nT;
+  const uint32_t lp = p.P[0];
+  if (lp != 4 && lp != 8 && lp != 16) return fastKronKernelNotFound;
+  for (uint32_t i = 0; i < g; i++) if (p.P[i] != lp || p.Q[i] != lp) return fastKronKernelNotFound;
+  const uint32_t perLaunch = (lp == 4) ? 3 : (lp == 8) ? 2 : 1;
+  if (g > 2 * perLaunch) return fastKronKernelNotFound;             // the KMM part may use temp2 only
+  uint64_t KA = 1, T = 1;
+  for (uint32_t i = 0; i < g; i++) KA *= lp;
+  for (uint32_t i = 0; i < nT; i++) T *= tp;
+  const uint64_t K = KA * T;
+  if (p.batch > 1) {
+    if (p.strideX != (uint64_t)p.M * K || p.strideZ != (uint64_t)p.M * K) return fastKronKernelNotFound;
+    if (p.Y && p.beta != 0.0 && p.strideY != (uint64_t)p.M * K) return fastKronKernelNotFound;
+    for (uint32_t i = 0; i < g; i++) if (p.strideF[i] != 0) return fastKronKernelNotFound;
+  }
+  if ((uint64_t)p.M * p.batch > 65535 || (uint64_t)p.M * KA >= (1ull << 31)) return fastKronKernelNotFound;
+
+  // part 1: trailing factors, X -> temp1, no epilogue
+  KronProblem q1 = p;
+  q1.M = (uint32_t)(p.M * KA); q1.N = nT;
+  for (uint32_t i = 0; i < nT; i++) {
+    q1.P[i] = p.P[g + i]; q1.Q[i] = p.Q[g + i]; q1.F[i] = p.F[g + i]; q1.strideF[i] = p.strideF[g + i];
+  }
+  q1.Z = temp1; q1.strideZ = (uint64_t)p.M * K;
+  q1.Y = nullptr; q1.strideY = 0; q1.alpha = 1.0; q1.beta = 0.0;
+  Plan plan1 = db_.selectOnline(q1, dev_, true);
+  if (plan1.size() != 1 || db_.kernels()[plan1[0].kernel].P == 0) return fastKronKernelNotFound;
+  if (execute(q1, plan1, nullptr, nullptr, true) != fastKronSuccess) return fastKronKernelNotFound;
+
+  // part 2: leading factors as a KMM over every row block; P x Q storage is the transpose of KMM's Q x P
+  KronProblem q2 = p;
+  q2.mm = MMType::KMM; q2.M = (uint32_t)T; q2.N = g;
+  q2.opF = (p.opF == fastKronOp_N) ? fastKronOp_T : fastKronOp_N;
+  q2.opX = fastKronOp_N;
+  q2.X = temp1; q2.strideX = K;
+  q2.strideZ = K; q2.strideY = K;
+  q2.batch = p.batch * p.M; q2.strided = true;
+  Plan plan2 = db_.selectOnline(q2, dev_, true);
+  if (plan2.size() > 2) return fastKronKernelNotFound;
+  for (auto& s : plan2) if (db_.kernels()[s.kernel].P == 0) return fastKronKernelNotFound;
+  if (execute(q2, plan2, temp2, nullptr, true) != fastKronSuccess) return fastKronKernelNotFound;
+
+  lastPlan_ = p.str();
+  for (auto& s : plan1)
+    lastPlan_ += ";" + std::to_string(g + s.lo) + "-" + std::to_string(g + s.hi) + ":" + db_.kernels()[s.kernel].name;
+  for (auto& s : plan2)
+    lastPlan_ += ";" + std::to_string(s.lo) + "-" + std::to_string(s.hi) + ":" + db_.kernels()[s.kernel].name;
+  fastKronError e = execute(q1, plan1, nullptr, nullptr);
+  if (e != fastKronSuccess) return e;
+  return execute(q2, plan2, temp2, nullptr);
 }
 
 // Everything of a launch's arguments that follows from the problem and the factor range; the caller

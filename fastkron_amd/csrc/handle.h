@@ -41,6 +41,10 @@ class Handle {
   // Runs `plan` on the stream; temps may be null when the plan has a single launch.
   fastKronError execute(const KronProblem& p, const Plan& plan, void* temp1, void* temp2, bool dryRun = false);
   fastKronError tune(const KronProblem& p, Plan* best);
+  // MKM chains longer than a whole-row kernel can take: trailing factors by the row kernel on
+  // M * prod(leading P) virtual rows, leading factors as a batched KMM over the row blocks.
+  // Returns fastKronKernelNotFound when the problem does not have that form.
+  fastKronError trySplitLeadingTrailing(const KronProblem& p, void* temp1, void* temp2);
 
   const std::string& lastPlan() const { return lastPlan_; }
   void setTunedDB(const char* path);

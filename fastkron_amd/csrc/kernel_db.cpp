@@ -100,7 +100,7 @@ static bool kmmRegCanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo,
   if (p.dt != DType::F32 || p.mm != MMType::KMM || hi - lo + 1 != k.fused || p.forward) return false;
   for (uint32_t i = lo; i <= hi; i++) if (p.P[i] != k.P || p.Q[i] != k.Q) return false;
   if (first && p.opX == 2) return false;
-  return p.colsBefore(hi) % 64 == 0 && p.M >= 16;
+  return p.colsBefore(hi) % k.tileK == 0 && p.M >= 16;
 }
 static hipError_t kmmRegLaunch(const KernelInfo&, const StepArgs& a, hipStream_t s) { return launchKmmReg(a, s); }
 static bool kmmRegCheck(const KernelInfo&, const StepArgs& a) { return kmmRegSupported(a); }
@@ -125,13 +125,16 @@ void registerRowKernels(std::vector<KernelInfo>& out) {
   k32.variant = 0; k32.canRun = row32CanRun; k32.launch = row32Launch; k32.check = row32Check;
   out.push_back(k32);
 
-  for (uint32_t P : {4u, 8u}) {
+  // deepest fusion first: the online selection takes the first kernel that fits at a given depth
+  for (auto pn : {std::pair<uint32_t, uint32_t>{4, 3}, {8, 2}, {4, 2}, {4, 1}, {8, 1}, {16, 1}}) {
     KernelInfo kk{};
-    const std::string ps = std::to_string(P);
-    kk.fused = (P == 4) ? 3 : 2;
+    const std::string ps = std::to_string(pn.first);
+    uint32_t G = 1;
+    for (uint32_t i = 0; i < pn.second; i++) G *= pn.first;
+    kk.fused = pn.second;
     kk.name = "kmm_hip_gfx950_256_f_" + ps + "x" + ps + "_" + ps + "x" + ps + "_" + std::to_string(kk.fused) +
-              "_64x64_mfma4x4x1_NN_strided_0_3";
-    kk.dt = DType::F32; kk.P = P; kk.Q = P; kk.tileM = 64; kk.tileK = 64; kk.threads = 256; kk.variant = 0;
+              "_64x" + std::to_string(G) + "_mfma4x4x1_NN_strided_0_3";
+    kk.dt = DType::F32; kk.P = pn.first; kk.Q = pn.first; kk.tileM = 64; kk.tileK = G; kk.threads = 256; kk.variant = 0;
     kk.canRun = kmmRegCanRun; kk.launch = kmmRegLaunch; kk.check = kmmRegCheck;
     out.push_back(kk);
   }

@@ -1,6 +1,7 @@
 // Fused steps for small square fp32 factors in the KMM layout (operands are K x M row-major, the M
-// columns are the contiguous dimension): NF factors of P x P with P^NF = 64, e.g. three 4x4 or two
-// 8x8 factors per launch (sgekmm with 4x4^6 runs as two launches of three factors).
+// columns are the contiguous dimension): NF factors of P x P with G = P^NF <= 64 values per lane, e.g.
+// three 4x4 or two 8x8 factors per launch (sgekmm with 4x4^6 runs as two launches of three factors),
+// or a single 8x8 / 16x16 factor.
 //
 //   out[(q_1..q_NF)*SG + sg, m] = sum_{k_1..k_NF} F_1[q_1,k_1] ... F_NF[q_NF,k_NF] * in[sg*64 + (k_1..k_NF), m]
 //
@@ -24,9 +25,10 @@ typedef float f4 __attribute__((ext_vector_type(4)));
 
 #define MFMA4(a, b, c) __builtin_amdgcn_mfma_f32_4x4x1f32((a), (b), (c), 0, 0, 0)
 
-template <int P, int NF> struct KmmRegCfg;
-template <> struct KmmRegCfg<4, 3> { static constexpr int G = 64; };
-template <> struct KmmRegCfg<8, 2> { static constexpr int G = 64; };
+template <int P, int NF> struct KmmRegCfg {
+  static constexpr int G = (NF == 1) ? P : (NF == 2) ? P * P : P * P * P;
+  static_assert(G <= 64 && P % 4 == 0 && NF >= 1 && NF <= 3, "unsupported KMM register tile");
+};
 
 constexpr int kKmmWaves = 4;
 
@@ -97,13 +99,14 @@ __global__ __launch_bounds__(256, HAS_Y ? 3 : 4) void kron_kmm_reg_kernel(const 
       // counter, so a load behind a store could only be waited for together with that store); a
       // rolling window of 16 registers keeps the loads in flight.
       const float* Y = (const float*)a.y + (size_t)bt * a.y_batch + (size_t)m * a.y_ldm;
-      float yw[16];
+      constexpr int YW = (G < 16) ? G : 16;
+      float yw[YW];
 #pragma unroll
-      for (int e = 0; e < 16; e++) yw[e] = Y[(int64_t)((uint64_t)e * SG + sg) * a.y_ldc];
+      for (int e = 0; e < YW; e++) yw[e] = Y[(int64_t)((uint64_t)e * SG + sg) * a.y_ldc];
 #pragma unroll
       for (int e = 0; e < G; e++) {
-        x[e] = alpha * x[e] + beta * yw[e & 15];
-        if (e + 16 < G) yw[e & 15] = Y[(int64_t)((uint64_t)(e + 16) * SG + sg) * a.y_ldc];
+        x[e] = alpha * x[e] + beta * yw[e % YW];
+        if (e + YW < G) yw[e % YW] = Y[(int64_t)((uint64_t)(e + YW) * SG + sg) * a.y_ldc];
       }
     } else {
 #pragma unroll
@@ -114,19 +117,29 @@ __global__ __launch_bounds__(256, HAS_Y ? 3 : 4) void kron_kmm_reg_kernel(const 
   for (int e = 0; e < G; e++) out[(int64_t)((uint64_t)e * SG + sg) * a.out_ldc] = x[e];
 }
 
+// Tile width (values per lane) for a supported (P, nf) pair, 0 otherwise.
+static uint32_t kmmRegTile(uint32_t P, uint32_t nf) {
+  if (P == 4 && nf >= 1 && nf <= 3) return nf == 1 ? 4 : nf == 2 ? 16 : 64;
+  if (P == 8 && nf >= 1 && nf <= 2) return nf == 1 ? 8 : 64;
+  if (P == 16 && nf == 1) return 16;
+  return 0;
+}
+
 bool kmmRegSupported(const StepArgs& a) {
-  if (!((a.nf == 3 && a.p[0] == 4) || (a.nf == 2 && a.p[0] == 8))) return false;
+  const uint32_t G = kmmRegTile(a.p[0], a.nf);
+  if (!G) return false;
   for (uint32_t j = 0; j < a.nf; j++) if (a.p[j] != a.p[0] || a.q[j] != a.p[0]) return false;
   if (a.in_ldm != 1 || a.out_ldm != 1 || (a.y && a.y_ldm != 1)) return false;
-  if (a.Kin % 64) return false;
-  const uint64_t tiles = (a.Kin / 64) * ((a.M + 63) / 64);
+  if (a.Kin % G) return false;
+  const uint64_t tiles = (a.Kin / G) * ((a.M + 63) / 64);
   return tiles < (1ull << 31) && a.batch <= 65535;
 }
 
 template <int P, int NF>
 static hipError_t launchKmmRegT(const StepArgs& a, hipStream_t stream) {
+  constexpr int G = KmmRegCfg<P, NF>::G;
   const uint32_t mTiles = (a.M + 63) / 64;
-  const uint32_t totalTiles = (uint32_t)((a.Kin / 64) * mTiles);
+  const uint32_t totalTiles = (uint32_t)((a.Kin / G) * mTiles);
   dim3 grid((totalTiles + kKmmWaves - 1) / kKmmWaves, a.batch), block(256);
   if (a.y && a.epilogue)
     hipLaunchKernelGGL((kron_kmm_reg_kernel<P, NF, true>), grid, block, 0, stream, a, mTiles, totalTiles);
@@ -137,8 +150,15 @@ static hipError_t launchKmmRegT(const StepArgs& a, hipStream_t stream) {
 
 hipError_t launchKmmReg(const StepArgs& a, hipStream_t stream) {
   if (!kmmRegSupported(a)) return hipErrorInvalidValue;
-  if (a.p[0] == 4) return launchKmmRegT<4, 3>(a, stream);
-  return launchKmmRegT<8, 2>(a, stream);
+  switch (a.p[0] * 10 + a.nf) {
+    case 41:  return launchKmmRegT<4, 1>(a, stream);
+    case 42:  return launchKmmRegT<4, 2>(a, stream);
+    case 43:  return launchKmmRegT<4, 3>(a, stream);
+    case 81:  return launchKmmRegT<8, 1>(a, stream);
+    case 82:  return launchKmmRegT<8, 2>(a, stream);
+    case 161: return launchKmmRegT<16, 1>(a, stream);
+  }
+  return hipErrorInvalidValue;
 }
 
 }  // namespace fk

@@ -317,3 +317,24 @@ def test_row_kernels_need_whole_blocks(fk):
     """A row count that is not a whole number of blocks takes the generic kernels instead."""
     check(fk, ko.MKM, 12, [8] * 4, [8] * 4, np.float32, alpha=1.0, beta=0.0, seed=93)
     assert all("generic" in k for _, _, k in fk.last_plan())
+
+
+@pytest.mark.parametrize("M,Ps", [(4, [8] * 6), (2, [8] * 7), (3, [4, 4] + [8] * 5), (2, [16] * 5), (1, [16] * 6),
+                                  (2, [4, 4, 4] + [16] * 4), (2, [8, 8] + [16] * 4)])
+def test_long_chains_split_into_row_kernel_plus_leading_kmm(fk, M, Ps):
+    """Chains longer than a whole-row kernel takes: trailing factors by the row kernel on M*K_A virtual rows,
+    leading factors as a batched KMM over the row blocks (2-3 launches instead of N)."""
+    check(fk, ko.MKM, M, Ps, Ps, np.float32, alpha=1.5, beta=0.5, seed=101)
+    plan = fk.last_plan()
+    assert len(plan) <= 3 and any("kmm_" in k for _, _, k in plan) and any("mkm_" in k for _, _, k in plan), plan
+    check(fk, ko.MKM, M, Ps, Ps, np.float32, alpha=1.0, beta=0.0, seed=102, opFs=ko.OP_T)
+    check(fk, ko.MKM, M, Ps, Ps, np.float32, alpha=1.0, beta=1.0, seed=103, batch=2, share_f=True)
+    # per-batch factors cannot use the split (the KMM part flattens batch and rows): still correct
+    check(fk, ko.MKM, M, Ps, Ps, np.float32, alpha=1.0, beta=1.0, seed=104, batch=2)
+
+
+@pytest.mark.parametrize("M,Ps", [(64, [8]), (70, [8] * 3), (64, [16]), (100, [16, 16]), (64, [4]), (80, [4, 4]), (64, [4] * 4)])
+def test_kmm_register_kernel_more_tiles(fk, M, Ps):
+    check(fk, ko.KMM, M, Ps, Ps, np.float32, alpha=1.5, beta=0.5, seed=111)
+    assert all("mfma4x4x1" in k for _, _, k in fk.last_plan()), fk.last_plan()
+    check(fk, ko.KMM, M, Ps, Ps, np.float32, alpha=1.0, beta=0.0, seed=112, batch=3)
