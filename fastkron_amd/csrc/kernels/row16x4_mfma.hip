@@ -32,12 +32,13 @@ typedef float f4 __attribute__((ext_vector_type(4)));
 
 #define MFMA16(a, b, c) __builtin_amdgcn_mfma_f32_16x16x4f32((a), (b), (c), 0, 0, 0)
 
+
 #ifdef FK_ROW_TIMING
-// Experiment-only build: phase time stamps (s_memtime) of wave 0 of every workgroup.
-__device__ unsigned long long g_rowTiming[1024 * 8];
-#define FK_STAMP(k) do { if (tid == 0 && blockIdx.x < 1024) g_rowTiming[blockIdx.x * 8 + (k)] = __builtin_readcyclecounter(); } while (0)
+// Experiment-only build: phase time stamps (s_memtime) of wave 0, [workgroup][item][phase].
+__device__ unsigned long long g_rowTiming[256 * 4 * 8];
+#define FK_STAMP(k) do { if (tid == 0 && blockIdx.x < 256 && itn < 4) g_rowTiming[(blockIdx.x * 4 + itn) * 8 + (k)] = __builtin_readcyclecounter(); } while (0)
 extern "C" void fkDebugReadRowTiming(unsigned long long* out) {
-  (void)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_rowTiming), sizeof(unsigned long long) * 1024 * 8);
+  (void)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_rowTiming), sizeof(unsigned long long) * 256 * 4 * 8);
 }
 #else
 #define FK_STAMP(k)
@@ -45,180 +46,235 @@ extern "C" void fkDebugReadRowTiming(unsigned long long* out) {
 
 constexpr int kRowLen = 65536;
 constexpr int kLdsWords = 32768;           // 128 KB: one half of a row
+constexpr int kPF = 8;                     // blocks (of 16) of the next item loaded one item ahead
 
 template <bool HAS_Y>
-__global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a, const uint32_t firstWave,
-                                                               const uint32_t groups, const uint32_t delayCycles) {
+__global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a, const uint32_t blocksPerBatch,
+                                                               const uint32_t totalItems, const uint32_t groups,
+                                                               const uint32_t delayCycles) {
   extern __shared__ float lds[];
   const int tid = threadIdx.x;
-  // One workgroup fills a CU, so every CU alternates between an HBM phase (load, store) and an
-  // on-chip phase (MFMA, LDS exchange).  Workgroups that start together stay in lockstep and leave
-  // HBM idle during the on-chip phases; delaying a part of the first wave of workgroups by a fraction
-  // of the row period interleaves the phases of different CUs.  Later workgroups inherit the offset.
+  // One workgroup fills a CU, so every CU alternates between HBM phases (load, store) and on-chip
+  // phases (MFMA, LDS exchange).  Workgroups are persistent (one per CU, looping over row blocks);
+  // delaying a part of them at start interleaves the phases of different CUs a little.
   if (groups > 1) {
-    const uint32_t wg = blockIdx.x + blockIdx.y * gridDim.x;
-    const uint32_t g = (wg >> 3) % groups;   // workgroups go round-robin over the 8 XCDs: keep every group on every XCD
-    if (wg < firstWave && g != 0) {
-      // pure s_sleep (64 cycles per unit): polling a clock from thousands of waves would itself load the memory path
-      const uint32_t n = (g * delayCycles) >> 12;                 // units of 64*64 cycles
-      for (uint32_t k = 0; k < n; k++) __builtin_amdgcn_s_sleep(64);
-    }
+    const uint32_t g = (blockIdx.x >> 3) % groups;   // workgroups go round-robin over the 8 XCDs: keep every group on every XCD
+    // pure s_sleep (64 cycles per unit): polling a clock from thousands of waves would itself load the memory path
+    const uint32_t n = (g * delayCycles) >> 12;
+    for (uint32_t k = 0; k < n; k++) __builtin_amdgcn_s_sleep(64);
   }
-  const int l = tid & 63;
+  const int l0 = tid & 63;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);      // wave-uniform: keeps row addresses in SGPRs
-  const int i = l & 15, kb = l >> 4;
-  const uint32_t m = blockIdx.x, b = blockIdx.y;
-  FK_STAMP(0);
-#ifdef FK_ROW_TIMING
-  if (tid == 0 && blockIdx.x < 1024) g_rowTiming[blockIdx.x * 8 + 6] = wall_clock64();
-#endif
 
-  // m counts blocks of 65536 contiguous elements: one row for four factors, 16^(4-nf) rows otherwise
-  const float* X = (const float*)a.in + (size_t)b * a.in_batch + (size_t)m * kRowLen;
-  float* Z = (float*)a.out + (size_t)b * a.out_batch + (size_t)m * kRowLen;
+  uint32_t item = blockIdx.x;
+  if (item >= totalItems) return;
 
-  // Factor operands (B side of every product).  a.f[0] is the last factor (F4) ... a.f[3] the first (F1).
-  // First product of a chain: B_c[k][j] = F[4c + k][j]; second product: B_r[k][j] = F[4k + r][j].
-  // With fewer than four factors the leading digits are row indices (16^(4-nf) consecutive rows form the
-  // same contiguous 65536-element block) and their factor slots hold the identity.
-  float FA[4], FB[4], FC[4], FD[4];
-  {
-    auto fetch = [&](int j, int p, int q) -> float {
-      if (j >= (int)a.nf) return (p == q) ? 1.f : 0.f;
+  // Factors: a.f[0] is the last factor (F4) ... a.f[3] the first (F1); with fewer than four factors the
+  // leading digits are row indices (16^(4-nf) consecutive rows form the same contiguous 65536-element
+  // block) and their factor slots hold the identity.  The four 16x16 matrices are staged in LDS behind
+  // the exchange buffer, fl[j*256 + p*16 + q], and the B operands of a stage are read from there right
+  // before the stage: LDS reads do not queue behind the row loads the way small global loads would
+  // (vector memory operations retire in order).
+  float* fl = lds + kLdsWords;
+  auto stageFactors = [&](uint32_t b) {
+    const int j = tid >> 8, p = (tid >> 4) & 15, q = tid & 15;
+    float v = (p == q) ? 1.f : 0.f;
+    if (j < (int)a.nf) {
       const float* f = (const float*)a.f[j] + (size_t)b * a.f_batch[j];
-      return f[(int64_t)p * a.f_sp[j] + (int64_t)q * a.f_sq[j]];
-    };
-#pragma unroll
-    for (int c = 0; c < 4; c++) {
-      FA[c] = fetch(1, 4 * c + kb, i);      // F3: first product of stage 1
-      FB[c] = fetch(0, 4 * kb + c, i);      // F4: second product of stage 1
-      FC[c] = fetch(3, 4 * c + kb, i);      // F1: first product of stage 2
-      FD[c] = fetch(2, 4 * kb + c, i);      // F2: second product of stage 2
+      v = f[(int64_t)p * a.f_sp[j] + (int64_t)q * a.f_sq[j]];
     }
-  }
-
-  // ---- load: wave w reads the 16 KB of k1 = w; x[t][c] = X[k1=w][k2=t][k3=4c+kb][k4=i] ----
-  float x[16][4];
-  {
-    const float* xp = X + w * 4096 + l;
-#pragma unroll
-    for (int t = 0; t < 16; t++)
-#pragma unroll
-      for (int c = 0; c < 4; c++) x[t][c] = xp[t * 256 + c * 64];
-  }
-
-  // ---- stage 1: contract k3 (first product) and k4 (second product) ----
-#pragma unroll
-  for (int t = 0; t < 16; t++) {
-    f4 d = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int c = 0; c < 4; c++) d = MFMA16(x[t][c], FA[c], d);
-    f4 e = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int r = 0; r < 4; r++) e = MFMA16(d[r], FB[r], e);
-#pragma unroll
-    for (int r = 0; r < 4; r++) x[t][r] = e[r];       // = Y[k1=w][k2=t][q3=4kb+r][q4=i]
-    // half 0 of exchange 1 goes out as soon as it exists, under the products of the next blocks
-#pragma unroll
-    for (int rr = 0; rr < 2; rr++)
-      lds[((kb * 2 + rr) * 16 + i) * 256 + ((w * 16 + t) ^ l)] = e[rr];
-  }
-
-  FK_STAMP(1);
-  // ---- exchange 1: rows (q3,q4), columns (k1,k2); half h holds the rows with bit 1 of q3 == h ----
-  float z[16][4];
-#pragma unroll
-  for (int h = 0; h < 2; h++) {
-    if (h) {
-      __syncthreads();
-#pragma unroll
-      for (int t = 0; t < 16; t++)
-#pragma unroll
-        for (int rr = 0; rr < 2; rr++) {
-          const int row = (kb * 2 + rr) * 16 + i;
-          lds[row * 256 + ((w * 16 + t) ^ l)] = x[t][2 + rr];
-        }
-    }
-    __syncthreads();
-#pragma unroll
-    for (int u = 0; u < 16; u++) {
-      if (((u >> 1) & 1) != h) continue;
-      const int row = ((u >> 2) * 2 + (u & 1)) * 16 + w;
-      const int swz = w + 16 * (u >> 2);
-#pragma unroll
-      for (int c = 0; c < 4; c++) z[u][c] = lds[row * 256 + ((c * 64 + l) ^ swz)];   // Y[k1=4c+kb][k2=i][q3=u][q4=w]
-    }
-  }
+    fl[tid] = v;
+  };
+  bool perBatchFactors = false;
+  for (uint32_t j = 0; j < a.nf; j++) perBatchFactors |= (a.f_batch[j] != 0);
+  stageFactors(item / blocksPerBatch);
   __syncthreads();
-  FK_STAMP(2);
 
-  // ---- stage 2: contract k1 (first product) and k2 (second product) ----
+  // An item is a block of 65536 contiguous elements: one row for four factors, 16^(4-nf) rows otherwise.
+  // xa holds blocks t = 0..kPF-1 (k2) of the item about to be processed; it is loaded one item ahead, under the
+  // second stage, the second exchange and the stores of the previous item.
+  float xa[kPF][4];
+  {
+    const float* xp = (const float*)a.in + (size_t)(item / blocksPerBatch) * a.in_batch +
+                      (size_t)(item % blocksPerBatch) * kRowLen + w * 4096 + l0;
 #pragma unroll
-  for (int u = 0; u < 16; u++) {
-    f4 d = {0.f, 0.f, 0.f, 0.f};
+    for (int t = 0; t < kPF; t++)
 #pragma unroll
-    for (int c = 0; c < 4; c++) d = MFMA16(z[u][c], FC[c], d);
-    f4 e = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int r = 0; r < 4; r++) e = MFMA16(d[r], FD[r], e);
-#pragma unroll
-    for (int r = 0; r < 4; r++) z[u][r] = e[r];       // = Z[q1=4kb+r][q2=i][q3=u][q4=w]
-    // half 0 of exchange 2 (every wave passed the barrier after its last read of exchange 1)
-#pragma unroll
-    for (int rr = 0; rr < 2; rr++)
-      lds[((kb * 2 + rr) * 16 + i) * 256 + ((u * 16 + w) ^ (i * 4) ^ kb)] = e[rr];
+      for (int c = 0; c < 4; c++) xa[t][c] = xp[t * 256 + c * 64];
   }
 
-  FK_STAMP(3);
-  // ---- exchange 2: rows (q1,q2), columns (q3,q4); half h holds the rows with bit 1 of q1 == h.
-  //      Reader: wave w owns q2 = w, lane owns columns 4l .. 4l+3, register index is q1. ----
-  f4 o[16];
+  for (int itn = 0; item < totalItems; item += gridDim.x, itn++) {
+    FK_STAMP(0);
+    // The lane id is laundered once per item: the hundreds of lane-dependent LDS offsets below are
+    // loop invariant, and hoisting them out of the item loop would pin them all in registers.
+    int l = l0;
+    asm volatile("" : "+v"(l));
+    const int i = l & 15, kb = l >> 4;
+    const uint32_t m = item % blocksPerBatch, b = item / blocksPerBatch;
+    const float* X = (const float*)a.in + (size_t)b * a.in_batch + (size_t)m * kRowLen;
+    float* Z = (float*)a.out + (size_t)b * a.out_batch + (size_t)m * kRowLen;
+    if (perBatchFactors && item != blockIdx.x && b != (item - gridDim.x) / blocksPerBatch) {   // a new batch: restage its factors
+      stageFactors(b);                                               // (all waves are past the closing barrier of the previous item)
+      __syncthreads();
+    }
+
+    // ---- second half of the row: x[t][c] = X[k1=w][k2=t][k3=4c+kb][k4=i], t = 8..15 ----
+    float xb[16 - kPF][4];
+    {
+      const float* xp = X + w * 4096 + l + kPF * 256;
 #pragma unroll
-  for (int h = 0; h < 2; h++) {
-    if (h) {
+      for (int t = 0; t < 16 - kPF; t++)
+#pragma unroll
+        for (int c = 0; c < 4; c++) xb[t][c] = xp[t * 256 + c * 64];
+    }
+
+    // ---- stage 1: contract k3 (first product) and k4 (second product), block by block.  The half of
+    //      the result with bit 1 of q3 clear goes to LDS at once, under the products of the next blocks. ----
+    {
+      // first product of a chain: B_c[k][j] = F[4c + k][j]; second product: B_r[k][j] = F[4k + r][j]
+      float FA[4], FB[4];
+#pragma unroll
+      for (int c = 0; c < 4; c++) {
+        FA[c] = fl[1 * 256 + (4 * c + kb) * 16 + i];      // F3
+        FB[c] = fl[0 * 256 + (4 * kb + c) * 16 + i];      // F4
+      }
+      auto stage1 = [&](auto& x, const int nt, const int t0) {
+#pragma unroll
+        for (int t = 0; t < nt; t++) {
+          f4 d = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int c = 0; c < 4; c++) d = MFMA16(x[t][c], FA[c], d);
+          f4 e = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int r = 0; r < 4; r++) e = MFMA16(d[r], FB[r], e);
+#pragma unroll
+          for (int r = 0; r < 4; r++) x[t][r] = e[r];     // = Y[k1=w][k2=t0+t][q3=4kb+r][q4=i]
+#pragma unroll
+          for (int rr = 0; rr < 2; rr++)
+            lds[((kb * 2 + rr) * 16 + i) * 256 + ((w * 16 + t0 + t) ^ l)] = e[rr];
+        }
+      };
+      stage1(xa, kPF, 0);
+      stage1(xb, 16 - kPF, kPF);
+    }
+
+    FK_STAMP(1);
+    // ---- exchange 1: rows (q3,q4), columns (k1,k2); half h holds the rows with bit 1 of q3 == h.
+    //      Reader layout: z[u][c] = Y[k1=4c+kb][k2=i][q3=u][q4=w]. ----
+    float z[16][4];
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+      if (h) {
+        __syncthreads();
+#pragma unroll
+        for (int t = 0; t < 16; t++)
+#pragma unroll
+          for (int rr = 0; rr < 2; rr++) {
+            const int row = (kb * 2 + rr) * 16 + i;
+            lds[row * 256 + ((w * 16 + t) ^ l)] = (t < kPF) ? xa[t < kPF ? t : 0][2 + rr] : xb[t < kPF ? 0 : t - kPF][2 + rr];
+          }
+      }
       __syncthreads();
 #pragma unroll
-      for (int u = 0; u < 16; u++)
+      for (int u = 0; u < 16; u++) {
+        if (((u >> 1) & 1) != h) continue;
+        const int row = ((u >> 2) * 2 + (u & 1)) * 16 + w;
+        const int swz = w + 16 * (u >> 2);
 #pragma unroll
-        for (int rr = 0; rr < 2; rr++) {
-          const int row = (kb * 2 + rr) * 16 + i;
-          lds[row * 256 + ((u * 16 + w) ^ (i * 4) ^ kb)] = z[u][2 + rr];
-        }
+        for (int c = 0; c < 4; c++) z[u][c] = lds[row * 256 + ((c * 64 + l) ^ swz)];
+      }
     }
     __syncthreads();
-#pragma unroll
-    for (int q1hi = 0; q1hi < 4; q1hi++)
-#pragma unroll
-      for (int rr = 0; rr < 2; rr++) {
-        const int row = (q1hi * 2 + rr) * 16 + w;
-        const f4 v = *(const f4*)&lds[row * 256 + ((l * 4) ^ (w * 4))];
-        f4 p;                                           // word e of v is column 4l + (e ^ q1hi)
-        p[0] = v[0 ^ q1hi]; p[1] = v[1 ^ q1hi]; p[2] = v[2 ^ q1hi]; p[3] = v[3 ^ q1hi];
-        o[4 * q1hi + 2 * h + rr] = p;
-      }
-  }
 
-  FK_STAMP(4);
-  // ---- epilogue and store: every wave-level store covers 1 KB of contiguous columns ----
-  const float alpha = (float)a.alpha, beta = (float)a.beta;
-  const float* Y = HAS_Y ? (const float*)a.y + (size_t)b * a.y_batch + (size_t)m * kRowLen : nullptr;
+    FK_STAMP(2);
+    // ---- the first half of the next item streams in from here on ----
+    {
+      const uint32_t nx = item + gridDim.x;
+      if (nx < totalItems) {
+        const float* xp = (const float*)a.in + (size_t)(nx / blocksPerBatch) * a.in_batch +
+                          (size_t)(nx % blocksPerBatch) * kRowLen + w * 4096 + l;
 #pragma unroll
-  for (int q1 = 0; q1 < 16; q1++) {
-    const int col = q1 * 4096 + w * 256 + l * 4;
-    f4 v = o[q1];
-    if (a.epilogue) {
-      v = v * alpha;
-      if (HAS_Y) {
-        const f4 yv = *(const f4*)(Y + col);
-        v = v + yv * beta;
+        for (int t = 0; t < kPF; t++)
+#pragma unroll
+          for (int c = 0; c < 4; c++) xa[t][c] = xp[t * 256 + c * 64];
       }
     }
-    *(f4*)(Z + col) = v;
+
+    // ---- stage 2: contract k1 (first product) and k2 (second product); half 0 of exchange 2 goes out
+    //      at once (rows (q1,q2), columns (q3,q4); half h holds the rows with bit 1 of q1 == h) ----
+    {
+      float FC[4], FD[4];
+#pragma unroll
+      for (int c = 0; c < 4; c++) {
+        FC[c] = fl[3 * 256 + (4 * c + kb) * 16 + i];      // F1
+        FD[c] = fl[2 * 256 + (4 * kb + c) * 16 + i];      // F2
+      }
+#pragma unroll
+      for (int u = 0; u < 16; u++) {
+        f4 d = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int c = 0; c < 4; c++) d = MFMA16(z[u][c], FC[c], d);
+        f4 e = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int r = 0; r < 4; r++) e = MFMA16(d[r], FD[r], e);
+#pragma unroll
+        for (int r = 0; r < 4; r++) z[u][r] = e[r];       // = Z[q1=4kb+r][q2=i][q3=u][q4=w]
+#pragma unroll
+        for (int rr = 0; rr < 2; rr++)
+          lds[((kb * 2 + rr) * 16 + i) * 256 + ((u * 16 + w) ^ (i * 4) ^ kb)] = e[rr];
+      }
+    }
+
+    FK_STAMP(3);
+    // ---- exchange 2 and store, half by half.  Reader: wave w owns q2 = w, lane owns columns 4l..4l+3,
+    //      register index is q1; every wave-level store covers 1 KB of contiguous columns. ----
+    const float alpha = (float)a.alpha, beta = (float)a.beta;
+    const float* Y = HAS_Y ? (const float*)a.y + (size_t)b * a.y_batch + (size_t)m * kRowLen : nullptr;
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+      if (h) {
+        __syncthreads();
+#pragma unroll
+        for (int u = 0; u < 16; u++)
+#pragma unroll
+          for (int rr = 0; rr < 2; rr++) {
+            const int row = (kb * 2 + rr) * 16 + i;
+            lds[row * 256 + ((u * 16 + w) ^ (i * 4) ^ kb)] = z[u][2 + rr];
+          }
+      }
+      __syncthreads();
+      // four vectors at a time: their Y values are fetched before their first store (loads and stores
+      // share one in-order counter)
+#pragma unroll
+      for (int g = 0; g < 2; g++) {
+        f4 o[4], yv[HAS_Y ? 4 : 1];
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+          const int q1hi = 2 * g + (k >> 1), rr = k & 1;
+          const int row = (q1hi * 2 + rr) * 16 + w;
+          const f4 v = *(const f4*)&lds[row * 256 + ((l * 4) ^ (w * 4))];
+          f4 p;                                           // word e of v is column 4l + (e ^ q1hi)
+          p[0] = v[0 ^ q1hi]; p[1] = v[1 ^ q1hi]; p[2] = v[2 ^ q1hi]; p[3] = v[3 ^ q1hi];
+          o[k] = p;
+          if (HAS_Y) yv[k] = *(const f4*)(Y + (4 * q1hi + 2 * h + rr) * 4096 + w * 256 + l * 4);
+        }
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+          const int q1hi = 2 * g + (k >> 1), rr = k & 1;
+          const int col = (4 * q1hi + 2 * h + rr) * 4096 + w * 256 + l * 4;
+          f4 v = o[k];
+          if (a.epilogue) {
+            v = v * alpha;
+            if (HAS_Y) v = v + yv[k] * beta;
+          }
+          *(f4*)(Z + col) = v;
+        }
+      }
+    }
+    FK_STAMP(4);
+    __syncthreads();      // every wave has read its last LDS word before the next item's stage 1 writes
+    FK_STAMP(5);
   }
-  FK_STAMP(5);
-#ifdef FK_ROW_TIMING
-  if (tid == 0 && blockIdx.x < 1024) g_rowTiming[blockIdx.x * 8 + 7] = wall_clock64();
-#endif
 }
 
 // Rows per workgroup: 16^(4-nf).
@@ -242,7 +298,7 @@ bool row16x4Supported(const StepArgs& a) {
 hipError_t launchRow16x4(const StepArgs& a, hipStream_t stream) {
   if (!row16x4Supported(a)) return hipErrorInvalidValue;
   static bool attrSet = false;
-  const size_t ldsBytes = kLdsWords * sizeof(float);
+  const size_t ldsBytes = (kLdsWords + 4 * 256) * sizeof(float);
   if (!attrSet) {
     hipError_t e = hipFuncSetAttribute((const void*)kron_row16x4_kernel<true>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes);
@@ -252,25 +308,29 @@ hipError_t launchRow16x4(const StepArgs& a, hipStream_t stream) {
     if (e != hipSuccess) return e;
     attrSet = true;
   }
-  dim3 grid(a.M / row16Rows(a), a.batch), block(1024);
   static int cus = 0;
-  static uint32_t groups = 3, delay = 20000;           // three start groups, 20000 cycles (about 9 us) apart
+  static uint32_t groups = 1, delay = 0;               // start stagger off by default (measured: no gain once the next item is prefetched)
   if (!cus) {
     int dev = 0;
     hipDeviceProp_t prop;
     if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) cus = prop.multiProcessorCount;
     else cus = 256;
-    if (const char* e = getenv("FASTKRON_ROW_STAGGER")) {   // "<groups>,<ticks>" for experiments
+    if (const char* e = getenv("FASTKRON_ROW_STAGGER")) {   // "<groups>,<cycles>" for experiments
       unsigned g = 0, d = 0;
       if (sscanf(e, "%u,%u", &g, &d) == 2) { groups = g; delay = d; }
     }
   }
-  const uint32_t firstWave = (uint32_t)cus;
-  const uint32_t g = ((uint64_t)grid.x * a.batch > (uint64_t)cus) ? groups : 1;   // a single wave of rows gains nothing
+  const uint32_t blocksPerBatch = a.M / row16Rows(a);
+  const uint64_t total = (uint64_t)blocksPerBatch * a.batch;
+  if (total >= (1ull << 32)) return hipErrorInvalidValue;
+  // persistent workgroups, one per CU; a single wave of items gains nothing from the start stagger
+  const uint32_t wgs = total < (uint64_t)cus ? (uint32_t)total : (uint32_t)cus;
+  const uint32_t g = (total > (uint64_t)cus) ? groups : 1;
+  dim3 grid(wgs), block(1024);
   if (a.y && a.epilogue)
-    hipLaunchKernelGGL(kron_row16x4_kernel<true>, grid, block, ldsBytes, stream, a, firstWave, g, delay);
+    hipLaunchKernelGGL(kron_row16x4_kernel<true>, grid, block, ldsBytes, stream, a, blocksPerBatch, (uint32_t)total, g, delay);
   else
-    hipLaunchKernelGGL(kron_row16x4_kernel<false>, grid, block, ldsBytes, stream, a, firstWave, g, delay);
+    hipLaunchKernelGGL(kron_row16x4_kernel<false>, grid, block, ldsBytes, stream, a, blocksPerBatch, (uint32_t)total, g, delay);
   return hipGetLastError();
 }
 

@@ -44,7 +44,22 @@ __global__ __launch_bounds__(512, 4) void kron_row32x16x3_kernel(const StepArgs 
   const float* F2p = (const float*)a.f[1] + (size_t)bt * a.f_batch[1];
   const float* F1p = (const float*)a.f[2] + (size_t)bt * a.f_batch[2];
 
-  // Y first (8 values per lane, in the store layout): on gfx9 loads and stores share one in-order
+  // factor operands: first product B_c[k][j] = F2[4c+k][j]; second product B_{h,r}[k][j] = F3[16h+4k+r][j]
+  float FA[8], FB[2][4];
+#pragma unroll
+  for (int c = 0; c < 8; c++) FA[c] = F2p[(int64_t)(4 * c + hi) * a.f_sp[1] + (int64_t)lo * a.f_sq[1]];
+#pragma unroll
+  for (int h = 0; h < 2; h++)
+#pragma unroll
+    for (int r = 0; r < 4; r++)
+      FB[h][r] = F3p[(int64_t)(16 * h + 4 * hi + r) * a.f_sp[0] + (int64_t)lo * a.f_sq[0]];
+  // (the small factor loads go out before the row data: vector memory operations retire in order)
+
+  float FC[8];
+#pragma unroll
+  for (int c = 0; c < 8; c++) FC[c] = F1p[(int64_t)(4 * c + hi) * a.f_sp[2] + (int64_t)lo * a.f_sq[2]];
+
+  // Y next (8 values per lane, in the store layout): on gfx9 loads and stores share one in-order
   // counter, so a load issued after a store could only be waited for together with that store.
   const float* Y = HAS_Y ? (const float*)a.y + (size_t)bt * a.y_batch + (size_t)m * a.y_ldm : nullptr;
   float yv[2][4];
@@ -66,16 +81,6 @@ __global__ __launch_bounds__(512, 4) void kron_row32x16x3_kernel(const StepArgs 
 #pragma unroll
         for (int h = 0; h < 2; h++) x[g][h][c] = xp[g * 1024 + c * 128 + h * 16];
   }
-
-  // factor operands: first product B_c[k][j] = F2[4c+k][j]; second product B_{h,r}[k][j] = F3[16h+4k+r][j]
-  float FA[8], FB[2][4];
-#pragma unroll
-  for (int c = 0; c < 8; c++) FA[c] = F2p[(int64_t)(4 * c + hi) * a.f_sp[1] + (int64_t)lo * a.f_sq[1]];
-#pragma unroll
-  for (int h = 0; h < 2; h++)
-#pragma unroll
-    for (int r = 0; r < 4; r++)
-      FB[h][r] = F3p[(int64_t)(16 * h + 4 * hi + r) * a.f_sp[0] + (int64_t)lo * a.f_sq[0]];
 
   // ---- stage 1 ----
   float y[4][4];
@@ -114,11 +119,7 @@ __global__ __launch_bounds__(512, 4) void kron_row32x16x3_kernel(const StepArgs 
     for (int c = 0; c < 8; c++) z[bq][c] = lds[q2 * 512 + ((((4 * c + hi) << 4) | lo) ^ ((q2 >> 2) << 4))];
   }
 
-  // ---- stage 2: D[i = q1][j = q3] = sum_k1 F1[k1][q1] * z[k1][q3]; A_c[i][k] = F1[4c+k][i] ----
-  float FC[8];
-#pragma unroll
-  for (int c = 0; c < 8; c++) FC[c] = F1p[(int64_t)(4 * c + hi) * a.f_sp[2] + (int64_t)lo * a.f_sq[2]];
-
+  // ---- stage 2: D[i = q1][j = q3] = sum_k1 F1[k1][q1] * z[k1][q3]; A_c[i][k] = F1[4c+k][i] (FC, loaded up front) ----
   const float alpha = (float)a.alpha, beta = (float)a.beta;
 #pragma unroll
   for (int bq = 0; bq < 2; bq++) {

@@ -97,16 +97,8 @@ __global__ __launch_bounds__(512, 4) void kron_row8x5_kernel(const StepArgs a) {
   float* Z = (float*)a.out + (size_t)bt * a.out_batch + (size_t)m * kRow8Len;
 
   FK8_STAMP(0); FK8_STAMP(6);
-  // ---- load: x[k1][k2] = X[k1][k2][k3 = w][(k4,k5) = l] ----
-  float x[8][8];
-  {
-    const float* xp = X + w * 64 + l;
-#pragma unroll
-    for (int i = 0; i < 8; i++)
-#pragma unroll
-      for (int j = 0; j < 8; j++) x[i][j] = xp[i * 4096 + j * 512];
-  }
-  // factors to LDS (a.f[0] is the last factor F5 ... a.f[nf-1] the first).  With fewer than five
+  // factors to LDS, ahead of the row loads (vector memory operations retire in order, so these small
+  // loads must not queue behind 128 KB of row data).  a.f[0] is the last factor F5 ... a.f[nf-1] the first.  With fewer than five
   // factors the leading digits are row indices (8^(5-nf) consecutive rows form the same contiguous
   // 32768-element block) and their factor slots hold the identity.
   if (tid < 320) {
@@ -118,6 +110,16 @@ __global__ __launch_bounds__(512, 4) void kron_row8x5_kernel(const StepArgs a) {
       v = fp[(int64_t)p * a.f_sp[j] + (int64_t)q * a.f_sq[j]];
     }
     fl[tid] = v;
+  }
+  // ---- load: x[k1][k2] = X[k1][k2][k3 = w][(k4,k5) = l]; k2 outermost, so the slices of the first
+  //      contraction (all k1 for one k2) complete in issue order ----
+  float x[8][8];
+  {
+    const float* xp = X + w * 64 + l;
+#pragma unroll
+    for (int j = 0; j < 8; j++)
+#pragma unroll
+      for (int i = 0; i < 8; i++) x[i][j] = xp[i * 4096 + j * 512];
   }
   __syncthreads();
 
