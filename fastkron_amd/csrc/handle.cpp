@@ -174,21 +174,22 @@ fastKronError Handle::xgemm(KronProblem p, fastKronBackend backend, void* temp1,
 // on a K_A x T matrix whose T columns are contiguous.  Two or three launches instead of N.  The layout
 // between the two parts is [row][k_A][q_B] (digits in place), which only these two sub-problems see.
 fastKronError Handle::trySplitLeadingTrailing(const KronProblem& p, void* temp1, void* temp2) {
-  if (p.mm != MMType::MKM || p.dt != DType::F32 || p.forward || p.opX != fastKronOp_N) return fastKronKernelNotFound;
+  if (p.mm != MMType::MKM || p.forward || p.opX != fastKronOp_N) return fastKronKernelNotFound;
   if (!temp1 || !temp2 || p.N < 3) return fastKronKernelNotFound;
-  // trailing run of identical 8x8 (at most 5) or 16x16 (at most 4) factors
+  // trailing run of identical square factors that one whole-row kernel fuses:
+  // fp32 8x8 (five) or 16x16 (four); fp64 32x32 or 64x64 (two)
   const uint32_t tp = p.P[p.N - 1];
-  if ((tp != 8 && tp != 16) || p.Q[p.N - 1] != tp) return fastKronKernelNotFound;
-  const uint32_t maxT = (tp == 8) ? 5 : 4;
+  if (p.Q[p.N - 1] != tp) return fastKronKernelNotFound;
+  uint32_t maxT = 0;
+  if (p.dt == DType::F32) maxT = (tp == 8) ? 5 : (tp == 16) ? 4 : 0;
+  else                    maxT = (tp == 32 || tp == 64) ? 2 : 0;
+  if (maxT == 0) return fastKronKernelNotFound;
   uint32_t nT = 0;
   while (nT < maxT && nT < p.N && p.P[p.N - 1 - nT] == tp && p.Q[p.N - 1 - nT] == tp) nT++;
   if (nT != maxT || nT == p.N) return fastKronKernelNotFound;      // shorter chains are whole-row problems already
   const uint32_t g = p.N - nT;
   const uint32_t lp = p.P[0];
-  if (lp != 4 && lp != 8 && lp != 16) return fastKronKernelNotFound;
   for (uint32_t i = 0; i < g; i++) if (p.P[i] != lp || p.Q[i] != lp) return fastKronKernelNotFound;
-  const uint32_t perLaunch = (lp == 4) ? 3 : (lp == 8) ? 2 : 1;
-  if (g > 2 * perLaunch) return fastKronKernelNotFound;             // the KMM part may use temp2 only
   uint64_t KA = 1, T = 1;
   for (uint32_t i = 0; i < g; i++) KA *= lp;
   for (uint32_t i = 0; i < nT; i++) T *= tp;

@@ -85,7 +85,8 @@ static bool row32Check(const KernelInfo&, const StepArgs& a) { return row32x16x3
 // ---- single-factor MFMA step (fp64 and fp32) ----
 static bool stepF64CanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
                           const DeviceInfo& dev) {
-  if (p.dt != k.dt || p.mm != MMType::MKM || lo != hi) return false;
+  const MMType mm = (k.variant == 1) ? MMType::KMM : MMType::MKM;
+  if (p.dt != k.dt || p.mm != mm || lo != hi) return false;
   if (p.P[lo] != k.P || p.Q[lo] != k.Q) return false;
   if (first && p.opX == 2) return false;
   (void)dev;
@@ -93,6 +94,28 @@ static bool stepF64CanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo
 }
 static hipError_t stepF64Launch(const KernelInfo& k, const StepArgs& a, hipStream_t s) { return launchStepMfma(a, k.dt, s); }
 static bool stepF64Check(const KernelInfo& k, const StepArgs& a) { return stepMfmaSupported(a, k.dt); }
+
+// ---- two fused square fp64 factors covering whole rows ----
+static bool pairCanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
+                       const DeviceInfo& dev) {
+  if (p.dt != DType::F64 || p.mm != MMType::MKM || hi - lo + 1 != 2 || p.forward) return false;
+  for (uint32_t i = lo; i <= hi; i++) if (p.P[i] != k.P || p.Q[i] != k.Q) return false;
+  if (p.colsBefore(hi) != (uint64_t)k.P * k.P) return false;
+  if (first && p.opX == 2) return false;
+  return dev.ldsPerBlock >= (int)(2 * k.P * k.P * 8);
+}
+static hipError_t pairLaunch(const KernelInfo&, const StepArgs& a, hipStream_t s) { return launchPairMfma(a, s); }
+static bool pairCheck(const KernelInfo&, const StepArgs& a) { return pairMfmaSupported(a); }
+
+// ---- KMM-layout step with a 64x64 fp64 factor ----
+static bool kmm64CanRun(const KernelInfo&, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
+                        const DeviceInfo&) {
+  if (p.dt != DType::F64 || p.mm != MMType::KMM || lo != hi || p.P[lo] != 64 || p.Q[lo] != 64) return false;
+  if (first && p.opX == 2) return false;
+  return p.M % 64 == 0;
+}
+static hipError_t kmm64Launch(const KernelInfo&, const StepArgs& a, hipStream_t s) { return launchKmm64F64(a, s); }
+static bool kmm64Check(const KernelInfo&, const StepArgs& a) { return kmm64F64Supported(a); }
 
 // ---- KMM-layout register kernel: NF fused PxP fp32 factors with P^NF = 64 ----
 static bool kmmRegCanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
@@ -139,13 +162,35 @@ void registerRowKernels(std::vector<KernelInfo>& out) {
     out.push_back(kk);
   }
 
+  for (uint32_t P : {64u, 32u}) {
+    KernelInfo kp{};
+    const std::string ps = std::to_string(P);
+    kp.name = "mkm_hip_gfx950_256_d_" + ps + "x" + ps + "_" + ps + "x" + ps + "_2_1x" + std::to_string(P * P) +
+              (P == 64 ? "_mfma4x4x4" : "_mfma16x16x4") + "_NN_strided_0_3";
+    kp.dt = DType::F64; kp.P = P; kp.Q = P; kp.fused = 2; kp.tileM = 1; kp.tileK = P * P; kp.threads = 256; kp.variant = 0;
+    kp.canRun = pairCanRun; kp.launch = pairLaunch; kp.check = pairCheck;
+    out.push_back(kp);
+  }
+
+  {
+    KernelInfo kk{};
+    kk.name = "kmm_hip_gfx950_256_d_64x64_64x64_1_64x64_mfma4x4x4_NN_strided_0_3";
+    kk.dt = DType::F64; kk.P = 64; kk.Q = 64; kk.fused = 1; kk.tileM = 64; kk.tileK = 64; kk.threads = 256; kk.variant = 2;
+    kk.canRun = kmm64CanRun; kk.launch = kmm64Launch; kk.check = kmm64Check;
+    out.push_back(kk);
+  }
+
+  // variant 1 = the same kernel on the KMM layout (tiles of 16 consecutive m)
+  for (uint32_t variant : {0u, 1u})
   for (DType dt : {DType::F64, DType::F32})
   for (uint32_t P : {16u, 32u, 64u, 128u}) {
     KernelInfo kd{};
     const std::string ps = std::to_string(P);
-    kd.name = std::string("mkm_hip_gfx950_256_") + (dt == DType::F64 ? "d_" : "f_") + ps + "x" + ps + "_" + ps + "x" + ps + "_1_1x" + std::to_string(16 * P) +
+    kd.name = std::string(variant ? "kmm" : "mkm") + "_hip_gfx950_256_" + (dt == DType::F64 ? "d_" : "f_") + ps + "x" + ps +
+              "_" + ps + "x" + ps + "_1_" + (variant ? "16x" + ps : "1x" + std::to_string(16 * P)) +
               "_mfma16x16x4_NN_strided_0_3";
-    kd.dt = dt; kd.P = P; kd.Q = P; kd.fused = 1; kd.tileM = 1; kd.tileK = 16 * P; kd.threads = 256; kd.variant = 0;
+    kd.dt = dt; kd.P = P; kd.Q = P; kd.fused = 1; kd.tileM = variant ? 16 : 1; kd.tileK = variant ? P : 16 * P;
+    kd.threads = 256; kd.variant = variant;
     kd.canRun = stepF64CanRun; kd.launch = stepF64Launch; kd.check = stepF64Check;
     out.push_back(kd);
   }

@@ -20,9 +20,17 @@ hipError_t launchRow8x5(const StepArgs& a, hipStream_t stream);
 bool row32x16x3Supported(const StepArgs& a);
 hipError_t launchRow32x16x3(const StepArgs& a, hipStream_t stream);
 
-// One step with a 16x16 / 32x32 / 64x64 factor on the matrix cores, fp64 or fp32 (MKM layout).
+// Two fused 32x32 or 64x64 fp64 factors on rows of exactly P*P columns (MKM layout), one wave per row.
+bool pairMfmaSupported(const StepArgs& a);
+hipError_t launchPairMfma(const StepArgs& a, hipStream_t stream);
+
+// One step with a 16x16 ... 128x128 factor on the matrix cores, fp64 or fp32, MKM or KMM layout.
 bool stepMfmaSupported(const StepArgs& a, DType dt);
 hipError_t launchStepMfma(const StepArgs& a, DType dt, hipStream_t stream);
+
+// One step with a 64x64 fp64 factor on the KMM layout (4x4x4 matrix-core instruction, 64-column tiles).
+bool kmm64F64Supported(const StepArgs& a);
+hipError_t launchKmm64F64(const StepArgs& a, hipStream_t stream);
 
 // KMM layout, fp32: three fused 4x4 or two fused 8x8 factors held in registers, lanes along M.
 bool kmmRegSupported(const StepArgs& a);

@@ -1,0 +1,411 @@
+// Two fused square fp64 factors (P = Q in {32, 64}) on rows of exactly P*P columns, MKM layout, on the
+// matrix cores (V_MFMA_F64_16X16X4_F64): Z = X (F_b x F_a) with one read of X and one write of Z.  Serves
+// dgemkm with two such factors directly and, on "virtual rows" (every contiguous block of P*P columns of a
+// longer row), the trailing two factors of longer chains; the leading factors are then applied across the
+// blocks by the KMM-layout step kernel.
+//
+//   out[q_b*P + q_a] = sum_{k_b, k_a} in[k_b*P + k_a] * F_a[k_a, q_a] * F_b[k_b, q_b]
+//
+// A wave owns one row (a P x P tile, 32 KB for P = 64) at a time; no exchange through LDS is needed
+// because the accumulator layout of the first product is an operand layout of the second:
+//   * product 1, D1[k_b][q_a] = sum_{k_a} X[k_b][k_a] F_a[k_a][q_a]: X is the A operand (lane = 16*k + k_b,
+//     contraction index k_a = (P/4)*k + c, so a lane reads P/4 consecutive doubles of its row), F_a the B
+//     operand from LDS.  D1 sits at register k_b/4, lane 16*(k_b%4) + q_a;
+//   * product 2, D2[q_b][q_a] = sum_{k_b} F_b^T[q_b][k_b] D1[k_b][q_a]: register r of D1 *is* a B operand
+//     (lane = 16*k' + q_a) for the contraction indices k_b = 16*g + 4*r + k'; F_b^T comes from LDS as the
+//     A operand.  D2 sits at register q_b/4, lane 16*(q_b%4) + q_a: a quarter wave stores 16 consecutive
+//     doubles (one 128-byte line).
+// Both factors are staged in LDS once per workgroup.  Workgroups are persistent, one per CU with one wave
+// per SIMD: that leaves a wave 512 registers, enough to hold the next row (128 registers for P = 64) while
+// the current one is multiplied, so memory and matrix pipe overlap inside every wave.
+// alpha / beta*Y are applied in the store when this launch writes Z.
+//
+//
+// The 64x64 case is bound by the matrix pipe, and V_MFMA_F64_4X4X4_4B_F64 sustains about 1.5 times the rate
+// of the 16x16x4 instruction on this device, so 64x64 has its own kernel built on it (kron_pair64_f64_kernel;
+// the chained-product kernel above serves 32x32, which is bound by memory).  One instruction multiplies four
+// independent 4x4x4 blocks; the blocks are four neighbouring groups of four output columns q_a, so the
+// factor operand is used as stored and the other operand is the same for the four blocks:
+//   * product 1: A = X[k_b = 4t+i][k_a = 16k+c], the same for every block: read from LDS (the wave stages 16
+//     rows of its tile at a time there) with four lanes per address; B = F_a[16k+c][16g+4blk+j], also from
+//     LDS.  D1[t][g] sits at lane 16*(k_b%4) + q_a%16;
+//   * product 2: that register is the B operand for the contraction indices k_b = 4t+k; A = F_b[4t+k][4u+i]
+//     comes from LDS, again one address per four lanes.  D2 sits at lane 16*(q_b%4) + q_a%16: a quarter wave
+//     stores 16 consecutive doubles.
+// Every LDS read feeds four products (two reads per four products in product 1).  Waves work independently
+// (no barrier after the factors are staged), two per SIMD - the instruction only reaches its rate with two
+// waves issuing - which leaves a wave 256 registers: 128 for D1, 32 for the quarter tile in flight.
+//
+// Role of the reference's fused shared-memory kernel (reference src/kernels/cuda/kernel.cuh:53-224 with
+// FusedFacs = 2, CUDA cores only); the chained matrix-core products are specific to this kernel.
+// Algorithmic traffic per launch: read M*P*P, write M*P*P elements (+ M*P*P for Y).
+#include <hip/hip_runtime.h>
+#include "../problem.h"
+#include "launch.h"
+
+namespace fk {
+
+typedef double pd4 __attribute__((ext_vector_type(4)));
+typedef double pd2 __attribute__((ext_vector_type(2)));
+
+constexpr int kPairWaves = 4;
+
+template <int P, bool HAS_Y>
+__global__ __launch_bounds__(256, 1) void kron_pair_f64_kernel(const StepArgs a) {
+  constexpr int PB = P / 16;             // 16-wide blocks per digit
+  constexpr int PC = P / 4;              // products per block of product 1, doubles per lane and row
+  extern __shared__ double pairLds[];
+  double* fA = pairLds;                  // F_a[k_a][q_a], row-major P x P
+  double* fB = pairLds + P * P;          // F_b[k_b][q_b]
+  const int tid = threadIdx.x;
+  const int l0 = tid & 63;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const uint32_t bt = blockIdx.y;
+
+  const double* inB = (const double*)a.in + (size_t)bt * a.in_batch;
+  double* outB = (double*)a.out + (size_t)bt * a.out_batch;
+  const double* YB = HAS_Y ? (const double*)a.y + (size_t)bt * a.y_batch : nullptr;
+  const double alpha = a.alpha, beta = a.beta;
+
+  {
+    const double* Fa = (const double*)a.f[0] + (size_t)bt * a.f_batch[0];
+    const double* Fb = (const double*)a.f[1] + (size_t)bt * a.f_batch[1];
+    for (int i = tid; i < P * P; i += 256) {
+      const int p = i / P, q = i % P;
+      fA[i] = Fa[(int64_t)p * a.f_sp[0] + (int64_t)q * a.f_sq[0]];
+      fB[i] = Fb[(int64_t)p * a.f_sp[1] + (int64_t)q * a.f_sq[1]];
+    }
+  }
+  __syncthreads();
+
+  const uint32_t stride = gridDim.x * kPairWaves;
+  auto loadRow = [&](uint32_t row, double (&x)[PB][PC]) {
+    const int lo = l0 & 15, hi = l0 >> 4;
+    const double* xp = inB + (size_t)row * a.in_ldm + lo * P + PC * hi;
+#pragma unroll
+    for (int g = 0; g < PB; g++)
+#pragma unroll
+      for (int c = 0; c < PC; c += 2) {
+        const pd2 v = *(const pd2*)(xp + g * 16 * P + c);
+        x[g][c] = v[0]; x[g][c + 1] = v[1];
+      }
+  };
+
+  auto computeRow = [&](uint32_t row, const double (&x)[PB][PC]) {
+    // the lane id is made opaque once per row so that the LDS reads below (the same for every row) are
+    // not hoisted out of the loop into registers
+    int l = l0;
+    asm volatile("" : "+v"(l));
+    const int lo = l & 15, hi = l >> 4;
+    double* out = outB + (size_t)row * a.out_ldm;
+    const double* Y = HAS_Y ? YB + (size_t)row * a.y_ldm : nullptr;
+
+#pragma unroll 1
+    for (int jb = 0; jb < PB; jb++) {
+      int ofs = 16 * jb + lo;
+      asm volatile("" : "+v"(ofs));
+      pd4 d1[PB];
+#pragma unroll
+      for (int g = 0; g < PB; g++) d1[g] = (pd4){0, 0, 0, 0};
+#pragma unroll
+      for (int c = 0; c < PC; c++) {
+        const double b = fA[(PC * hi + c) * P + ofs];
+#pragma unroll
+        for (int g = 0; g < PB; g++) d1[g] = __builtin_amdgcn_mfma_f64_16x16x4f64(x[g][c], b, d1[g], 0, 0, 0);
+      }
+      // two independent accumulator chains at a time keep the matrix pipe full with one wave per SIMD
+#pragma unroll
+      for (int jb2 = 0; jb2 < PB; jb2 += 2) {
+        pd4 acc[2] = {(pd4){0, 0, 0, 0}, (pd4){0, 0, 0, 0}};
+#pragma unroll
+        for (int g = 0; g < PB; g++)
+#pragma unroll
+          for (int r = 0; r < 4; r++)
+#pragma unroll
+            for (int u = 0; u < 2; u++) {
+              const double fa = fB[(16 * g + 4 * r + hi) * P + 16 * (jb2 + u) + lo];
+              acc[u] = __builtin_amdgcn_mfma_f64_16x16x4f64(fa, d1[g][r], acc[u], 0, 0, 0);
+            }
+        double yv[2][4];
+        if (HAS_Y) {
+#pragma unroll
+          for (int u = 0; u < 2; u++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) yv[u][r] = Y[(16 * (jb2 + u) + hi + 4 * r) * P + ofs];
+        }
+#pragma unroll
+        for (int u = 0; u < 2; u++)
+#pragma unroll
+          for (int r = 0; r < 4; r++) {               // q_b = 16*(jb2+u) + 4*r + hi, q_a = 16*jb + lo
+            double v = acc[u][r];
+            if (a.epilogue) {
+              v *= alpha;
+              if (HAS_Y) v += beta * yv[u][r];
+            }
+            out[(16 * (jb2 + u) + hi + 4 * r) * P + ofs] = v;
+          }
+      }
+    }
+  };
+
+  // register double buffer over rows: the next row streams in under the products of the current one
+  uint32_t row = blockIdx.x * kPairWaves + w;
+  double xa[PB][PC], xb[PB][PC];
+  if (row < a.M) loadRow(row, xa);
+  while (row < a.M) {
+    if (row + stride < a.M) loadRow(row + stride, xb);
+    computeRow(row, xa);
+    row += stride;
+    if (row >= a.M) break;
+    if (row + stride < a.M) loadRow(row + stride, xa);
+    computeRow(row, xb);
+    row += stride;
+  }
+}
+
+
+constexpr int kP64 = 64;
+constexpr int kPair64Waves = 8;                     // one workgroup of 8 waves per CU, two waves per SIMD
+constexpr int kPair64XWords = 16 * 64;              // doubles of X staging per wave: 16 rows of the tile
+constexpr size_t kPair64LdsBytes = (2 * kP64 * kP64 + kPair64Waves * kPair64XWords) * sizeof(double);
+
+template <bool HAS_Y>
+__global__ __launch_bounds__(512, 2) void kron_pair64_f64_kernel(const StepArgs a) {
+  constexpr int P = kP64;
+  extern __shared__ double pairLds[];
+  double* fA = pairLds;                              // F_a[k_a][q_a], row-major
+  double* fB = pairLds + P * P;                      // F_b[k_b][q_b] at k_b*64 + (q_b ^ 4*(k_b%4))
+  const int tid = threadIdx.x;
+  const int l0 = tid & 63;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  double* xs = pairLds + 2 * P * P + w * kPair64XWords;   // this wave's X staging
+  const uint32_t bt = blockIdx.y;
+
+  const double* inB = (const double*)a.in + (size_t)bt * a.in_batch;
+  double* outB = (double*)a.out + (size_t)bt * a.out_batch;
+  const double* YB = HAS_Y ? (const double*)a.y + (size_t)bt * a.y_batch : nullptr;
+  // multiplying by 1.0 is exact: launches that do not write Z need no branch around the scaling
+  const double alpha = a.epilogue ? a.alpha : 1.0, beta = a.beta;
+
+  {
+    const double* Fa = (const double*)a.f[0] + (size_t)bt * a.f_batch[0];
+    const double* Fb = (const double*)a.f[1] + (size_t)bt * a.f_batch[1];
+    for (int i = tid; i < P * P; i += 512) {
+      const int p = i / P, q = i % P;
+      fA[i] = Fa[(int64_t)p * a.f_sp[0] + (int64_t)q * a.f_sq[0]];
+      fB[p * P + (q ^ (4 * (p & 3)))] = Fb[(int64_t)p * a.f_sp[1] + (int64_t)q * a.f_sq[1]];
+    }
+  }
+  __syncthreads();
+
+  const uint32_t stride = gridDim.x * kPair64Waves;
+  // lane l holds, of the 16 rows of a part, the doubles (j*64 + l)*2 + {0, 1}, j = 0..7.  One part (a
+  // quarter of the tile) is in flight at a time: it is requested when the part before it has been written
+  // to LDS, and arrives under that part's products (part 0 of the next tile under all of product 2).
+  pd2 x[8];
+  auto loadPart = [&](uint32_t row, int tb) {
+    const double* xp = inB + (size_t)row * a.in_ldm + 2 * l0 + tb * 1024;
+#pragma unroll
+    for (int j = 0; j < 8; j++) x[j] = *(const pd2*)(xp + j * 128);
+  };
+
+  auto computeRow = [&](uint32_t row, uint32_t next) {
+    // the lane id is made opaque once per row: the LDS reads of the factors are the same for every row and
+    // must not be hoisted out of the loop into registers
+    int l = l0;
+    asm volatile("" : "+v"(l));
+    const int i4 = l & 3, k4 = l >> 4, n16 = l & 15;  // operand lane = i + 4*blk + 16*k = n + 16*k
+    double* out = outB + (size_t)row * a.out_ldm;
+    const double* Y = HAS_Y ? YB + (size_t)row * a.y_ldm : nullptr;
+
+    // staging position of element (r, col) of a 16-row part: r*64 + 16*k + ((c + 4*(r%4) + k) % 16),
+    // col = 16*k + c: the 16 addresses (i, k) of one operand read fall into 16 different bank pairs
+    const int wr = l >> 5, wk = (l & 31) >> 3, wc = 2 * (l & 7);
+    double d1[16][4];
+#pragma unroll
+    for (int tb = 0; tb < 4; tb++) {
+#pragma unroll
+      for (int j = 0; j < 8; j++) {
+        const int r = 2 * j + wr;
+#pragma unroll
+        for (int e = 0; e < 2; e++) xs[r * 64 + 16 * wk + ((wc + e + 4 * (r & 3) + wk) & 15)] = x[j][e];
+      }
+      if (tb < 3) loadPart(row, tb + 1); else loadPart(next, 0);
+#pragma unroll
+      for (int tt = 0; tt < 4; tt++)
+#pragma unroll
+        for (int g = 0; g < 4; g++) d1[4 * tb + tt][g] = 0.0;
+      // operands of step c+1 are read before the products of step c are issued
+      double an[4], bn[4];
+#pragma unroll
+      for (int tt = 0; tt < 4; tt++) an[tt] = xs[(4 * tt + i4) * 64 + 16 * k4 + ((4 * i4 + k4) & 15)];
+#pragma unroll
+      for (int g = 0; g < 4; g++) bn[g] = fA[(16 * k4) * 64 + 16 * g + n16];
+#pragma unroll
+      for (int c = 0; c < 16; c++) {
+        double ac[4], bc[4];
+#pragma unroll
+        for (int tt = 0; tt < 4; tt++) { ac[tt] = an[tt]; bc[tt] = bn[tt]; }
+        if (c + 1 < 16) {
+#pragma unroll
+          for (int tt = 0; tt < 4; tt++) an[tt] = xs[(4 * tt + i4) * 64 + 16 * k4 + ((c + 1 + 4 * i4 + k4) & 15)];
+#pragma unroll
+          for (int g = 0; g < 4; g++) bn[g] = fA[(16 * k4 + c + 1) * 64 + 16 * g + n16];
+        }
+        asm volatile("" ::: "memory");
+#pragma unroll
+        for (int tt = 0; tt < 4; tt++)
+#pragma unroll
+          for (int g = 0; g < 4; g++)
+            d1[4 * tb + tt][g] = __builtin_amdgcn_mfma_f64_4x4x4f64(ac[tt], bc[g], d1[4 * tb + tt][g], 0, 0, 0);
+      }
+    }
+
+    const int orow = l >> 4, ocol = l & 15;         // result lane = 16*(q_b%4) + q_a%16
+    // fully unrolled, so that the 64 stores of a row are counted when the next row waits for its
+    // prefetched part (see the note on the peeled first row)
+#pragma unroll
+    for (int ub = 0; ub < 4; ub++) {
+      // F_b[4t + k][16ub + 4uu + i] at (4t + k)*64 + 16ub + 4*(uu ^ k) + i
+      int fo[4];
+#pragma unroll
+      for (int uu = 0; uu < 4; uu++) {
+        fo[uu] = k4 * 64 + 16 * ub + 4 * (uu ^ k4) + i4;
+        asm volatile("" : "+v"(fo[uu]));
+      }
+      double acc[4][4];
+#pragma unroll
+      for (int uu = 0; uu < 4; uu++)
+#pragma unroll
+        for (int g = 0; g < 4; g++) acc[uu][g] = 0.0;
+      double fn[4];
+#pragma unroll
+      for (int uu = 0; uu < 4; uu++) fn[uu] = fB[fo[uu]];
+#pragma unroll
+      for (int t = 0; t < 16; t++) {
+        double fc[4];
+#pragma unroll
+        for (int uu = 0; uu < 4; uu++) fc[uu] = fn[uu];
+        if (t + 1 < 16) {
+#pragma unroll
+          for (int uu = 0; uu < 4; uu++) fn[uu] = fB[fo[uu] + 4 * (t + 1) * 64];
+        }
+        asm volatile("" ::: "memory");
+#pragma unroll
+        for (int uu = 0; uu < 4; uu++)
+#pragma unroll
+          for (int g = 0; g < 4; g++)
+            acc[uu][g] = __builtin_amdgcn_mfma_f64_4x4x4f64(fc[uu], d1[t][g], acc[uu][g], 0, 0, 0);
+      }
+      const int o0 = (16 * ub + orow) * 64 + ocol;   // q_b = 16ub + 4uu + orow, q_a = 16g + ocol
+      // Y in two halves, each read before the stores of its half (registers are short with Y)
+#pragma unroll
+      for (int uh = 0; uh < 4; uh += 2) {
+        double yv[2][4];
+        if (HAS_Y) {
+#pragma unroll
+          for (int uu = 0; uu < 2; uu++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) yv[uu][g] = Y[o0 + 4 * (uh + uu) * 64 + 16 * g];
+        }
+#pragma unroll
+        for (int uu = 0; uu < 2; uu++)
+#pragma unroll
+          for (int g = 0; g < 4; g++) {
+            double v = acc[uh + uu][g] * alpha;
+            if (HAS_Y) v += beta * yv[uu][g];
+            out[o0 + 4 * (uh + uu) * 64 + 16 * g] = v;
+          }
+      }
+    }
+  };
+
+  uint32_t row = blockIdx.x * kPair64Waves + w;
+  if (row >= a.M) return;
+  // the last row of a wave prefetches its own first part again: no branch around memory operations
+  auto nextOf = [&](uint32_t r) { return r + stride < a.M ? r + stride : r; };
+  loadPart(row, 0);
+  // The first row is peeled off the loop.  Loads and stores retire through one in-order counter and
+  // the wait for a prefetched part is counted in younger operations; entering the loop only from a
+  // complete row lets that count include the 64 stores issued behind the prefetch, so that the wait
+  // at the top of a row does not drain the previous row's stores.
+  computeRow(row, nextOf(row));
+  for (row += stride; row < a.M; row += stride) computeRow(row, nextOf(row));
+}
+
+bool pairMfmaSupported(const StepArgs& a) {
+  if (a.nf != 2) return false;
+  const uint32_t P = a.p[0];
+  if ((P != 64 && P != 32) || a.q[0] != P || a.p[1] != P || a.q[1] != P) return false;
+  if (a.Kin != (uint64_t)P * P || a.Kout != a.Kin) return false;
+  if (a.in_ldc != 1 || a.out_ldc != 1 || (a.y && a.y_ldc != 1)) return false;
+  if (((uintptr_t)a.in & 15) || (a.in_ldm & 1) || (a.in_batch & 1)) return false;      // 128-bit loads
+  return a.batch <= 65535;
+}
+
+template <int P>
+static hipError_t launchPairT(const StepArgs& a, hipStream_t stream) {
+  static int cus = 0;
+  if (!cus) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    cus = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+              ? prop.multiProcessorCount : 256;
+  }
+  const size_t ldsBytes = 2 * P * P * sizeof(double);
+  uint32_t wgs = (uint32_t)cus * (P == 64 ? 1 : 3);     // the 32x32 kernel needs a third of the registers
+  if (a.batch > 1) wgs = (wgs + a.batch - 1) / a.batch;
+  const uint32_t need = (a.M + kPairWaves - 1) / kPairWaves;
+  if (wgs > need) wgs = need;
+  if (wgs == 0) wgs = 1;
+  dim3 grid(wgs, a.batch), block(256);
+  static bool attr[2] = {false, false};
+  const bool y = a.y && a.epilogue;
+  if (!attr[y]) {
+    hipError_t e = y ? hipFuncSetAttribute((const void*)kron_pair_f64_kernel<P, true>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes)
+                     : hipFuncSetAttribute((const void*)kron_pair_f64_kernel<P, false>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes);
+    if (e != hipSuccess) return e;
+    attr[y] = true;
+  }
+  if (y) hipLaunchKernelGGL((kron_pair_f64_kernel<P, true>), grid, block, ldsBytes, stream, a);
+  else   hipLaunchKernelGGL((kron_pair_f64_kernel<P, false>), grid, block, ldsBytes, stream, a);
+  return hipGetLastError();
+}
+
+static hipError_t launchPair64(const StepArgs& a, hipStream_t stream) {
+  static int cus = 0;
+  if (!cus) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    cus = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+              ? prop.multiProcessorCount : 256;
+  }
+  uint32_t wgs = (uint32_t)cus;                     // persistent, one workgroup per CU
+  if (a.batch > 1) wgs = (wgs + a.batch - 1) / a.batch;
+  const uint32_t need = (a.M + kPair64Waves - 1) / kPair64Waves;
+  if (wgs > need) wgs = need;
+  if (wgs == 0) wgs = 1;
+  dim3 grid(wgs, a.batch), block(64 * kPair64Waves);
+  static bool attr[2] = {false, false};
+  const bool y = a.y && a.epilogue;
+  if (!attr[y]) {
+    hipError_t e = y ? hipFuncSetAttribute((const void*)kron_pair64_f64_kernel<true>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)kPair64LdsBytes)
+                     : hipFuncSetAttribute((const void*)kron_pair64_f64_kernel<false>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)kPair64LdsBytes);
+    if (e != hipSuccess) return e;
+    attr[y] = true;
+  }
+  if (y) hipLaunchKernelGGL((kron_pair64_f64_kernel<true>), grid, block, kPair64LdsBytes, stream, a);
+  else   hipLaunchKernelGGL((kron_pair64_f64_kernel<false>), grid, block, kPair64LdsBytes, stream, a);
+  return hipGetLastError();
+}
+
+hipError_t launchPairMfma(const StepArgs& a, hipStream_t stream) {
+  if (!pairMfmaSupported(a)) return hipErrorInvalidValue;
+  return a.p[0] == 64 ? launchPair64(a, stream) : launchPairT<32>(a, stream);
+}
+
+}  // namespace fk

@@ -51,7 +51,11 @@ constexpr int kStepWaves = 4;            // waves per workgroup
 
 // QS > 1 splits the Q output columns of a tile over QS wave tasks (each keeps only its Q/QS columns of
 // the factor in registers); used for 128x128, whose factor does not fit the register file of one wave.
-template <typename T, int P, int Q, int QS, bool HAS_Y>
+//
+// KMM = true is the same step on the KMM layout (element (m, col) at m + col*M, the M index contiguous): a
+// tile is then 16 consecutive m of one slice, the B operand lane 16*k + m reads in[(s*P + p)*M + m] (16
+// consecutive elements per quarter wave and product), and the stores are the same 16-element runs.
+template <typename T, int P, int Q, int QS, bool HAS_Y, bool KMM>
 __global__ __launch_bounds__(256, 2) void kron_step_mfma_kernel(const StepArgs a, const uint32_t tilesPerRow,
                                                                 const uint32_t totalTiles) {
   using M16 = Mfma16<T>;
@@ -92,6 +96,15 @@ __global__ __launch_bounds__(256, 2) void kron_step_mfma_kernel(const StepArgs a
       fa[c][ib] = F[(int64_t)(PC * hi + c) * a.f_sp[0] + (int64_t)(q0 + 16 * ib + lo) * a.f_sq[0]];
 
   auto loadTile = [&](uint32_t t, T (&x)[PC]) {
+    if (KMM) {
+      const uint64_t s = t / tilesPerRow;
+      const uint32_t m0 = (t % tilesPerRow) * 16;
+      const uint32_t m = (m0 + lo < a.M) ? m0 + lo : m0;
+      const T* xp = inB + m + (s * P + PC * hi) * (uint64_t)a.in_ldc;
+#pragma unroll
+      for (int c = 0; c < PC; c++) x[c] = xp[(uint64_t)c * a.in_ldc];
+      return;
+    }
     const uint32_t m = t / tilesPerRow;
     const uint64_t s0 = (uint64_t)(t % tilesPerRow) * 16;
     const uint64_t s = (s0 + lo < S) ? s0 + lo : s0;
@@ -120,24 +133,38 @@ __global__ __launch_bounds__(256, 2) void kron_step_mfma_kernel(const StepArgs a
 #pragma unroll
       for (int ib = 0; ib < NB; ib++) acc[ib] = M16::mma(fa[c][ib], x[c], acc[ib]);
 
-    const uint32_t m = t / tilesPerRow;
-    const uint64_t s = (uint64_t)(t % tilesPerRow) * 16 + lo;
-    if (s >= S) continue;
-    T* out = outB + (size_t)m * a.out_ldm;
-    const T* Y = HAS_Y ? YB + (size_t)m * a.y_ldm : nullptr;
+    // element (q, tile lane) of the output lives at out + q*qStride (+ the lane's own offset, in `out`)
+    T* out;
+    const T* Y = nullptr;
+    uint64_t qStride, yStride = 0;
+    if (KMM) {
+      const uint64_t s = t / tilesPerRow;
+      const uint32_t m = (t % tilesPerRow) * 16 + lo;
+      if (m >= a.M) continue;
+      out = outB + m + s * (uint64_t)a.out_ldc;
+      qStride = S * (uint64_t)a.out_ldc;
+      if (HAS_Y) { Y = YB + m + s * (uint64_t)a.y_ldc; yStride = S * (uint64_t)a.y_ldc; }
+    } else {
+      const uint32_t m = t / tilesPerRow;
+      const uint64_t s = (uint64_t)(t % tilesPerRow) * 16 + lo;
+      if (s >= S) continue;
+      out = outB + (size_t)m * a.out_ldm + s;
+      qStride = S;
+      if (HAS_Y) { Y = YB + (size_t)m * a.y_ldm + s; yStride = S; }
+    }
     // all Y loads of the tile before its first store (loads and stores share one in-order counter)
     T yv[HAS_Y ? NB : 1][4];
     if (HAS_Y) {
 #pragma unroll
       for (int ib = 0; ib < NB; ib++)
 #pragma unroll
-        for (int r = 0; r < 4; r++) yv[ib][r] = Y[(uint64_t)(q0 + 16 * ib + M16::row(r, hi)) * S + s];
+        for (int r = 0; r < 4; r++) yv[ib][r] = Y[(uint64_t)(q0 + 16 * ib + M16::row(r, hi)) * yStride];
     }
 #pragma unroll
     for (int ib = 0; ib < NB; ib++)
 #pragma unroll
       for (int r = 0; r < 4; r++) {
-        const uint64_t col = (uint64_t)(q0 + 16 * ib + M16::row(r, hi)) * S + s;
+        const uint64_t col = (uint64_t)(q0 + 16 * ib + M16::row(r, hi)) * qStride;
         T v = acc[ib][r];
         if (a.epilogue) {
           v *= alpha;
@@ -148,16 +175,23 @@ __global__ __launch_bounds__(256, 2) void kron_step_mfma_kernel(const StepArgs a
   }
 }
 
+// KMM layout: the M index is the contiguous one (and there is more than one row)
+static bool stepMfmaIsKmm(const StepArgs& a) { return a.in_ldm == 1 && a.in_ldc != 1; }
+
 bool stepMfmaSupported(const StepArgs& a, DType dt) {
   if (a.nf != 1) return false;
   const uint32_t P = a.p[0], Q = a.q[0];
   if (!((P == 128 && Q == 128) || (P == 64 && Q == 64) || (P == 32 && Q == 32) || (P == 16 && Q == 16))) return false;
-  if (a.in_ldc != 1 || a.out_ldc != 1 || (a.y && a.y_ldc != 1)) return false;
   if (a.Kin % P) return false;
+  const uint64_t S = a.Kin / P;
+  if (stepMfmaIsKmm(a)) {
+    if (a.out_ldm != 1 || (a.y && a.y_ldm != 1)) return false;
+    return S * ((a.M + 15) / 16) < (1ull << 31) && a.batch <= 65535;
+  }
+  if (a.in_ldc != 1 || a.out_ldc != 1 || (a.y && a.y_ldc != 1)) return false;
   // 16-byte alignment of every slice for the 128-bit loads
   const uint64_t vmask = 16 / dtypeSize(dt) - 1;
   if (((uintptr_t)a.in & 15) || ((uint64_t)a.in_ldm & vmask) || (a.in_batch & vmask)) return false;
-  const uint64_t S = a.Kin / P;
   const uint64_t tiles = (S + 15) / 16;
   return tiles * a.M < (1ull << 31) && a.batch <= 65535;
 }
@@ -165,8 +199,9 @@ bool stepMfmaSupported(const StepArgs& a, DType dt) {
 template <typename T, int P, int Q, int QS>
 static hipError_t launchStepMfmaT(const StepArgs& a, hipStream_t stream) {
   const uint64_t S = a.Kin / P;
-  const uint32_t tilesPerRow = (uint32_t)((S + 15) / 16);
-  const uint32_t totalTiles = tilesPerRow * a.M;
+  const bool kmm = stepMfmaIsKmm(a);
+  const uint32_t tilesPerRow = kmm ? (a.M + 15) / 16 : (uint32_t)((S + 15) / 16);
+  const uint32_t totalTiles = kmm ? (uint32_t)(tilesPerRow * S) : tilesPerRow * a.M;
   static int cus = 0;
   if (!cus) {
     int dev = 0;
@@ -176,16 +211,22 @@ static hipError_t launchStepMfmaT(const StepArgs& a, hipStream_t stream) {
   }
   // persistent workgroups: 2 per CU (8 waves, 2 per SIMD at up to 256 VGPRs), fewer when there is not enough work
   uint32_t wgs = (uint32_t)cus * 2;
+  if (a.batch > 1) wgs = (wgs + a.batch - 1) / a.batch;         // the batch index is the second grid dimension
+  if (wgs < (uint32_t)(QS + kStepWaves - 1) / kStepWaves) wgs = (QS + kStepWaves - 1) / kStepWaves;
   const uint32_t need = (totalTiles * QS + kStepWaves - 1) / kStepWaves;
   if (wgs > need) wgs = need;
   static_assert(kStepWaves % QS == 0 || QS % kStepWaves == 0, "wave tasks must tile the workgroups");
   if (QS > kStepWaves) wgs = (wgs + QS / kStepWaves - 1) / (QS / kStepWaves) * (QS / kStepWaves);
   if (wgs >= 64) wgs = wgs / 8 * 8;      // a multiple of the XCD count keeps the renumbering on
   dim3 grid(wgs, a.batch), block(256);
-  if (a.y && a.epilogue)
-    hipLaunchKernelGGL((kron_step_mfma_kernel<T, P, Q, QS, true>), grid, block, 0, stream, a, tilesPerRow, totalTiles);
-  else
-    hipLaunchKernelGGL((kron_step_mfma_kernel<T, P, Q, QS, false>), grid, block, 0, stream, a, tilesPerRow, totalTiles);
+  const bool y = a.y && a.epilogue;
+  if (kmm) {
+    if (y) hipLaunchKernelGGL((kron_step_mfma_kernel<T, P, Q, QS, true, true>), grid, block, 0, stream, a, tilesPerRow, totalTiles);
+    else   hipLaunchKernelGGL((kron_step_mfma_kernel<T, P, Q, QS, false, true>), grid, block, 0, stream, a, tilesPerRow, totalTiles);
+  } else {
+    if (y) hipLaunchKernelGGL((kron_step_mfma_kernel<T, P, Q, QS, true, false>), grid, block, 0, stream, a, tilesPerRow, totalTiles);
+    else   hipLaunchKernelGGL((kron_step_mfma_kernel<T, P, Q, QS, false, false>), grid, block, 0, stream, a, tilesPerRow, totalTiles);
+  }
   return hipGetLastError();
 }
 

@@ -206,7 +206,7 @@ def test_mfma_step_kernel(fk, M, Ps, dt):
     """Steps with 16/32/64-wide square factors run on the matrix cores (fp64 and fp32), including tiles
     with fewer than 16 slices and mixed chains."""
     check(fk, ko.MKM, M, Ps, Ps, dt, alpha=1.5, beta=0.5, seed=41)
-    assert all("mfma16x16x4" in k for _, _, k in fk.last_plan()), fk.last_plan()
+    assert all("_mfma" in k for _, _, k in fk.last_plan()), fk.last_plan()
     check(fk, ko.MKM, M, Ps, Ps, dt, alpha=1.0, beta=0.0, seed=42, opFs=ko.OP_T)
     check(fk, ko.MKM, M, Ps, Ps, dt, alpha=1.0, beta=1.0, seed=43, batch=2)
 
@@ -338,3 +338,51 @@ def test_kmm_register_kernel_more_tiles(fk, M, Ps):
     check(fk, ko.KMM, M, Ps, Ps, np.float32, alpha=1.5, beta=0.5, seed=111)
     assert all("mfma4x4x1" in k for _, _, k in fk.last_plan()), fk.last_plan()
     check(fk, ko.KMM, M, Ps, Ps, np.float32, alpha=1.0, beta=0.0, seed=112, batch=3)
+
+
+@pytest.mark.parametrize("M,P", [(1, 64), (7, 64), (64, 64), (3, 32), (50, 32)])
+def test_fp64_pair_kernel(fk, M, P):
+    """Two fused 64x64 / 32x32 fp64 factors: chained matrix-core products, one wave per row."""
+    check(fk, ko.MKM, M, [P, P], [P, P], np.float64, alpha=1.5, beta=0.5, seed=121)
+    plan = fk.last_plan()
+    assert len(plan) == 1 and f"_2_1x{P * P}_" in plan[0][2], plan
+    check(fk, ko.MKM, M, [P, P], [P, P], np.float64, alpha=1.0, beta=0.0, seed=122, opFs=ko.OP_T)
+    check(fk, ko.MKM, M, [P, P], [P, P], np.float64, alpha=1.0, beta=1.0, seed=123, batch=3)
+    check(fk, ko.MKM, M, [P, P], [P, P], np.float64, alpha=2.0, beta=0.0, seed=124, batch=2, share_f=True)
+    check(fk, ko.MKM, M, [P, P], [P, P], np.float64, alpha=1.0, beta=0.0, seed=125, integer=True)
+
+
+@pytest.mark.parametrize("M,Ps", [(2, [64] * 3), (1, [32] * 3), (3, [32] * 4), (2, [16, 64, 64]), (2, [128, 32, 32])])
+def test_fp64_chains_split_into_pair_kernel_plus_leading_kmm_step(fk, M, Ps):
+    """fp64 chains of 32- or 64-wide factors: trailing pair fused per block, leading factors as KMM-layout
+    matrix-core steps across the blocks."""
+    check(fk, ko.MKM, M, Ps, Ps, np.float64, alpha=1.5, beta=0.5, seed=131)
+    plan = fk.last_plan()
+    assert len(plan) == len(Ps) - 1 and plan[0][2].startswith("mkm_") and all(k.startswith("kmm_") for _, _, k in plan[1:]), plan
+    check(fk, ko.MKM, M, Ps, Ps, np.float64, alpha=1.0, beta=0.0, seed=132, opFs=ko.OP_T)
+    check(fk, ko.MKM, M, Ps, Ps, np.float64, alpha=1.0, beta=1.0, seed=133, batch=2, share_f=True)
+    check(fk, ko.MKM, M, Ps, Ps, np.float64, alpha=1.0, beta=1.0, seed=134, batch=2)
+
+
+@pytest.mark.parametrize("dt", [np.float64, np.float32])
+@pytest.mark.parametrize("M,Ps", [(16, [64]), (100, [32]), (37, [64, 64]), (5, [128]), (48, [16, 32]), (1000, [32, 32]),
+                                  (20, [128, 64])])
+def test_kmm_layout_mfma_step_kernel(fk, M, Ps, dt):
+    """GeKMM with 16..128-wide square factors on the matrix cores, tiles of 16 consecutive columns of X,
+    including column counts that are not a multiple of 16."""
+    check(fk, ko.KMM, M, Ps, Ps, dt, alpha=1.5, beta=0.5, seed=141)
+    assert all(k.startswith("kmm_") and "generic" not in k for _, _, k in fk.last_plan()), fk.last_plan()
+    check(fk, ko.KMM, M, Ps, Ps, dt, alpha=1.0, beta=0.0, seed=142, opFs=ko.OP_T)
+    check(fk, ko.KMM, M, Ps, Ps, dt, alpha=1.0, beta=1.0, seed=143, batch=2)
+    check(fk, ko.KMM, M, Ps, Ps, dt, alpha=1.0, beta=0.0, seed=144, integer=True)
+
+
+@pytest.mark.parametrize("M,Ps", [(64, [64]), (192, [64]), (128, [64, 64]), (64, [16, 64])])
+def test_kmm_layout_fp64_64x64_step_on_4x4x4_matrix_instruction(fk, M, Ps):
+    """dgekmm with 64x64 factors and a multiple of 64 columns of X: 64-column tiles, 4x4x4 instruction."""
+    check(fk, ko.KMM, M, Ps, Ps, np.float64, alpha=1.5, beta=0.5, seed=151)
+    assert any("mfma4x4x4" in k for _, _, k in fk.last_plan()), fk.last_plan()
+    check(fk, ko.KMM, M, Ps, Ps, np.float64, alpha=1.0, beta=0.0, seed=152, opFs=ko.OP_T)
+    check(fk, ko.KMM, M, Ps, Ps, np.float64, alpha=1.0, beta=1.0, seed=153, batch=3)
+    check(fk, ko.KMM, M, Ps, Ps, np.float64, alpha=2.0, beta=0.0, seed=154, batch=2, share_f=True)
+    check(fk, ko.KMM, M, Ps, Ps, np.float64, alpha=1.0, beta=0.0, seed=155, integer=True)
