@@ -46,7 +46,7 @@ extern "C" void fkDebugReadRowTiming(unsigned long long* out) {
 
 constexpr int kRowLen = 65536;
 constexpr int kLdsWords = 32768;           // 128 KB: one half of a row
-constexpr int kPF = 8;                     // blocks (of 16) of the next item loaded one item ahead
+constexpr int kPF = 5;                     // blocks (of 16) of the next item loaded one item ahead
 
 template <bool HAS_Y>
 __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a, const uint32_t blocksPerBatch,
@@ -103,7 +103,7 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a,
       for (int c = 0; c < 4; c++) xa[t][c] = xp[t * 256 + c * 64];
   }
 
-  for (int itn = 0; item < totalItems; item += gridDim.x, itn++) {
+  auto processItem = [&](const uint32_t item) {
     FK_STAMP(0);
     // The lane id is laundered once per item: the hundreds of lane-dependent LDS offsets below are
     // loop invariant, and hoisting them out of the item loop would pin them all in registers.
@@ -274,7 +274,14 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a,
     FK_STAMP(4);
     __syncthreads();      // every wave has read its last LDS word before the next item's stage 1 writes
     FK_STAMP(5);
-  }
+  };
+
+  // The first item is peeled off the loop.  Loads and stores retire through one in-order counter, and the
+  // wait for the prefetched blocks is counted in younger operations: entering the loop only from a complete
+  // item lets that count include the stores issued behind the prefetch, so that the wait at the top of an
+  // item does not drain the previous item's stores.
+  processItem(item);
+  for (item += gridDim.x; item < totalItems; item += gridDim.x) processItem(item);
 }
 
 // Rows per workgroup: 16^(4-nf).
