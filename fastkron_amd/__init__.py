@@ -1,9 +1,9 @@
 """fastkron_amd -- MI355X (gfx950) Kronecker-matrix multiplication behind FastKron's C API.
 
 The product is `lib/libFastKron.so` (C ABI, include/fastkron.h).  This package is the thin Python
-side: `capi` holds the ctypes declarations, `FastKron` wraps a handle, and `gemkm` / `gekmm` mirror
-the PyTorch front end of the reference (reference pyfastkron/fastkrontorch.py:404-465) for tensors
-that live in HBM.  PyTorch is used for device memory and streams only; all arithmetic happens in the
+side: `capi` holds the ctypes declarations, `FastKron` wraps a handle, and `torch_frontend` (`gemkm`,
+`gekmm`, the autograd functions `MKM` / `KMM`) mirrors the PyTorch front end of the reference (reference
+pyfastkron/fastkrontorch.py:340-465) for tensors that live in HBM.  PyTorch is used for device memory and streams only; all arithmetic happens in the
 library's HIP kernels, and a missing library or a CPU tensor is an error, never a fallback.
 """
 import ctypes
@@ -11,7 +11,7 @@ import ctypes
 from . import capi
 from .capi import (BACKEND_HIP, OP_N, OP_T, OPT_NONE, OPT_TUNE, OPT_USE_FUSION, SUCCESS)
 
-__all__ = ["FastKron", "FastKronError", "gemkm", "gekmm", "capi"]
+__all__ = ["FastKron", "FastKronError", "gemkm", "gekmm", "MKM", "KMM", "capi"]
 
 
 class FastKronError(RuntimeError):
@@ -182,52 +182,10 @@ def default_handle():
     return _default
 
 
-def _check(x, fs, y):
-    import torch
-    if not x.is_cuda:
-        raise RuntimeError("fastkron_amd runs on HBM-resident tensors only (no CPU path)")
-    for t in list(fs) + ([y] if y is not None else []):
-        if t.device != x.device or t.dtype != x.dtype:
-            raise RuntimeError("all operands must share device and dtype")
-    if x.dtype not in (torch.float32, torch.float64):
-        raise TypeError("float32 and float64 only")
-
-
-def gemkm(x, fs, alpha=1.0, beta=0.0, y=None, handle=None):
-    """z = alpha * x @ (fs[0] (x) ... (x) fs[-1]) + beta * y for 2-D x (M, prod P); fs[i] is (P_i, Q_i)."""
-    import torch
-    _check(x, fs, y)
-    h = handle or default_handle()
-    h.set_stream(torch.cuda.current_stream())
-    x = x.contiguous()
-    fs = [f.contiguous() for f in fs]
-    M = x.shape[0]
-    Ps, Qs = [f.shape[0] for f in fs], [f.shape[1] for f in fs]
-    ye, te = h.sizes(M, Ps, Qs)
-    z = torch.empty(ye, dtype=x.dtype, device=x.device)
-    t1 = torch.empty(te, dtype=x.dtype, device=x.device)
-    t2 = torch.empty(te, dtype=x.dtype, device=x.device)
-    e = h.xgemkm(M, Ps, Qs, x, fs, z, alpha, beta, y.contiguous() if y is not None else None, t1, t2)
-    if e != SUCCESS:
-        raise FastKronError(e, "gemkm")
-    return z.view(M, -1)
-
-
-def gekmm(fs, x, alpha=1.0, beta=0.0, y=None, handle=None):
-    """z = alpha * (fs[0] (x) ... (x) fs[-1]) @ x + beta * y for 2-D x (prod P, M); fs[i] is (Q_i, P_i)."""
-    import torch
-    _check(x, fs, y)
-    h = handle or default_handle()
-    h.set_stream(torch.cuda.current_stream())
-    x = x.contiguous()
-    fs = [f.contiguous() for f in fs]
-    M = x.shape[1]
-    Ps, Qs = [f.shape[1] for f in fs], [f.shape[0] for f in fs]
-    ye, te = h.sizes(M, Ps, Qs)
-    z = torch.empty(ye, dtype=x.dtype, device=x.device)
-    t1 = torch.empty(te, dtype=x.dtype, device=x.device)
-    t2 = torch.empty(te, dtype=x.dtype, device=x.device)
-    e = h.xgekmm(M, Ps, Qs, x, fs, z, alpha, beta, y.contiguous() if y is not None else None, t1, t2)
-    if e != SUCCESS:
-        raise FastKronError(e, "gekmm")
-    return z.view(-1, M)
+def __getattr__(name):
+    # gemkm / gekmm / MKM / KMM live in torch_frontend; importing them lazily keeps `import fastkron_amd`
+    # usable by hosts that only want the ctypes declarations
+    if name in ("gemkm", "gekmm", "MKM", "KMM"):
+        from . import torch_frontend
+        return getattr(torch_frontend, name)
+    raise AttributeError(f"module 'fastkron_amd' has no attribute '{name}'")
