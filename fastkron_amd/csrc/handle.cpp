@@ -130,7 +130,9 @@ fastKronError Handle::xgemm(KronProblem p, fastKronBackend backend, void* temp1,
   const std::string key = p.str();
   bool have = false;
   if (!p.forward) have = db_.lookupTuned(key, &plan);
-  if (!have && !canTune() && useFusion()) {
+  // chains longer than one whole-block kernel: the two-part plan, when the problem and the buffers allow it
+  // (the tuner only searches single chains of launches, so it is asked after this)
+  if (!have && useFusion()) {
     e = trySplitLeadingTrailing(p, temp1, temp2);
     if (e != fastKronKernelNotFound) return e;
   }

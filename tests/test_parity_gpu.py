@@ -386,3 +386,26 @@ def test_kmm_layout_fp64_64x64_step_on_4x4x4_matrix_instruction(fk, M, Ps):
     check(fk, ko.KMM, M, Ps, Ps, np.float64, alpha=1.0, beta=1.0, seed=153, batch=3)
     check(fk, ko.KMM, M, Ps, Ps, np.float64, alpha=2.0, beta=0.0, seed=154, batch=2, share_f=True)
     check(fk, ko.KMM, M, Ps, Ps, np.float64, alpha=1.0, beta=0.0, seed=155, integer=True)
+
+
+def test_tuning_tool_writes_plans_for_the_given_shapes(tmp_path, capsys):
+    """`python -m fastkron_amd.tune`: tunes each shape through the C API and keeps the plans in the file."""
+    from fastkron_amd import tune
+    db = str(tmp_path / "plans.txt")
+    assert tune.main(["--db", db, "--mmtype", "mkm", "--type", "float", "-m", "16", "32", "--same-factors", "3", "8,8"]) == 0
+    assert tune.main(["--db", db, "--mmtype", "kmm", "--type", "double", "-m", "64", "--distinct-factors", "4,4", "8,8"]) == 0
+    out = capsys.readouterr().out
+    assert out.count("GFLOP/s") == 3
+    text = open(db).read()
+    assert "16x512*(8x8^3)_NN_f" in text and "32x512*(8x8^3)_NN_f" in text and "(4x4(x)8x8)*32x64_NN_d" in text
+
+
+def test_two_part_plan_also_applies_with_tuning_enabled():
+    import fastkron_amd
+    h = fastkron_amd.FastKron(tune=True)
+    try:
+        check(h, ko.MKM, 2, [64] * 3, [64] * 3, np.float64, alpha=1.0, beta=0.0, seed=161)
+        plan = h.last_plan()
+        assert len(plan) == 2 and plan[0][2].startswith("mkm_") and plan[1][2].startswith("kmm_"), plan
+    finally:
+        h.close()
