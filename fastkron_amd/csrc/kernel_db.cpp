@@ -52,8 +52,12 @@ static bool row16CanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, 
   if (first && p.opX == 2) return false;
   return dev.ldsPerBlock >= 131072 && k.dt == p.dt;
 }
-static hipError_t row16Launch(const KernelInfo&, const StepArgs& a, hipStream_t s) { return launchRow16x4(a, s); }
-static bool row16Check(const KernelInfo&, const StepArgs& a) { return row16x4Supported(a); }
+static hipError_t row16Launch(const KernelInfo& k, const StepArgs& a, hipStream_t s) {
+  return k.threads == 512 ? launchRow16x4W8(a, s) : launchRow16x4(a, s);
+}
+static bool row16Check(const KernelInfo& k, const StepArgs& a) {
+  return k.threads == 512 ? row16x4W8Supported(a) : row16x4Supported(a);
+}
 
 // ---- whole-row kernel for five fused 8x8 fp32 factors ----
 static bool row8CanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
@@ -129,12 +133,16 @@ static hipError_t kmmRegLaunch(const KernelInfo&, const StepArgs& a, hipStream_t
 static bool kmmRegCheck(const KernelInfo&, const StepArgs& a) { return kmmRegSupported(a); }
 
 void registerRowKernels(std::vector<KernelInfo>& out) {
-  KernelInfo k{};
   // grammar: <mm>_<backend>_<arch>_<threads>_<type>_<PxQ>_<TilePxTileQ>_<fused>_<TileMxTileK>_<regs>_<ops>_<batch>_<p2p>_<opt>
-  k.name = "mkm_hip_gfx950_1024_f_16x16_16x16_4_1x65536_mfma16x16x4_NN_strided_0_3";
-  k.dt = DType::F32; k.P = 16; k.Q = 16; k.fused = 4; k.tileM = 1; k.tileK = 65536; k.threads = 1024; k.variant = 0;
-  k.canRun = row16CanRun; k.launch = row16Launch; k.check = row16Check;
-  out.push_back(k);
+  // two builds of the 16x16 whole-block kernel: 16 waves (preferred online), 8 waves with the whole next block
+  // prefetched (a candidate for the tuner)
+  for (uint32_t threads : {1024u, 512u}) {
+    KernelInfo k{};
+    k.name = "mkm_hip_gfx950_" + std::to_string(threads) + "_f_16x16_16x16_4_1x65536_mfma16x16x4_NN_strided_0_3";
+    k.dt = DType::F32; k.P = 16; k.Q = 16; k.fused = 4; k.tileM = 1; k.tileK = 65536; k.threads = threads; k.variant = 0;
+    k.canRun = row16CanRun; k.launch = row16Launch; k.check = row16Check;
+    out.push_back(k);
+  }
 
   KernelInfo k8{};
   k8.name = "mkm_hip_gfx950_512_f_8x8_8x8_5_1x32768_mfma4x4x1_NN_strided_0_3";

@@ -12,6 +12,10 @@ hipError_t launchGenericStep(const StepArgs& a, DType dt, hipStream_t stream);
 bool row16x4Supported(const StepArgs& a);
 hipError_t launchRow16x4(const StepArgs& a, hipStream_t stream);
 
+// The same with 8 waves of 128 values per lane and the whole next block prefetched.
+bool row16x4W8Supported(const StepArgs& a);
+hipError_t launchRow16x4W8(const StepArgs& a, hipStream_t stream);
+
 // Five fused 8x8 fp32 factors on rows of exactly 8^5 columns, one workgroup per row, two per CU.
 bool row8x5Supported(const StepArgs& a);
 hipError_t launchRow8x5(const StepArgs& a, hipStream_t stream);

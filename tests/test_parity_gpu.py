@@ -409,3 +409,25 @@ def test_two_part_plan_also_applies_with_tuning_enabled():
         assert len(plan) == 2 and plan[0][2].startswith("mkm_") and plan[1][2].startswith("kmm_"), plan
     finally:
         h.close()
+
+
+def test_eight_wave_build_of_the_16x16_block_kernel(tmp_path):
+    """The 8-wave build (128 values per lane, whole next block prefetched) is an alternative for the tuner; a
+    tuned-plan file naming it forces it here.  Several blocks per workgroup, Y, per-batch factors, short chains."""
+    import fastkron_amd
+    name = "mkm_hip_gfx950_512_f_16x16_16x16_4_1x65536_mfma16x16x4_NN_strided_0_3"
+    db = tmp_path / "plans.txt"
+    db.write_text("".join(f"{prob} 0.1 1 0 {n - 1} {name}\n" for prob, n in
+                          [("600x65536*(16x16^4)_NN_f", 4), ("3x65536*(16x16^4)_NN_f", 4),
+                           ("2x65536*(16x16^4)_NN_f_stridedBatched_3", 4), ("64x4096*(16x16^3)_NN_f", 3),
+                           ("512x256*(16x16^2)_NN_f", 2), ("2x65536*(16x16^4)_NT_f", 4)]))
+    h = fastkron_amd.FastKron()
+    h.set_tuned_db(str(db))
+    try:
+        for M, n, kw in [(600, 4, dict(alpha=1.0, beta=0.0)), (3, 4, dict(alpha=1.5, beta=0.5)),
+                         (2, 4, dict(alpha=1.0, beta=1.0, batch=3)), (64, 3, dict(alpha=2.0, beta=1.0)),
+                         (512, 2, dict(alpha=1.0, beta=0.0)), (2, 4, dict(alpha=1.0, beta=0.0, opFs=ko.OP_T))]:
+            check(h, ko.MKM, M, [16] * n, [16] * n, np.float32, seed=171 + M, **kw)
+            assert h.last_plan() == [(0, n - 1, name)], h.last_plan()
+    finally:
+        h.close()
