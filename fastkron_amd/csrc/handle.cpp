@@ -179,12 +179,12 @@ fastKronError Handle::trySplitLeadingTrailing(const KronProblem& p, void* temp1,
   if (p.mm != MMType::MKM || p.forward || p.opX != fastKronOp_N) return fastKronKernelNotFound;
   if (!temp1 || !temp2 || p.N < 3) return fastKronKernelNotFound;
   // trailing run of identical square factors that one whole-row kernel fuses:
-  // fp32 8x8 (five) or 16x16 (four); fp64 32x32 or 64x64 (two)
+  // fp32 8x8 (five), 16x16 (four), 32x32 or 64x64 (two); fp64 32x32 or 64x64 (two)
   const uint32_t tp = p.P[p.N - 1];
   if (p.Q[p.N - 1] != tp) return fastKronKernelNotFound;
   uint32_t maxT = 0;
-  if (p.dt == DType::F32) maxT = (tp == 8) ? 5 : (tp == 16) ? 4 : 0;
-  else                    maxT = (tp == 32 || tp == 64) ? 2 : 0;
+  if (tp == 32 || tp == 64)    maxT = 2;
+  else if (p.dt == DType::F32) maxT = (tp == 8) ? 5 : (tp == 16) ? 4 : 0;
   if (maxT == 0) return fastKronKernelNotFound;
   uint32_t nT = 0;
   while (nT < maxT && nT < p.N && p.P[p.N - 1 - nT] == tp && p.Q[p.N - 1 - nT] == tp) nT++;
@@ -224,7 +224,8 @@ fastKronError Handle::trySplitLeadingTrailing(const KronProblem& p, void* temp1,
   q2.strideZ = K; q2.strideY = K;
   q2.batch = p.batch * p.M; q2.strided = true;
   Plan plan2 = db_.selectOnline(q2, dev_, true);
-  if (plan2.size() > 2) return fastKronKernelNotFound;
+  // more than two leading launches ping-pong between temp2 and Z, which must then not be Y
+  if (plan2.size() > 2 && p.Y == p.Z && p.beta != 0.0) return fastKronKernelNotFound;
   for (auto& s : plan2) if (db_.kernels()[s.kernel].P == 0) return fastKronKernelNotFound;
   if (execute(q2, plan2, temp2, nullptr, true) != fastKronSuccess) return fastKronKernelNotFound;
 

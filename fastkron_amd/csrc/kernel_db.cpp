@@ -99,17 +99,17 @@ static bool stepF64CanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo
 static hipError_t stepF64Launch(const KernelInfo& k, const StepArgs& a, hipStream_t s) { return launchStepMfma(a, k.dt, s); }
 static bool stepF64Check(const KernelInfo& k, const StepArgs& a) { return stepMfmaSupported(a, k.dt); }
 
-// ---- two fused square fp64 factors covering whole rows ----
+// ---- two fused square factors covering whole rows ----
 static bool pairCanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
                        const DeviceInfo& dev) {
-  if (p.dt != DType::F64 || p.mm != MMType::MKM || hi - lo + 1 != 2 || p.forward) return false;
+  if (p.dt != k.dt || p.mm != MMType::MKM || hi - lo + 1 != 2 || p.forward) return false;
   for (uint32_t i = lo; i <= hi; i++) if (p.P[i] != k.P || p.Q[i] != k.Q) return false;
   if (p.colsBefore(hi) != (uint64_t)k.P * k.P) return false;
   if (first && p.opX == 2) return false;
-  return dev.ldsPerBlock >= (int)(2 * k.P * k.P * 8);
+  return dev.ldsPerBlock >= (int)(2 * k.P * k.P * 8 + 8 * 8192);
 }
-static hipError_t pairLaunch(const KernelInfo&, const StepArgs& a, hipStream_t s) { return launchPairMfma(a, s); }
-static bool pairCheck(const KernelInfo&, const StepArgs& a) { return pairMfmaSupported(a); }
+static hipError_t pairLaunch(const KernelInfo& k, const StepArgs& a, hipStream_t s) { return launchPairMfma(a, k.dt, s); }
+static bool pairCheck(const KernelInfo& k, const StepArgs& a) { return pairMfmaSupported(a, k.dt); }
 
 // ---- KMM-layout step with a 64x64 fp64 factor ----
 static bool kmm64CanRun(const KernelInfo&, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
@@ -170,12 +170,16 @@ void registerRowKernels(std::vector<KernelInfo>& out) {
     out.push_back(kk);
   }
 
+  for (DType dt : {DType::F64, DType::F32})
   for (uint32_t P : {64u, 32u}) {
     KernelInfo kp{};
     const std::string ps = std::to_string(P);
-    kp.name = "mkm_hip_gfx950_256_d_" + ps + "x" + ps + "_" + ps + "x" + ps + "_2_1x" + std::to_string(P * P) +
-              (P == 64 ? "_mfma4x4x4" : "_mfma16x16x4") + "_NN_strided_0_3";
-    kp.dt = DType::F64; kp.P = P; kp.Q = P; kp.fused = 2; kp.tileM = 1; kp.tileK = P * P; kp.threads = 256; kp.variant = 0;
+    const bool f64 = dt == DType::F64;
+    kp.name = std::string("mkm_hip_gfx950_") + (f64 && P == 64 ? "512" : "256") + (f64 ? "_d_" : "_f_") + ps + "x" + ps + "_" +
+              ps + "x" + ps + "_2_1x" + std::to_string(P * P) + (f64 && P == 64 ? "_mfma4x4x4" : "_mfma16x16x4") +
+              "_NN_strided_0_3";
+    kp.dt = dt; kp.P = P; kp.Q = P; kp.fused = 2; kp.tileM = 1; kp.tileK = P * P; kp.threads = (f64 && P == 64) ? 512 : 256;
+    kp.variant = 0;
     kp.canRun = pairCanRun; kp.launch = pairLaunch; kp.check = pairCheck;
     out.push_back(kp);
   }

@@ -24,9 +24,9 @@ hipError_t launchRow8x5(const StepArgs& a, hipStream_t stream);
 bool row32x16x3Supported(const StepArgs& a);
 hipError_t launchRow32x16x3(const StepArgs& a, hipStream_t stream);
 
-// Two fused 32x32 or 64x64 fp64 factors on rows of exactly P*P columns (MKM layout), one wave per row.
-bool pairMfmaSupported(const StepArgs& a);
-hipError_t launchPairMfma(const StepArgs& a, hipStream_t stream);
+// Two fused 32x32 or 64x64 factors (fp64 or fp32) on rows of exactly P*P columns (MKM layout), one wave per row.
+bool pairMfmaSupported(const StepArgs& a, DType dt);
+hipError_t launchPairMfma(const StepArgs& a, DType dt, hipStream_t stream);
 
 // One step with a 16x16 ... 128x128 factor on the matrix cores, fp64 or fp32, MKM or KMM layout.
 bool stepMfmaSupported(const StepArgs& a, DType dt);

@@ -1,6 +1,6 @@
-// Two fused square fp64 factors (P = Q in {32, 64}) on rows of exactly P*P columns, MKM layout, on the
-// matrix cores (V_MFMA_F64_16X16X4_F64): Z = X (F_b x F_a) with one read of X and one write of Z.  Serves
-// dgemkm with two such factors directly and, on "virtual rows" (every contiguous block of P*P columns of a
+// Two fused square factors (P = Q in {32, 64}, fp64 or fp32) on rows of exactly P*P columns, MKM layout, on the
+// matrix cores (V_MFMA_F64_16X16X4_F64 / V_MFMA_F32_16X16X4_F32): Z = X (F_b x F_a) with one read of X and one
+// write of Z.  Serves gemkm with two such factors directly and, on "virtual rows" (every contiguous block of P*P columns of a
 // longer row), the trailing two factors of longer chains; the leading factors are then applied across the
 // blocks by the KMM-layout step kernel.
 //
@@ -47,29 +47,49 @@ namespace fk {
 
 typedef double pd4 __attribute__((ext_vector_type(4)));
 typedef double pd2 __attribute__((ext_vector_type(2)));
+typedef float pf4 __attribute__((ext_vector_type(4)));
 
 constexpr int kPairWaves = 4;
 
-template <int P, bool HAS_Y>
-__global__ __launch_bounds__(256, 1) void kron_pair_f64_kernel(const StepArgs a) {
+// The 16x16x4 instruction per element type; row(r, hi) = row index, within a 16x16 accumulator, of register r
+// in the lane group hi = lane / 16 (fp64: register i/4, lane group i%4; fp32: register i%4, lane group i/4).
+template <typename T> struct PairMfma;
+template <> struct PairMfma<double> {
+  using Acc = pd4;
+  static __device__ __forceinline__ Acc mma(double a, double b, Acc c) { return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0); }
+  static __device__ __forceinline__ int row(int r, int hi) { return 4 * r + hi; }
+};
+template <> struct PairMfma<float> {
+  using Acc = pf4;
+  static __device__ __forceinline__ Acc mma(float a, float b, Acc c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
+  static __device__ __forceinline__ int row(int r, int hi) { return 4 * hi + r; }
+};
+
+template <typename T, int P, bool HAS_Y>
+__global__ __launch_bounds__(256, 2) void kron_pair_kernel(const StepArgs a) {
+  using MF = PairMfma<T>;
+  using Acc = typename MF::Acc;
   constexpr int PB = P / 16;             // 16-wide blocks per digit
-  constexpr int PC = P / 4;              // products per block of product 1, doubles per lane and row
-  extern __shared__ double pairLds[];
-  double* fA = pairLds;                  // F_a[k_a][q_a], row-major P x P
-  double* fB = pairLds + P * P;          // F_b[k_b][q_b]
+  constexpr int PC = P / 4;              // products per block of product 1, elements per lane and row
+  constexpr int VE = 16 / sizeof(T);     // elements per 128-bit load
+  typedef T VT __attribute__((ext_vector_type(VE)));
+  extern __shared__ double pairLdsRaw[];
+  T* fA = (T*)pairLdsRaw;                // F_a[k_a][q_a], row-major P x P
+  T* fB = fA + P * P;                    // F_b[k_b][q_b]
   const int tid = threadIdx.x;
   const int l0 = tid & 63;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const uint32_t bt = blockIdx.y;
 
-  const double* inB = (const double*)a.in + (size_t)bt * a.in_batch;
-  double* outB = (double*)a.out + (size_t)bt * a.out_batch;
-  const double* YB = HAS_Y ? (const double*)a.y + (size_t)bt * a.y_batch : nullptr;
-  const double alpha = a.alpha, beta = a.beta;
+  const T* inB = (const T*)a.in + (size_t)bt * a.in_batch;
+  T* outB = (T*)a.out + (size_t)bt * a.out_batch;
+  const T* YB = HAS_Y ? (const T*)a.y + (size_t)bt * a.y_batch : nullptr;
+  // multiplying by 1 is exact: launches that do not write Z need no branch around the scaling
+  const T alpha = a.epilogue ? (T)a.alpha : (T)1, beta = (T)a.beta;
 
   {
-    const double* Fa = (const double*)a.f[0] + (size_t)bt * a.f_batch[0];
-    const double* Fb = (const double*)a.f[1] + (size_t)bt * a.f_batch[1];
+    const T* Fa = (const T*)a.f[0] + (size_t)bt * a.f_batch[0];
+    const T* Fb = (const T*)a.f[1] + (size_t)bt * a.f_batch[1];
     for (int i = tid; i < P * P; i += 256) {
       const int p = i / P, q = i % P;
       fA[i] = Fa[(int64_t)p * a.f_sp[0] + (int64_t)q * a.f_sq[0]];
@@ -79,87 +99,91 @@ __global__ __launch_bounds__(256, 1) void kron_pair_f64_kernel(const StepArgs a)
   __syncthreads();
 
   const uint32_t stride = gridDim.x * kPairWaves;
-  auto loadRow = [&](uint32_t row, double (&x)[PB][PC]) {
+  auto loadRow = [&](uint32_t row, T (&x)[PB][PC]) {
     const int lo = l0 & 15, hi = l0 >> 4;
-    const double* xp = inB + (size_t)row * a.in_ldm + lo * P + PC * hi;
+    const T* xp = inB + (size_t)row * a.in_ldm + lo * P + PC * hi;
 #pragma unroll
     for (int g = 0; g < PB; g++)
 #pragma unroll
-      for (int c = 0; c < PC; c += 2) {
-        const pd2 v = *(const pd2*)(xp + g * 16 * P + c);
-        x[g][c] = v[0]; x[g][c + 1] = v[1];
+      for (int c = 0; c < PC; c += VE) {
+        const VT v = *(const VT*)(xp + g * 16 * P + c);
+#pragma unroll
+        for (int e = 0; e < VE; e++) x[g][c + e] = v[e];
       }
   };
 
-  auto computeRow = [&](uint32_t row, const double (&x)[PB][PC]) {
+  auto computeRow = [&](uint32_t row, const T (&x)[PB][PC]) {
     // the lane id is made opaque once per row so that the LDS reads below (the same for every row) are
     // not hoisted out of the loop into registers
     int l = l0;
     asm volatile("" : "+v"(l));
     const int lo = l & 15, hi = l >> 4;
-    double* out = outB + (size_t)row * a.out_ldm;
-    const double* Y = HAS_Y ? YB + (size_t)row * a.y_ldm : nullptr;
+    T* out = outB + (size_t)row * a.out_ldm;
+    const T* Y = HAS_Y ? YB + (size_t)row * a.y_ldm : nullptr;
 
 #pragma unroll 1
     for (int jb = 0; jb < PB; jb++) {
       int ofs = 16 * jb + lo;
       asm volatile("" : "+v"(ofs));
-      pd4 d1[PB];
+      Acc d1[PB];
 #pragma unroll
-      for (int g = 0; g < PB; g++) d1[g] = (pd4){0, 0, 0, 0};
+      for (int g = 0; g < PB; g++) d1[g] = (Acc){0, 0, 0, 0};
 #pragma unroll
       for (int c = 0; c < PC; c++) {
-        const double b = fA[(PC * hi + c) * P + ofs];
+        const T b = fA[(PC * hi + c) * P + ofs];
 #pragma unroll
-        for (int g = 0; g < PB; g++) d1[g] = __builtin_amdgcn_mfma_f64_16x16x4f64(x[g][c], b, d1[g], 0, 0, 0);
+        for (int g = 0; g < PB; g++) d1[g] = MF::mma(x[g][c], b, d1[g]);
       }
-      // two independent accumulator chains at a time keep the matrix pipe full with one wave per SIMD
+      // register r of d1[g] holds the rows k_b = 16g + row(r, hi): the B operand of product 2 for them;
+      // two independent accumulator chains at a time
 #pragma unroll
       for (int jb2 = 0; jb2 < PB; jb2 += 2) {
-        pd4 acc[2] = {(pd4){0, 0, 0, 0}, (pd4){0, 0, 0, 0}};
+        Acc acc[2] = {(Acc){0, 0, 0, 0}, (Acc){0, 0, 0, 0}};
 #pragma unroll
         for (int g = 0; g < PB; g++)
 #pragma unroll
           for (int r = 0; r < 4; r++)
 #pragma unroll
             for (int u = 0; u < 2; u++) {
-              const double fa = fB[(16 * g + 4 * r + hi) * P + 16 * (jb2 + u) + lo];
-              acc[u] = __builtin_amdgcn_mfma_f64_16x16x4f64(fa, d1[g][r], acc[u], 0, 0, 0);
+              const T fa = fB[(16 * g + MF::row(r, hi)) * P + 16 * (jb2 + u) + lo];
+              acc[u] = MF::mma(fa, d1[g][r], acc[u]);
             }
-        double yv[2][4];
+        T yv[2][4];
         if (HAS_Y) {
 #pragma unroll
           for (int u = 0; u < 2; u++)
 #pragma unroll
-            for (int r = 0; r < 4; r++) yv[u][r] = Y[(16 * (jb2 + u) + hi + 4 * r) * P + ofs];
+            for (int r = 0; r < 4; r++) yv[u][r] = Y[(16 * (jb2 + u) + MF::row(r, hi)) * P + ofs];
         }
 #pragma unroll
         for (int u = 0; u < 2; u++)
 #pragma unroll
-          for (int r = 0; r < 4; r++) {               // q_b = 16*(jb2+u) + 4*r + hi, q_a = 16*jb + lo
-            double v = acc[u][r];
-            if (a.epilogue) {
-              v *= alpha;
-              if (HAS_Y) v += beta * yv[u][r];
-            }
-            out[(16 * (jb2 + u) + hi + 4 * r) * P + ofs] = v;
+          for (int r = 0; r < 4; r++) {               // q_b = 16*(jb2+u) + row(r, hi), q_a = 16*jb + lo
+            T v = acc[u][r] * alpha;
+            if (HAS_Y) v += beta * yv[u][r];
+            out[(16 * (jb2 + u) + MF::row(r, hi)) * P + ofs] = v;
           }
       }
     }
   };
 
   // register double buffer over rows: the next row streams in under the products of the current one
+  // (the last row of a wave requests itself again rather than branching around the loads: a register that
+  // keeps its old value on one path would stay live on every path)
   uint32_t row = blockIdx.x * kPairWaves + w;
-  double xa[PB][PC], xb[PB][PC];
-  if (row < a.M) loadRow(row, xa);
-  while (row < a.M) {
-    if (row + stride < a.M) loadRow(row + stride, xb);
+  if (row >= a.M) return;
+  auto nextOf = [&](uint32_t r) { return r + stride < a.M ? r + stride : r; };
+  T xa[PB][PC], xb[PB][PC];
+  loadRow(row, xa);
+  while (true) {
+    loadRow(nextOf(row), xb);
     computeRow(row, xa);
     row += stride;
     if (row >= a.M) break;
-    if (row + stride < a.M) loadRow(row + stride, xa);
+    loadRow(nextOf(row), xa);
     computeRow(row, xb);
     row += stride;
+    if (row >= a.M) break;
   }
 }
 
@@ -333,17 +357,18 @@ __global__ __launch_bounds__(512, 2) void kron_pair64_f64_kernel(const StepArgs 
   for (row += stride; row < a.M; row += stride) computeRow(row, nextOf(row));
 }
 
-bool pairMfmaSupported(const StepArgs& a) {
+bool pairMfmaSupported(const StepArgs& a, DType dt) {
   if (a.nf != 2) return false;
   const uint32_t P = a.p[0];
   if ((P != 64 && P != 32) || a.q[0] != P || a.p[1] != P || a.q[1] != P) return false;
   if (a.Kin != (uint64_t)P * P || a.Kout != a.Kin) return false;
   if (a.in_ldc != 1 || a.out_ldc != 1 || (a.y && a.y_ldc != 1)) return false;
-  if (((uintptr_t)a.in & 15) || (a.in_ldm & 1) || (a.in_batch & 1)) return false;      // 128-bit loads
+  const uint64_t vmask = 16 / dtypeSize(dt) - 1;                                      // 128-bit loads
+  if (((uintptr_t)a.in & 15) || ((uint64_t)a.in_ldm & vmask) || (a.in_batch & vmask)) return false;
   return a.batch <= 65535;
 }
 
-template <int P>
+template <typename T, int P>
 static hipError_t launchPairT(const StepArgs& a, hipStream_t stream) {
   static int cus = 0;
   if (!cus) {
@@ -352,8 +377,8 @@ static hipError_t launchPairT(const StepArgs& a, hipStream_t stream) {
     cus = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
               ? prop.multiProcessorCount : 256;
   }
-  const size_t ldsBytes = 2 * P * P * sizeof(double);
-  uint32_t wgs = (uint32_t)cus * (P == 64 ? 1 : 3);     // the 32x32 kernel needs a third of the registers
+  const size_t ldsBytes = 2 * P * P * sizeof(T);
+  uint32_t wgs = (uint32_t)cus * (P == 32 ? 4 : 2);   // persistent; the 32x32 kernels need few registers
   if (a.batch > 1) wgs = (wgs + a.batch - 1) / a.batch;
   const uint32_t need = (a.M + kPairWaves - 1) / kPairWaves;
   if (wgs > need) wgs = need;
@@ -362,15 +387,15 @@ static hipError_t launchPairT(const StepArgs& a, hipStream_t stream) {
   static bool attr[2] = {false, false};
   const bool y = a.y && a.epilogue;
   if (!attr[y]) {
-    hipError_t e = y ? hipFuncSetAttribute((const void*)kron_pair_f64_kernel<P, true>,
+    hipError_t e = y ? hipFuncSetAttribute((const void*)kron_pair_kernel<T, P, true>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes)
-                     : hipFuncSetAttribute((const void*)kron_pair_f64_kernel<P, false>,
+                     : hipFuncSetAttribute((const void*)kron_pair_kernel<T, P, false>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes);
     if (e != hipSuccess) return e;
     attr[y] = true;
   }
-  if (y) hipLaunchKernelGGL((kron_pair_f64_kernel<P, true>), grid, block, ldsBytes, stream, a);
-  else   hipLaunchKernelGGL((kron_pair_f64_kernel<P, false>), grid, block, ldsBytes, stream, a);
+  if (y) hipLaunchKernelGGL((kron_pair_kernel<T, P, true>), grid, block, ldsBytes, stream, a);
+  else   hipLaunchKernelGGL((kron_pair_kernel<T, P, false>), grid, block, ldsBytes, stream, a);
   return hipGetLastError();
 }
 
@@ -403,9 +428,10 @@ static hipError_t launchPair64(const StepArgs& a, hipStream_t stream) {
   return hipGetLastError();
 }
 
-hipError_t launchPairMfma(const StepArgs& a, hipStream_t stream) {
-  if (!pairMfmaSupported(a)) return hipErrorInvalidValue;
-  return a.p[0] == 64 ? launchPair64(a, stream) : launchPairT<32>(a, stream);
+hipError_t launchPairMfma(const StepArgs& a, DType dt, hipStream_t stream) {
+  if (!pairMfmaSupported(a, dt)) return hipErrorInvalidValue;
+  if (dt == DType::F64) return a.p[0] == 64 ? launchPair64(a, stream) : launchPairT<double, 32>(a, stream);
+  return a.p[0] == 64 ? launchPairT<float, 64>(a, stream) : launchPairT<float, 32>(a, stream);
 }
 
 }  // namespace fk

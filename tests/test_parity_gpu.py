@@ -340,28 +340,30 @@ def test_kmm_register_kernel_more_tiles(fk, M, Ps):
     check(fk, ko.KMM, M, Ps, Ps, np.float32, alpha=1.0, beta=0.0, seed=112, batch=3)
 
 
-@pytest.mark.parametrize("M,P", [(1, 64), (7, 64), (64, 64), (3, 32), (50, 32)])
-def test_fp64_pair_kernel(fk, M, P):
-    """Two fused 64x64 / 32x32 fp64 factors: chained matrix-core products, one wave per row."""
-    check(fk, ko.MKM, M, [P, P], [P, P], np.float64, alpha=1.5, beta=0.5, seed=121)
+@pytest.mark.parametrize("dt", [np.float64, np.float32])
+@pytest.mark.parametrize("M,P", [(1, 64), (7, 64), (64, 64), (3, 32), (50, 32), (2100, 32)])
+def test_pair_kernel(fk, M, P, dt):
+    """Two fused 64x64 / 32x32 factors (fp64, fp32): chained matrix-core products, one wave per row."""
+    check(fk, ko.MKM, M, [P, P], [P, P], dt, alpha=1.5, beta=0.5, seed=121)
     plan = fk.last_plan()
     assert len(plan) == 1 and f"_2_1x{P * P}_" in plan[0][2], plan
-    check(fk, ko.MKM, M, [P, P], [P, P], np.float64, alpha=1.0, beta=0.0, seed=122, opFs=ko.OP_T)
-    check(fk, ko.MKM, M, [P, P], [P, P], np.float64, alpha=1.0, beta=1.0, seed=123, batch=3)
-    check(fk, ko.MKM, M, [P, P], [P, P], np.float64, alpha=2.0, beta=0.0, seed=124, batch=2, share_f=True)
-    check(fk, ko.MKM, M, [P, P], [P, P], np.float64, alpha=1.0, beta=0.0, seed=125, integer=True)
+    check(fk, ko.MKM, M, [P, P], [P, P], dt, alpha=1.0, beta=0.0, seed=122, opFs=ko.OP_T)
+    check(fk, ko.MKM, M, [P, P], [P, P], dt, alpha=1.0, beta=1.0, seed=123, batch=3)
+    check(fk, ko.MKM, M, [P, P], [P, P], dt, alpha=2.0, beta=0.0, seed=124, batch=2, share_f=True)
+    check(fk, ko.MKM, M, [P, P], [P, P], dt, alpha=1.0, beta=0.0, seed=125, integer=True)
 
 
+@pytest.mark.parametrize("dt", [np.float64, np.float32])
 @pytest.mark.parametrize("M,Ps", [(2, [64] * 3), (1, [32] * 3), (3, [32] * 4), (2, [16, 64, 64]), (2, [128, 32, 32])])
-def test_fp64_chains_split_into_pair_kernel_plus_leading_kmm_step(fk, M, Ps):
-    """fp64 chains of 32- or 64-wide factors: trailing pair fused per block, leading factors as KMM-layout
+def test_chains_split_into_pair_kernel_plus_leading_kmm_step(fk, M, Ps, dt):
+    """Chains of 32- or 64-wide factors: trailing pair fused per block, leading factors as KMM-layout
     matrix-core steps across the blocks."""
-    check(fk, ko.MKM, M, Ps, Ps, np.float64, alpha=1.5, beta=0.5, seed=131)
+    check(fk, ko.MKM, M, Ps, Ps, dt, alpha=1.5, beta=0.5, seed=131)
     plan = fk.last_plan()
     assert len(plan) == len(Ps) - 1 and plan[0][2].startswith("mkm_") and all(k.startswith("kmm_") for _, _, k in plan[1:]), plan
-    check(fk, ko.MKM, M, Ps, Ps, np.float64, alpha=1.0, beta=0.0, seed=132, opFs=ko.OP_T)
-    check(fk, ko.MKM, M, Ps, Ps, np.float64, alpha=1.0, beta=1.0, seed=133, batch=2, share_f=True)
-    check(fk, ko.MKM, M, Ps, Ps, np.float64, alpha=1.0, beta=1.0, seed=134, batch=2)
+    check(fk, ko.MKM, M, Ps, Ps, dt, alpha=1.0, beta=0.0, seed=132, opFs=ko.OP_T)
+    check(fk, ko.MKM, M, Ps, Ps, dt, alpha=1.0, beta=1.0, seed=133, batch=2, share_f=True)
+    check(fk, ko.MKM, M, Ps, Ps, dt, alpha=1.0, beta=1.0, seed=134, batch=2)
 
 
 @pytest.mark.parametrize("dt", [np.float64, np.float32])
@@ -431,3 +433,12 @@ def test_eight_wave_build_of_the_16x16_block_kernel(tmp_path):
             assert h.last_plan() == [(0, n - 1, name)], h.last_plan()
     finally:
         h.close()
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_two_part_plan_with_three_leading_launches(fk, dt):
+    """32x32^5: fused trailing pair, then three KMM-layout steps that ping-pong between the second temporary and Z
+    (not possible when Y is Z: then the chain runs as single steps)."""
+    check(fk, ko.MKM, 1, [32] * 5, [32] * 5, dt, alpha=1.5, beta=0.5, seed=181)
+    plan = fk.last_plan()
+    assert len(plan) == 4 and plan[0][2].startswith("mkm_") and all(k.startswith("kmm_") for _, _, k in plan[1:]), plan
