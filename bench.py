@@ -24,6 +24,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0            # MI355X HBM3E
 FP64_PEAK_TFLOPS = 78.6          # MI355X fp64 (vector = matrix)
+FP32_PEAK_TFLOPS = 157.3         # MI355X fp32 (vector = matrix)
 
 # name: (call, M, Ps, Qs, dtype, alpha, beta, batch, bound)
 CONFIGS = {
@@ -104,13 +105,16 @@ def cpu_baseline(M, Ps, Qs, dt, alpha, beta, batch, budget_s):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=50)
+    ap.add_argument("--ramp-seconds", type=float, default=0.25,
+                    help="untimed steps run for this long before the warm-up steps (the GPU raises its clocks over "
+                         "the first tens of milliseconds of load; steady-state throughput is what is reported)")
     ap.add_argument("--config", default="c2", choices=sorted(CONFIGS))
     ap.add_argument("--tune", action="store_true", help="time candidate launch plans first (excluded from timing)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
-    ap.add_argument("--sets", type=int, default=2, help="operand sets rotated between steps")
+    ap.add_argument("--sets", type=int, default=3, help="operand sets rotated between steps (keeps the 256 MB Infinity Cache cold)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run 4 plain device copies of 256 MiB (a known-size kernel for scaling rocprof counters)")
     args = ap.parse_args()
@@ -172,6 +176,11 @@ def main():
             dst.copy_(src)                    # reads 256 MiB, writes 256 MiB
         torch.cuda.synchronize()
 
+    t_ramp = time.perf_counter()
+    while time.perf_counter() - t_ramp < args.ramp_seconds:
+        for i in range(20):
+            step(i)
+        torch.cuda.synchronize()
     for i in range(max(args.warmup, 1)):
         step(i)
     torch.cuda.synchronize()
@@ -214,6 +223,11 @@ def main():
         achieved = flop / launches / (kernel_ms * 1e-3) / 1e12
         roof = {"bound": "mfma", "achieved": round(achieved, 2), "peak": FP64_PEAK_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(achieved / FP64_PEAK_TFLOPS, 4), "traffic": traffic}
+    # the other roof of the same run, for reference: the fraction of the matrix peak of the element type
+    # and the fraction of the HBM peak that the compulsory bytes of the whole call correspond to
+    step_s = gpu_ms / args.steps * 1e-3
+    roof["matrix_frac"] = round(flop / step_s / 1e12 / (FP32_PEAK_TFLOPS if dts == "f32" else FP64_PEAK_TFLOPS), 4)
+    roof["compulsory_hbm_frac"] = round(cbytes / step_s / 1e9 / HBM_PEAK_GBS, 4)
     roof["kernel"] = sorted(set(k for _, _, k in plan))
     roof["launches_per_step"] = launches
     roof["kernel_ms"] = round(kernel_ms, 5)

@@ -21,8 +21,6 @@
 //
 // Algorithmic traffic: 4*65536 bytes read + 4*65536 bytes written per row (+ Y when beta != 0).
 #include <hip/hip_runtime.h>
-#include <cstdio>
-#include <cstdlib>
 #include "../problem.h"
 #include "launch.h"
 
@@ -33,16 +31,6 @@ typedef float f4 __attribute__((ext_vector_type(4)));
 #define MFMA16(a, b, c) __builtin_amdgcn_mfma_f32_16x16x4f32((a), (b), (c), 0, 0, 0)
 
 
-#ifdef FK_ROW_TIMING
-// Experiment-only build: phase time stamps (s_memtime) of wave 0, [workgroup][item][phase].
-__device__ unsigned long long g_rowTiming[256 * 4 * 8];
-#define FK_STAMP(k) do { if (tid == 0 && blockIdx.x < 256 && itn < 4) g_rowTiming[(blockIdx.x * 4 + itn) * 8 + (k)] = __builtin_readcyclecounter(); } while (0)
-extern "C" void fkDebugReadRowTiming(unsigned long long* out) {
-  (void)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_rowTiming), sizeof(unsigned long long) * 256 * 4 * 8);
-}
-#else
-#define FK_STAMP(k)
-#endif
 
 constexpr int kRowLen = 65536;
 constexpr int kLdsWords = 32768;           // 128 KB: one half of a row
@@ -50,19 +38,9 @@ constexpr int kPF = 5;                     // blocks (of 16) of the next item lo
 
 template <bool HAS_Y>
 __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a, const uint32_t blocksPerBatch,
-                                                               const uint32_t totalItems, const uint32_t groups,
-                                                               const uint32_t delayCycles) {
+                                                               const uint32_t totalItems) {
   extern __shared__ float lds[];
   const int tid = threadIdx.x;
-  // One workgroup fills a CU, so every CU alternates between HBM phases (load, store) and on-chip
-  // phases (MFMA, LDS exchange).  Workgroups are persistent (one per CU, looping over row blocks);
-  // delaying a part of them at start interleaves the phases of different CUs a little.
-  if (groups > 1) {
-    const uint32_t g = (blockIdx.x >> 3) % groups;   // workgroups go round-robin over the 8 XCDs: keep every group on every XCD
-    // pure s_sleep (64 cycles per unit): polling a clock from thousands of waves would itself load the memory path
-    const uint32_t n = (g * delayCycles) >> 12;
-    for (uint32_t k = 0; k < n; k++) __builtin_amdgcn_s_sleep(64);
-  }
   const int l0 = tid & 63;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);      // wave-uniform: keeps row addresses in SGPRs
 
@@ -104,7 +82,6 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a,
   }
 
   auto processItem = [&](const uint32_t item) {
-    FK_STAMP(0);
     // The lane id is laundered once per item: the hundreds of lane-dependent LDS offsets below are
     // loop invariant, and hoisting them out of the item loop would pin them all in registers.
     int l = l0;
@@ -158,7 +135,6 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a,
       stage1(xb, 16 - kPF, kPF);
     }
 
-    FK_STAMP(1);
     // ---- exchange 1: rows (q3,q4), columns (k1,k2); half h holds the rows with bit 1 of q3 == h.
     //      Reader layout: z[u][c] = Y[k1=4c+kb][k2=i][q3=u][q4=w]. ----
     float z[16][4];
@@ -186,7 +162,6 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a,
     }
     __syncthreads();
 
-    FK_STAMP(2);
     // ---- the first half of the next item streams in from here on ----
     {
       const uint32_t nx = item + gridDim.x;
@@ -225,7 +200,6 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a,
       }
     }
 
-    FK_STAMP(3);
     // ---- exchange 2 and store, half by half.  Reader: wave w owns q2 = w, lane owns columns 4l..4l+3,
     //      register index is q1; every wave-level store covers 1 KB of contiguous columns. ----
     const float alpha = (float)a.alpha, beta = (float)a.beta;
@@ -271,9 +245,7 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a,
         }
       }
     }
-    FK_STAMP(4);
     __syncthreads();      // every wave has read its last LDS word before the next item's stage 1 writes
-    FK_STAMP(5);
   };
 
   // The first item is peeled off the loop.  Loads and stores retire through one in-order counter, and the
@@ -316,28 +288,23 @@ hipError_t launchRow16x4(const StepArgs& a, hipStream_t stream) {
     attrSet = true;
   }
   static int cus = 0;
-  static uint32_t groups = 1, delay = 0;               // start stagger off by default (measured: no gain once the next item is prefetched)
   if (!cus) {
     int dev = 0;
     hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) cus = prop.multiProcessorCount;
-    else cus = 256;
-    if (const char* e = getenv("FASTKRON_ROW_STAGGER")) {   // "<groups>,<cycles>" for experiments
-      unsigned g = 0, d = 0;
-      if (sscanf(e, "%u,%u", &g, &d) == 2) { groups = g; delay = d; }
-    }
+    cus = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+              ? prop.multiProcessorCount : 256;
   }
   const uint32_t blocksPerBatch = a.M / row16Rows(a);
   const uint64_t total = (uint64_t)blocksPerBatch * a.batch;
   if (total >= (1ull << 32)) return hipErrorInvalidValue;
-  // persistent workgroups, one per CU; a single wave of items gains nothing from the start stagger
+  // persistent workgroups, one per CU.  (Delaying a part of the workgroups at start to interleave the HBM and
+  // on-chip phases of different CUs was measured and gains nothing once the next item is prefetched.)
   const uint32_t wgs = total < (uint64_t)cus ? (uint32_t)total : (uint32_t)cus;
-  const uint32_t g = (total > (uint64_t)cus) ? groups : 1;
   dim3 grid(wgs), block(1024);
   if (a.y && a.epilogue)
-    hipLaunchKernelGGL(kron_row16x4_kernel<true>, grid, block, ldsBytes, stream, a, blocksPerBatch, (uint32_t)total, g, delay);
+    hipLaunchKernelGGL(kron_row16x4_kernel<true>, grid, block, ldsBytes, stream, a, blocksPerBatch, (uint32_t)total);
   else
-    hipLaunchKernelGGL(kron_row16x4_kernel<false>, grid, block, ldsBytes, stream, a, blocksPerBatch, (uint32_t)total, g, delay);
+    hipLaunchKernelGGL(kron_row16x4_kernel<false>, grid, block, ldsBytes, stream, a, blocksPerBatch, (uint32_t)total);
   return hipGetLastError();
 }
 

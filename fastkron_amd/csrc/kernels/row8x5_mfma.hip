@@ -31,16 +31,6 @@ typedef float f4 __attribute__((ext_vector_type(4)));
 
 #define MFMA4(a, b, c) __builtin_amdgcn_mfma_f32_4x4x1f32((a), (b), (c), 0, 0, 0)
 
-#ifdef FK_ROW_TIMING
-// Experiment-only build: phase time stamps (s_memtime) of wave 0 of every workgroup.
-__device__ unsigned long long g_row8Timing[1024 * 8];
-#define FK8_STAMP(k) do { if (tid == 0 && blockIdx.x < 1024) g_row8Timing[blockIdx.x * 8 + (k)] = (k) >= 6 ? wall_clock64() : __builtin_readcyclecounter(); } while (0)
-extern "C" void fkDebugReadRow8Timing(unsigned long long* out) {
-  (void)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_row8Timing), sizeof(unsigned long long) * 1024 * 8);
-}
-#else
-#define FK8_STAMP(k)
-#endif
 
 constexpr int kRow8Len = 32768;
 constexpr int kRow8LdsWords = 16384 + 5 * 64;     // one half row + the five factors
@@ -96,7 +86,6 @@ __global__ __launch_bounds__(512, 4) void kron_row8x5_kernel(const StepArgs a) {
   const float* X = (const float*)a.in + (size_t)bt * a.in_batch + (size_t)m * kRow8Len;
   float* Z = (float*)a.out + (size_t)bt * a.out_batch + (size_t)m * kRow8Len;
 
-  FK8_STAMP(0); FK8_STAMP(6);
   // factors to LDS, ahead of the row loads (vector memory operations retire in order, so these small
   // loads must not queue behind 128 KB of row data).  a.f[0] is the last factor F5 ... a.f[nf-1] the first.  With fewer than five
   // factors the leading digits are row indices (8^(5-nf) consecutive rows form the same contiguous
@@ -130,7 +119,6 @@ __global__ __launch_bounds__(512, 4) void kron_row8x5_kernel(const StepArgs a) {
   loadFactor8(fl + 1 * 64, l, fa);
   contractSecond(x, fa);                         // x[q1][q2], wave = k3, lane = (k4,k5)
 
-  FK8_STAMP(1);
   // ---- exchange 1: half h holds q1 in [4h, 4h+4).  Group id = (q1 & 3, q2, k3) owns 64 floats
   //      (k4,k5) stored as 16 chunks of 4, chunk index XORed with the low 4 bits of the id.  Readers:
   //      thread tid' = (q1, q2, k3) reads its 64 floats as regs [k4][k5]; waves q1>>2 == h read. ----
@@ -158,14 +146,12 @@ __global__ __launch_bounds__(512, 4) void kron_row8x5_kernel(const StepArgs a) {
   }
   // now thread = (q1 = w, q2 = l >> 3, k3 = l & 7), y[k4][k5]
 
-  FK8_STAMP(2);
   // ---- stage B: contract k5 then k4 ----
   loadFactor8(fl + 4 * 64, l, fa);
   contractSecond(y, fa);
   loadFactor8(fl + 3 * 64, l, fa);
   contractFirst(y, fa);                          // y[q4][q5]
 
-  FK8_STAMP(3);
   // ---- exchange 2: half h holds q4 in [4h, 4h+4).  Group = (q1, q2>>1, k3) owns 64 floats
   //      (q2&1, q4lo, q5) as 16 chunks, chunk index XORed with k3.  Readers: wave = q1,
   //      lane = (q2&1, q4lo, q5), regs z[k3][g], g = q4hi*4 + (q2>>1). ----
@@ -198,7 +184,6 @@ __global__ __launch_bounds__(512, 4) void kron_row8x5_kernel(const StepArgs a) {
   }
   // thread = (q1 = w, lane = (q2&1, q4lo, q5)), z[k3][g], g = q4hi*4 + (q2>>1)
 
-  FK8_STAMP(4);
   // ---- stage C: contract k3 ----
   loadFactor8(fl + 2 * 64, l, fa);
   contractFirst(z, fa);
@@ -220,7 +205,6 @@ __global__ __launch_bounds__(512, 4) void kron_row8x5_kernel(const StepArgs a) {
       }
       Z[col] = v;
     }
-  FK8_STAMP(5); FK8_STAMP(7);
 }
 
 // Rows per workgroup: 8^(5-nf).
