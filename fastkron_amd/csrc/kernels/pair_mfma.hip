@@ -28,10 +28,11 @@
 // factor operand is used as stored and the other operand is the same for the four blocks:
 //   * product 1: A = X[k_b = 4t+i][k_a = 16k+c], the same for every block: read from LDS (the wave stages 16
 //     rows of its tile at a time there) with four lanes per address; B = F_a[16k+c][16g+4blk+j], also from
-//     LDS.  D1[t][g] sits at lane 16*(k_b%4) + q_a%16;
+//     LDS.  The 16 columns of product g are q_a = 32*(g/2) + 2n + g%2 (n = lane%16), so that a lane ends up with
+//     pairs of neighbouring columns; D1[t][g] sits at lane 16*(k_b%4) + n;
 //   * product 2: that register is the B operand for the contraction indices k_b = 4t+k; A = F_b[4t+k][4u+i]
-//     comes from LDS, again one address per four lanes.  D2 sits at lane 16*(q_b%4) + q_a%16: a quarter wave
-//     stores 16 consecutive doubles.
+//     comes from LDS, again one address per four lanes.  D2 sits at lane 16*(q_b%4) + n: 16-byte stores, a
+//     quarter wave writes 32 consecutive doubles with two of them.
 // Every LDS read feeds four products (two reads per four products in product 1).  Waves work independently
 // (no barrier after the factors are staged), two per SIMD - the instruction only reaches its rate with two
 // waves issuing - which leaves a wave 256 registers: 128 for D1, 32 for the quarter tile in flight.
@@ -264,7 +265,10 @@ __global__ __launch_bounds__(512, 2) void kron_pair64_f64_kernel(const StepArgs 
 #pragma unroll
       for (int tt = 0; tt < 4; tt++) an[tt] = xs[(4 * tt + i4) * 64 + 16 * k4 + ((4 * i4 + k4) & 15)];
 #pragma unroll
-      for (int g = 0; g < 4; g++) bn[g] = fA[(16 * k4) * 64 + 16 * g + n16];
+      for (int h = 0; h < 2; h++) {
+        const pd2 v = *(const pd2*)&fA[(16 * k4) * 64 + 32 * h + 2 * n16];
+        bn[2 * h] = v[0]; bn[2 * h + 1] = v[1];
+      }
 #pragma unroll
       for (int c = 0; c < 16; c++) {
         double ac[4], bc[4];
@@ -274,7 +278,10 @@ __global__ __launch_bounds__(512, 2) void kron_pair64_f64_kernel(const StepArgs 
 #pragma unroll
           for (int tt = 0; tt < 4; tt++) an[tt] = xs[(4 * tt + i4) * 64 + 16 * k4 + ((c + 1 + 4 * i4 + k4) & 15)];
 #pragma unroll
-          for (int g = 0; g < 4; g++) bn[g] = fA[(16 * k4 + c + 1) * 64 + 16 * g + n16];
+          for (int h = 0; h < 2; h++) {
+            const pd2 v = *(const pd2*)&fA[(16 * k4 + c + 1) * 64 + 32 * h + 2 * n16];
+            bn[2 * h] = v[0]; bn[2 * h + 1] = v[1];
+          }
         }
         asm volatile("" ::: "memory");
 #pragma unroll
@@ -321,24 +328,25 @@ __global__ __launch_bounds__(512, 2) void kron_pair64_f64_kernel(const StepArgs 
           for (int g = 0; g < 4; g++)
             acc[uu][g] = __builtin_amdgcn_mfma_f64_4x4x4f64(fc[uu], d1[t][g], acc[uu][g], 0, 0, 0);
       }
-      const int o0 = (16 * ub + orow) * 64 + ocol;   // q_b = 16ub + 4uu + orow, q_a = 16g + ocol
+      // q_b = 16ub + 4uu + orow; the products g = 2h, 2h+1 hold the neighbouring columns q_a = 32h + 2*ocol, +1
+      const int o0 = (16 * ub + orow) * 64 + 2 * ocol;
       // Y in two halves, each read before the stores of its half (registers are short with Y)
 #pragma unroll
       for (int uh = 0; uh < 4; uh += 2) {
-        double yv[2][4];
+        pd2 yv[2][2];
         if (HAS_Y) {
 #pragma unroll
           for (int uu = 0; uu < 2; uu++)
 #pragma unroll
-            for (int g = 0; g < 4; g++) yv[uu][g] = Y[o0 + 4 * (uh + uu) * 64 + 16 * g];
+            for (int h = 0; h < 2; h++) yv[uu][h] = *(const pd2*)(Y + o0 + 4 * (uh + uu) * 64 + 32 * h);
         }
 #pragma unroll
         for (int uu = 0; uu < 2; uu++)
 #pragma unroll
-          for (int g = 0; g < 4; g++) {
-            double v = acc[uh + uu][g] * alpha;
-            if (HAS_Y) v += beta * yv[uu][g];
-            out[o0 + 4 * (uh + uu) * 64 + 16 * g] = v;
+          for (int h = 0; h < 2; h++) {
+            pd2 v = {acc[uh + uu][2 * h] * alpha, acc[uh + uu][2 * h + 1] * alpha};
+            if (HAS_Y) v += beta * yv[uu][h];
+            *(pd2*)(out + o0 + 4 * (uh + uu) * 64 + 32 * h) = v;
           }
       }
     }
@@ -365,6 +373,10 @@ bool pairMfmaSupported(const StepArgs& a, DType dt) {
   if (a.in_ldc != 1 || a.out_ldc != 1 || (a.y && a.y_ldc != 1)) return false;
   const uint64_t vmask = 16 / dtypeSize(dt) - 1;                                      // 128-bit loads
   if (((uintptr_t)a.in & 15) || ((uint64_t)a.in_ldm & vmask) || (a.in_batch & vmask)) return false;
+  if (dt == DType::F64 && P == 64) {                                                  // and 128-bit stores / Y loads
+    if (((uintptr_t)a.out & 15) || ((uint64_t)a.out_ldm & 1) || (a.out_batch & 1)) return false;
+    if (a.y && (((uintptr_t)a.y & 15) || ((uint64_t)a.y_ldm & 1) || (a.y_batch & 1))) return false;
+  }
   return a.batch <= 65535;
 }
 
