@@ -8,7 +8,8 @@
 // reference src/gen_tuner_kernels.py:10,366; it runs 2 launches of 2 fused factors each).  Here the
 // row (256 KB) does not fit the 160 KB LDS either, so the LDS is only the exchange buffer:
 //
-//   stage 1  contract k3 then k4 with V_MFMA_F32_16X16X4_F32, chained in registers: the first
+//   load     one 16-byte load per lane and 256-element block (k3 = lane%16, k4 = 4*(lane/16) + register)
+//   stage 1  contract k4 then k3 with V_MFMA_F32_16X16X4_F32, chained in registers: the first
 //            product leaves D[i][j] in register i%4 of lane 16*(i/4)+j, which is exactly the A-operand
 //            layout (lane 16*k+i) of a second product that contracts the *row* index i of the first;
 //            the factor operand of the second product is loaded with its rows permuted (4*k + r)
@@ -71,14 +72,14 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a,
   // An item is a block of 65536 contiguous elements: one row for four factors, 16^(4-nf) rows otherwise.
   // xa holds blocks t = 0..kPF-1 (k2) of the item about to be processed; it is loaded one item ahead, under the
   // second stage, the second exchange and the stores of the previous item.
-  float xa[kPF][4];
+  // One 16-byte load per lane and block: x[t][r] = X[k1=w][k2=t][k3=i][k4=4kb+r] (i = l%16, kb = l/16), 1 KB per
+  // wave instruction; a quarter as many memory instructions as 4-byte loads would take.
+  f4 xa[kPF];
   {
     const float* xp = (const float*)a.in + (size_t)(item / blocksPerBatch) * a.in_batch +
-                      (size_t)(item % blocksPerBatch) * kRowLen + w * 4096 + l0;
+                      (size_t)(item % blocksPerBatch) * kRowLen + w * 4096 + (l0 & 15) * 16 + (l0 >> 4) * 4;
 #pragma unroll
-    for (int t = 0; t < kPF; t++)
-#pragma unroll
-      for (int c = 0; c < 4; c++) xa[t][c] = xp[t * 256 + c * 64];
+    for (int t = 0; t < kPF; t++) xa[t] = *(const f4*)(xp + t * 256);
   }
 
   auto processItem = [&](const uint32_t item) {
@@ -95,24 +96,24 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a,
       __syncthreads();
     }
 
-    // ---- second half of the row: x[t][c] = X[k1=w][k2=t][k3=4c+kb][k4=i], t = 8..15 ----
-    float xb[16 - kPF][4];
+    // ---- the rest of the row: blocks t = kPF..15 ----
+    f4 xb[16 - kPF];
     {
-      const float* xp = X + w * 4096 + l + kPF * 256;
+      const float* xp = X + w * 4096 + i * 16 + kb * 4 + kPF * 256;
 #pragma unroll
-      for (int t = 0; t < 16 - kPF; t++)
-#pragma unroll
-        for (int c = 0; c < 4; c++) xb[t][c] = xp[t * 256 + c * 64];
+      for (int t = 0; t < 16 - kPF; t++) xb[t] = *(const f4*)(xp + t * 256);
     }
 
     // ---- stage 1: contract k3 (first product) and k4 (second product), block by block.  The half of
     //      the result with bit 1 of q3 clear goes to LDS at once, under the products of the next blocks. ----
     {
-      // first product of a chain: B_c[k][j] = F[4c + k][j]; second product: B_r[k][j] = F[4k + r][j]
+      // both products of this chain take the contraction index as 4*k + r (lane group k, instruction r): the
+      // first contracts k4, which the 16-byte loads put in the registers of a lane, the second k3, which
+      // the first leaves in the registers of its accumulator: B_r[k][j] = F[4k + r][j]
       float FA[4], FB[4];
 #pragma unroll
       for (int c = 0; c < 4; c++) {
-        FA[c] = fl[1 * 256 + (4 * c + kb) * 16 + i];      // F3
+        FA[c] = fl[1 * 256 + (4 * kb + c) * 16 + i];      // F3
         FB[c] = fl[0 * 256 + (4 * kb + c) * 16 + i];      // F4
       }
       auto stage1 = [&](auto& x, const int nt, const int t0) {
@@ -120,12 +121,13 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a,
         for (int t = 0; t < nt; t++) {
           f4 d = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-          for (int c = 0; c < 4; c++) d = MFMA16(x[t][c], FA[c], d);
+          for (int r = 0; r < 4; r++) d = MFMA16(x[t][r], FB[r], d);     // d[k3][q4]
           f4 e = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-          for (int r = 0; r < 4; r++) e = MFMA16(d[r], FB[r], e);
-#pragma unroll
-          for (int r = 0; r < 4; r++) x[t][r] = e[r];     // = Y[k1=w][k2=t0+t][q3=4kb+r][q4=i]
+          for (int r = 0; r < 4; r++) e = MFMA16(d[r], FA[r], e);        // e[q4][q3]
+          // e[r] = Y[k1=w][k2=t0+t][q4=4kb+r][q3=i]: from here to the second exchange q3 and q4 appear with their
+          // roles swapped with respect to the comments below (the first exchange treats them alike)
+          x[t] = e;
 #pragma unroll
           for (int rr = 0; rr < 2; rr++)
             lds[((kb * 2 + rr) * 16 + i) * 256 + ((w * 16 + t0 + t) ^ l)] = e[rr];
@@ -167,11 +169,9 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a,
       const uint32_t nx = item + gridDim.x;
       if (nx < totalItems) {
         const float* xp = (const float*)a.in + (size_t)(nx / blocksPerBatch) * a.in_batch +
-                          (size_t)(nx % blocksPerBatch) * kRowLen + w * 4096 + l;
+                          (size_t)(nx % blocksPerBatch) * kRowLen + w * 4096 + i * 16 + kb * 4;
 #pragma unroll
-        for (int t = 0; t < kPF; t++)
-#pragma unroll
-          for (int c = 0; c < 4; c++) xa[t][c] = xp[t * 256 + c * 64];
+        for (int t = 0; t < kPF; t++) xa[t] = *(const f4*)(xp + t * 256);
       }
     }
 
@@ -196,7 +196,7 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a,
         for (int r = 0; r < 4; r++) z[u][r] = e[r];       // = Z[q1=4kb+r][q2=i][q3=u][q4=w]
 #pragma unroll
         for (int rr = 0; rr < 2; rr++)
-          lds[((kb * 2 + rr) * 16 + i) * 256 + ((u * 16 + w) ^ (i * 4) ^ kb)] = e[rr];
+          lds[((kb * 2 + rr) * 16 + i) * 256 + ((w * 16 + u) ^ (i * 4) ^ kb)] = e[rr];   // column q3*16 + q4 = w*16 + u
       }
     }
 
@@ -213,7 +213,7 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a,
 #pragma unroll
           for (int rr = 0; rr < 2; rr++) {
             const int row = (kb * 2 + rr) * 16 + i;
-            lds[row * 256 + ((u * 16 + w) ^ (i * 4) ^ kb)] = z[u][2 + rr];
+            lds[row * 256 + ((w * 16 + u) ^ (i * 4) ^ kb)] = z[u][2 + rr];
           }
       }
       __syncthreads();
