@@ -121,6 +121,18 @@ static bool kmm64CanRun(const KernelInfo&, const KronProblem& p, uint32_t lo, ui
 static hipError_t kmm64Launch(const KernelInfo&, const StepArgs& a, hipStream_t s) { return launchKmm64F64(a, s); }
 static bool kmm64Check(const KernelInfo&, const StepArgs& a) { return kmm64F64Supported(a); }
 
+// ---- KMM layout: six fused 4x4 fp32 factors covering all 4096 rows ----
+static bool kmm4x6CanRun(const KernelInfo&, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
+                         const DeviceInfo& dev) {
+  if (p.dt != DType::F32 || p.mm != MMType::KMM || hi - lo + 1 != 6 || p.forward) return false;
+  for (uint32_t i = lo; i <= hi; i++) if (p.P[i] != 4 || p.Q[i] != 4) return false;
+  if (p.colsBefore(hi) != 4096 || p.M % 8) return false;
+  if (first && p.opX == 2) return false;
+  return dev.ldsPerBlock >= 8 * (64 * 65 + 8) * 4;
+}
+static hipError_t kmm4x6Launch(const KernelInfo&, const StepArgs& a, hipStream_t s) { return launchKmm4x6(a, s); }
+static bool kmm4x6Check(const KernelInfo&, const StepArgs& a) { return kmm4x6Supported(a); }
+
 // ---- KMM-layout register kernel: NF fused PxP fp32 factors with P^NF = 64 ----
 static bool kmmRegCanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
                          const DeviceInfo&) {
@@ -155,6 +167,14 @@ void registerRowKernels(std::vector<KernelInfo>& out) {
   k32.dt = DType::F32; k32.P = 32; k32.Q = 16; k32.fused = 3; k32.tileM = 1; k32.tileK = 32768; k32.threads = 512;
   k32.variant = 0; k32.canRun = row32CanRun; k32.launch = row32Launch; k32.check = row32Check;
   out.push_back(k32);
+
+  {
+    KernelInfo k6{};
+    k6.name = "kmm_hip_gfx950_512_f_4x4_4x4_6_8x4096_mfma4x4x1_NN_strided_0_3";
+    k6.dt = DType::F32; k6.P = 4; k6.Q = 4; k6.fused = 6; k6.tileM = 8; k6.tileK = 4096; k6.threads = 512; k6.variant = 0;
+    k6.canRun = kmm4x6CanRun; k6.launch = kmm4x6Launch; k6.check = kmm4x6Check;
+    out.push_back(k6);
+  }
 
   // deepest fusion first: the online selection takes the first kernel that fits at a given depth
   for (auto pn : {std::pair<uint32_t, uint32_t>{4, 3}, {8, 2}, {4, 2}, {4, 1}, {8, 1}, {16, 1}}) {

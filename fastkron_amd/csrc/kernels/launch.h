@@ -36,6 +36,10 @@ hipError_t launchStepMfma(const StepArgs& a, DType dt, hipStream_t stream);
 bool kmm64F64Supported(const StepArgs& a);
 hipError_t launchKmm64F64(const StepArgs& a, hipStream_t stream);
 
+// KMM layout, fp32: six fused 4x4 factors on all 4096 rows of 8 columns per workgroup (one launch for 4x4^6).
+bool kmm4x6Supported(const StepArgs& a);
+hipError_t launchKmm4x6(const StepArgs& a, hipStream_t stream);
+
 // KMM layout, fp32: three fused 4x4 or two fused 8x8 factors held in registers, lanes along M.
 bool kmmRegSupported(const StepArgs& a);
 hipError_t launchKmmReg(const StepArgs& a, hipStream_t stream);

@@ -442,3 +442,19 @@ def test_two_part_plan_with_three_leading_launches(fk, dt):
     check(fk, ko.MKM, 1, [32] * 5, [32] * 5, dt, alpha=1.5, beta=0.5, seed=181)
     plan = fk.last_plan()
     assert len(plan) == 4 and plan[0][2].startswith("mkm_") and all(k.startswith("kmm_") for _, _, k in plan[1:]), plan
+
+
+@pytest.mark.parametrize("M", [8, 72, 512])
+def test_kmm_six_4x4_factors_in_one_launch(fk, M):
+    """sgekmm with 4x4^6: one launch, every workgroup owns 8 columns and all 4096 rows of them."""
+    Ps = [4] * 6
+    check(fk, ko.KMM, M, Ps, Ps, np.float32, alpha=1.5, beta=0.5, seed=191)
+    plan = fk.last_plan()
+    assert len(plan) == 1 and "_6_8x4096_" in plan[0][2], plan
+    check(fk, ko.KMM, M, Ps, Ps, np.float32, alpha=1.0, beta=0.0, seed=192, opFs=ko.OP_T)
+    check(fk, ko.KMM, M, Ps, Ps, np.float32, alpha=1.0, beta=1.0, seed=193, batch=3)
+    check(fk, ko.KMM, M, Ps, Ps, np.float32, alpha=2.0, beta=0.0, seed=194, batch=2, share_f=True)
+    check(fk, ko.KMM, M, Ps, Ps, np.float32, alpha=1.0, beta=0.0, seed=195, integer=True, use_temp2=False)
+    # column counts that are not a multiple of 8 keep the two-launch plan
+    check(fk, ko.KMM, M + 12, Ps, Ps, np.float32, alpha=1.5, beta=0.5, seed=196)
+    assert len(fk.last_plan()) == 2, fk.last_plan()
