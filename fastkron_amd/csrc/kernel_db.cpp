@@ -128,6 +128,10 @@ static bool kmm4x6CanRun(const KernelInfo&, const KronProblem& p, uint32_t lo, u
   for (uint32_t i = lo; i <= hi; i++) if (p.P[i] != 4 || p.Q[i] != 4) return false;
   if (p.colsBefore(hi) != 4096 || p.M % 8) return false;
   if (first && p.opX == 2) return false;
+  // Only while all column tiles are resident at once (one per CU): the tiles of an XCD then walk the rows of X
+  // together and their 32-byte pieces meet in its L2.  With more tiles than CUs that order is lost and the
+  // two-launch plan, which reads 256 bytes per row and wave, is faster (measured from M = 4096 on).
+  if ((uint64_t)(p.M / 8) * p.batch > (uint64_t)dev.cus) return false;
   return dev.ldsPerBlock >= 8 * (64 * 65 + 8) * 4;
 }
 static hipError_t kmm4x6Launch(const KernelInfo&, const StepArgs& a, hipStream_t s) { return launchKmm4x6(a, s); }

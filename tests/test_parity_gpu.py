@@ -453,8 +453,11 @@ def test_kmm_six_4x4_factors_in_one_launch(fk, M):
     assert len(plan) == 1 and "_6_8x4096_" in plan[0][2], plan
     check(fk, ko.KMM, M, Ps, Ps, np.float32, alpha=1.0, beta=0.0, seed=192, opFs=ko.OP_T)
     check(fk, ko.KMM, M, Ps, Ps, np.float32, alpha=1.0, beta=1.0, seed=193, batch=3)
+    assert len(fk.last_plan()) == 1, fk.last_plan()
     check(fk, ko.KMM, M, Ps, Ps, np.float32, alpha=2.0, beta=0.0, seed=194, batch=2, share_f=True)
     check(fk, ko.KMM, M, Ps, Ps, np.float32, alpha=1.0, beta=0.0, seed=195, integer=True, use_temp2=False)
-    # column counts that are not a multiple of 8 keep the two-launch plan
+    # column counts that are not a multiple of 8, or more column tiles than CUs, keep the two-launch plan
     check(fk, ko.KMM, M + 12, Ps, Ps, np.float32, alpha=1.5, beta=0.5, seed=196)
     assert len(fk.last_plan()) == 2, fk.last_plan()
+    check(fk, ko.KMM, M, Ps, Ps, np.float32, alpha=1.0, beta=1.0, seed=197, batch=40)
+    assert len(fk.last_plan()) == (1 if M * 40 // 8 <= 256 else 2), fk.last_plan()
