@@ -1,4 +1,5 @@
 #include "handle.h"
+#include "kernels/launch.h"
 
 #include <algorithm>
 #include <cstdio>
@@ -23,7 +24,9 @@ Handle::Handle(uint32_t backends) : backends_(backends) {
   if (!dbPath_.empty()) db_.loadFile(dbPath_);
 }
 
-Handle::~Handle() {}
+Handle::~Handle() {
+  if (mergeWs_) (void)hipFree(mergeWs_);
+}
 
 void Handle::setTunedDB(const char* path) {
   dbPath_ = path ? path : "";
@@ -53,7 +56,15 @@ fastKronError Handle::initHIP(void* ptrToStream) {
   if (!hasBackend(fastKronBackend_HIP)) return fastKronBackendNotAvailable;
   stream_ = ptrToStream ? *(hipStream_t*)ptrToStream : nullptr;
   hipInit_ = true;
-  return ensureDevice();
+  fastKronError e = ensureDevice();
+  if (e != fastKronSuccess) return e;
+  // workspace for merged factors (kMaxMergeGroups products of at most 64x64 doubles); allocated here so that
+  // the gemkm / gekmm calls themselves never allocate
+  if (!mergeWs_) {
+    mergeWsBytes_ = (size_t)kMaxMergeGroups * 64 * 64 * sizeof(double);
+    if (hipMalloc(&mergeWs_, mergeWsBytes_) != hipSuccess) { mergeWs_ = nullptr; mergeWsBytes_ = 0; }
+  }
+  return fastKronSuccess;
 }
 
 fastKronError Handle::setStream(fastKronBackend backend, void* ptrToStream) {
@@ -126,6 +137,11 @@ fastKronError Handle::xgemm(KronProblem p, fastKronBackend backend, void* temp1,
   fastKronError e = ensureDevice();
   if (e != fastKronSuccess) return e;
 
+  {
+    KronProblem merged;
+    if (useFusion() && mergeSmallFactors(p, &merged)) p = merged;
+  }
+
   Plan plan;
   const std::string key = p.str();
   bool have = false;
@@ -170,6 +186,69 @@ fastKronError Handle::xgemm(KronProblem p, fastKronBackend backend, void* temp1,
   return execute(p, plan, temp1, temp2);
 }
 
+static bool isPow2(uint32_t v) { return v && !(v & (v - 1)); }
+
+bool Handle::mergeSmallFactors(const KronProblem& p, KronProblem* out) {
+  if (!mergeWs_ || p.forward || p.N < 2) return false;
+  // fp32 GeKMM already fuses small factors in registers; everything else gains from merging
+  if (p.mm == MMType::KMM && p.dt == DType::F32) return false;
+  if (p.batch > 1) for (uint32_t i = 0; i < p.N; i++) if (p.strideF[i] != 0) return false;
+  const uint32_t target = (p.dt == DType::F32) ? 16 : 64;
+  // groups of adjacent square power-of-two factors, formed from the last factor towards the first, each as
+  // large as fits the target size
+  struct Grp { uint32_t lo, hi, size; };
+  Grp grp[kMaxFactors];
+  uint32_t ng = 0, mergedGroups = 0;
+  for (int hi = (int)p.N - 1; hi >= 0;) {
+    uint32_t size = p.P[hi];
+    int lo = hi;
+    const bool small = p.P[hi] == p.Q[hi] && isPow2(p.P[hi]) && p.P[hi] < target;
+    if (small)
+      while (lo > 0 && p.P[lo - 1] == p.Q[lo - 1] && isPow2(p.P[lo - 1]) && size * p.P[lo - 1] <= target &&
+             (uint32_t)(hi - lo + 1) < kMaxMergeSources) {
+        lo--; size *= p.P[lo];
+      }
+    // a product smaller than 8 is not worth a kernel of its own size class: leave such factors alone
+    if (lo < hi && size < 8) lo = hi, size = p.P[hi];
+    grp[ng++] = Grp{(uint32_t)lo, (uint32_t)hi, size};
+    if (lo < hi) mergedGroups++;
+    hi = lo - 1;
+  }
+  if (mergedGroups == 0 || mergedGroups > kMaxMergeGroups) return false;
+
+  const bool pMajor = (p.mm == MMType::MKM) == (p.opF == fastKronOp_N);   // as in makeStepArgs
+  MergeArgs ma{};
+  KronProblem q = p;
+  q.N = ng;
+  size_t wsOff = 0;
+  for (uint32_t g = 0; g < ng; g++) {
+    const Grp& G = grp[ng - 1 - g];                    // groups were collected last to first
+    q.strideF[g] = 0;
+    if (G.lo == G.hi) {
+      q.P[g] = p.P[G.lo]; q.Q[g] = p.Q[G.lo]; q.F[g] = p.F[G.lo]; q.strideF[g] = p.strideF[G.lo];
+      continue;
+    }
+    MergeGroup& mg = ma.g[ma.groups++];
+    mg.count = G.hi - G.lo + 1;
+    for (uint32_t j = 0; j < mg.count; j++) {
+      const uint32_t fi = G.lo + j;
+      mg.src[j] = p.F[fi]; mg.p[j] = p.P[fi]; mg.q[j] = p.Q[fi];
+      mg.sp[j] = pMajor ? (int64_t)p.Q[fi] : 1;
+      mg.sq[j] = pMajor ? 1 : (int64_t)p.P[fi];
+    }
+    const size_t bytes = (size_t)G.size * G.size * dtypeSize(p.dt);
+    if (wsOff + bytes > mergeWsBytes_) return false;
+    mg.dst = (char*)mergeWs_ + wsOff;
+    mg.dsp = pMajor ? (int64_t)G.size : 1;
+    mg.dsq = pMajor ? 1 : (int64_t)G.size;
+    wsOff += (bytes + 255) & ~(size_t)255;
+    q.P[g] = G.size; q.Q[g] = G.size; q.F[g] = mg.dst;
+  }
+  if (launchMergeFactors(ma, p.dt, stream_) != hipSuccess) return false;
+  *out = q;
+  return true;
+}
+
 // X (F_0 x ... x F_{N-1}) = first apply the trailing factors B = F_g x ... x F_{N-1} to every contiguous
 // block of prod(P_g..) columns (an MKM problem on M * K_A "virtual rows", K_A = prod of the leading P), then
 // apply the leading factors A = F_0 x ... x F_{g-1} across the blocks: for every row that is a KMM problem
@@ -188,12 +267,11 @@ fastKronError Handle::trySplitLeadingTrailing(const KronProblem& p, void* temp1,
   if (maxT == 0) return fastKronKernelNotFound;
   uint32_t nT = 0;
   while (nT < maxT && nT < p.N && p.P[p.N - 1 - nT] == tp && p.Q[p.N - 1 - nT] == tp) nT++;
-  if (nT != maxT || nT == p.N) return fastKronKernelNotFound;      // shorter chains are whole-row problems already
+  if (nT < 2 || nT == p.N) return fastKronKernelNotFound;         // a chain of nT factors alone is a whole-row problem
   const uint32_t g = p.N - nT;
-  const uint32_t lp = p.P[0];
-  for (uint32_t i = 0; i < g; i++) if (p.P[i] != lp || p.Q[i] != lp) return fastKronKernelNotFound;
+  for (uint32_t i = 0; i < g; i++) if (p.P[i] != p.Q[i]) return fastKronKernelNotFound;   // square: K and L agree
   uint64_t KA = 1, T = 1;
-  for (uint32_t i = 0; i < g; i++) KA *= lp;
+  for (uint32_t i = 0; i < g; i++) KA *= p.P[i];
   for (uint32_t i = 0; i < nT; i++) T *= tp;
   const uint64_t K = KA * T;
   if (p.batch > 1) {
@@ -226,7 +304,6 @@ fastKronError Handle::trySplitLeadingTrailing(const KronProblem& p, void* temp1,
   Plan plan2 = db_.selectOnline(q2, dev_, true);
   // more than two leading launches ping-pong between temp2 and Z, which must then not be Y
   if (plan2.size() > 2 && p.Y == p.Z && p.beta != 0.0) return fastKronKernelNotFound;
-  for (auto& s : plan2) if (db_.kernels()[s.kernel].P == 0) return fastKronKernelNotFound;
   if (execute(q2, plan2, temp2, nullptr, true) != fastKronSuccess) return fastKronKernelNotFound;
 
   lastPlan_ = p.str();

@@ -45,6 +45,10 @@ class Handle {
   // M * prod(leading P) virtual rows, leading factors as a batched KMM over the row blocks.
   // Returns fastKronKernelNotFound when the problem does not have that form.
   fastKronError trySplitLeadingTrailing(const KronProblem& p, void* temp1, void* temp2);
+  // Chains of 2x2 / 4x4 (fp64: also 8x8) factors: adjacent factors are replaced by their Kronecker product
+  // (16x16 in fp32, 64x64 in fp64), computed into the handle's workspace by one small launch, so that the
+  // kernels for those sizes apply.  Returns false when nothing is merged; on true `out` is the merged problem.
+  bool mergeSmallFactors(const KronProblem& p, KronProblem* out);
 
   const std::string& lastPlan() const { return lastPlan_; }
   void setTunedDB(const char* path);
@@ -65,6 +69,8 @@ class Handle {
   std::unordered_map<std::string, Plan> planCache_;   // online selections, per problem string
   std::string dbPath_;
   std::string lastPlan_;
+  void* mergeWs_ = nullptr;                           // device memory for merged factors, allocated by initHIP
+  size_t mergeWsBytes_ = 0;
 };
 
 }  // namespace fk

@@ -44,4 +44,7 @@ hipError_t launchKmm4x6(const StepArgs& a, hipStream_t stream);
 bool kmmRegSupported(const StepArgs& a);
 hipError_t launchKmmReg(const StepArgs& a, hipStream_t stream);
 
+// Kronecker products of adjacent small factors into the handle's workspace, one workgroup per product.
+hipError_t launchMergeFactors(const MergeArgs& a, DType dt, hipStream_t stream);
+
 }  // namespace fk

@@ -75,4 +75,22 @@ struct StepArgs {
   uint32_t epilogue;                   // 1: out = alpha*acc + beta*y (beta term skipped when y is null)
 };
 
+// Merging of adjacent small factors into their Kronecker product (kernels/merge_factors.hip).
+constexpr uint32_t kMaxMergeGroups = 16;   // merged factors per call
+constexpr uint32_t kMaxMergeSources = 6;   // factors per merged factor (six 2x2 make a 64x64)
+
+struct MergeGroup {
+  const void* src[kMaxMergeSources];
+  int64_t  sp[kMaxMergeSources], sq[kMaxMergeSources];   // element (p, q) of source j at src[j] + p*sp + q*sq
+  uint32_t p[kMaxMergeSources], q[kMaxMergeSources];
+  uint32_t count;
+  void*    dst;
+  int64_t  dsp, dsq;                                     // element (p, q) of the product at dst + p*dsp + q*dsq
+};
+
+struct MergeArgs {
+  MergeGroup g[kMaxMergeGroups];
+  uint32_t groups;
+};
+
 }  // namespace fk

@@ -399,7 +399,7 @@ def test_tuning_tool_writes_plans_for_the_given_shapes(tmp_path, capsys):
     out = capsys.readouterr().out
     assert out.count("GFLOP/s") == 3
     text = open(db).read()
-    assert "16x512*(8x8^3)_NN_f" in text and "32x512*(8x8^3)_NN_f" in text and "(4x4(x)8x8)*32x64_NN_d" in text
+    assert "16x512*(8x8^3)_NN_f" in text and "32x512*(8x8^3)_NN_f" in text and "(32x32^1)*32x64_NN_d" in text   # 4x4 (x) 8x8 runs as their 32x32 product
 
 
 def test_two_part_plan_also_applies_with_tuning_enabled():
@@ -461,3 +461,31 @@ def test_kmm_six_4x4_factors_in_one_launch(fk, M):
     assert len(fk.last_plan()) == 2, fk.last_plan()
     check(fk, ko.KMM, M, Ps, Ps, np.float32, alpha=1.0, beta=1.0, seed=197, batch=40)
     assert len(fk.last_plan()) == (1 if M * 40 // 8 <= 256 else 2), fk.last_plan()
+
+
+@pytest.mark.parametrize("mm,M,Ps,dt,launches", [
+    (ko.MKM, 4, [4] * 8, np.float32, 1),          # -> 16x16^4: one whole-block launch
+    (ko.MKM, 16, [2] * 12, np.float32, 1),        # -> 16x16^3
+    (ko.MKM, 4, [4] * 7, np.float32, 2),          # -> 4, 16x16^3: block kernel on 16 virtual rows + leading 4x4
+    (ko.MKM, 3, [4] * 7, np.float32, 4),          # same, but 12 virtual rows are no whole block: single steps
+    (ko.MKM, 5, [2, 4, 2, 4, 8, 2], np.float32, None),
+    (ko.MKM, 8, [4] * 6, np.float64, 1),          # -> 64x64^2: the fp64 pair kernel
+    (ko.MKM, 2, [8] * 5, np.float64, 2),          # -> 8, 64x64^2: pair kernel + leading 8x8
+    (ko.MKM, 3, [2] * 9, np.float64, 2),          # -> 8, 64
+    (ko.KMM, 64, [4] * 6, np.float64, 2),         # -> 64x64^2 on the KMM layout
+    (ko.KMM, 20, [2] * 7, np.float64, None),
+])
+def test_small_factors_are_merged_into_their_kronecker_products(fk, mm, M, Ps, dt, launches):
+    """Adjacent 2x2 / 4x4 (fp64: 8x8) factors are replaced by their product (16x16 in fp32, 64x64 in fp64),
+    computed on the device, so that the kernels for those sizes apply."""
+    check(fk, mm, M, Ps, Ps, dt, alpha=1.5, beta=0.5, seed=201)
+    plan = fk.last_plan()
+    assert sum(hi - lo + 1 for lo, hi, _ in plan) < len(Ps), plan           # the chain that ran is shorter
+    if launches is not None:
+        assert len(plan) == launches, plan
+    check(fk, mm, M, Ps, Ps, dt, alpha=1.0, beta=0.0, seed=202, opFs=ko.OP_T)
+    check(fk, mm, M, Ps, Ps, dt, alpha=1.0, beta=1.0, seed=203, batch=2, share_f=True)
+    check(fk, mm, M, Ps, Ps, dt, alpha=1.0, beta=0.0, seed=204, integer=True)
+    # per-batch factors are not merged (one product per batch element would be needed): still correct
+    check(fk, mm, M, Ps, Ps, dt, alpha=1.0, beta=1.0, seed=205, batch=2)
+    assert sum(hi - lo + 1 for lo, hi, _ in fk.last_plan()) == len(Ps)
