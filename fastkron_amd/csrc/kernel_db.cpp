@@ -30,7 +30,38 @@ static hipError_t genericLaunch(const KernelInfo& k, const StepArgs& a, hipStrea
   return launchGenericStep(a, k.dt, s);
 }
 
+// ---- several small factors of any shape fused through LDS ----
+static bool fusedSmallCanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
+                             const DeviceInfo&) {
+  const uint32_t nf = hi - lo + 1;
+  if (k.dt != p.dt || nf < 2 || nf > kMaxFused || p.forward) return false;
+  if (first && p.opX == 2) return false;                   // input and output in the same layout only
+  // groups made of sizes that have matrix-core kernels are left to those
+  bool dedicated = true;
+  for (uint32_t i = lo; i <= hi; i++) {
+    const bool sq = p.P[i] == p.Q[i];
+    const bool mfma = sq && (p.P[i] == 16 || (p.dt == DType::F32 && p.mm == MMType::KMM && (p.P[i] == 4 || p.P[i] == 8)));
+    if (!mfma) dedicated = false;
+  }
+  if (dedicated) return false;
+  uint32_t ps[kMaxFused], qs[kMaxFused];
+  for (uint32_t j = 0; j < nf; j++) { ps[j] = p.P[hi - j]; qs[j] = p.Q[hi - j]; }
+  const bool kmm = p.mm == MMType::KMM && p.M > 1;
+  return fusedSmallFits(nf, ps, qs, p.colsBefore(hi), p.M, kmm, p.dt);
+}
+static hipError_t fusedSmallLaunch(const KernelInfo& k, const StepArgs& a, hipStream_t s) {
+  return launchFusedSmall(a, k.dt, s);
+}
+static bool fusedSmallCheck(const KernelInfo& k, const StepArgs& a) { return fusedSmallSupported(a, k.dt); }
+
 void registerGenericKernels(std::vector<KernelInfo>& out) {
+  for (DType dt : {DType::F32, DType::F64}) {
+    KernelInfo k{};
+    k.name = std::string("gekmm_hip_gfx950_512_") + (dt == DType::F32 ? "f" : "d") + "_small_fused_lds_8";
+    k.dt = dt; k.P = 1; k.Q = 1; k.fused = kMaxFused; k.tileM = 0; k.tileK = 0; k.threads = 512; k.variant = 0;
+    k.canRun = fusedSmallCanRun; k.launch = fusedSmallLaunch; k.check = fusedSmallCheck;
+    out.push_back(k);
+  }
   for (DType dt : {DType::F32, DType::F64}) {
     KernelInfo k{};
     k.name = std::string("gekmm_hip_gfx950_256_") + (dt == DType::F32 ? "f" : "d") + "_generic_1";

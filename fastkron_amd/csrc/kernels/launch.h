@@ -44,6 +44,12 @@ hipError_t launchKmm4x6(const StepArgs& a, hipStream_t stream);
 bool kmmRegSupported(const StepArgs& a);
 hipError_t launchKmmReg(const StepArgs& a, hipStream_t stream);
 
+// Several small factors of any shape (P <= 16) fused through LDS, MKM or KMM layout, fp32 or fp64.
+// fusedSmallFits: whether a group of factors (p[0], q[0] applied first) on Kin input columns has a tile.
+bool fusedSmallFits(uint32_t nf, const uint32_t* p, const uint32_t* q, uint64_t Kin, uint32_t M, bool kmm, DType dt);
+bool fusedSmallSupported(const StepArgs& a, DType dt);
+hipError_t launchFusedSmall(const StepArgs& a, DType dt, hipStream_t stream);
+
 // Kronecker products of adjacent small factors into the handle's workspace, one workgroup per product.
 hipError_t launchMergeFactors(const MergeArgs& a, DType dt, hipStream_t stream);
 

@@ -314,9 +314,9 @@ def test_row_kernels_with_fewer_factors(fk, M, Ps, tag):
 
 
 def test_row_kernels_need_whole_blocks(fk):
-    """A row count that is not a whole number of blocks takes the generic kernels instead."""
+    """A row count that is not a whole number of blocks takes the kernels without that requirement instead."""
     check(fk, ko.MKM, 12, [8] * 4, [8] * 4, np.float32, alpha=1.0, beta=0.0, seed=93)
-    assert all("generic" in k for _, _, k in fk.last_plan())
+    assert all("generic" in k or "small_fused" in k for _, _, k in fk.last_plan())
 
 
 @pytest.mark.parametrize("M,Ps", [(4, [8] * 6), (2, [8] * 7), (3, [4, 4] + [8] * 5), (2, [16] * 5), (1, [16] * 6),
@@ -467,7 +467,7 @@ def test_kmm_six_4x4_factors_in_one_launch(fk, M):
     (ko.MKM, 4, [4] * 8, np.float32, 1),          # -> 16x16^4: one whole-block launch
     (ko.MKM, 16, [2] * 12, np.float32, 1),        # -> 16x16^3
     (ko.MKM, 4, [4] * 7, np.float32, 2),          # -> 4, 16x16^3: block kernel on 16 virtual rows + leading 4x4
-    (ko.MKM, 3, [4] * 7, np.float32, 4),          # same, but 12 virtual rows are no whole block: single steps
+    (ko.MKM, 3, [4] * 7, np.float32, None),       # same, but 12 virtual rows are no whole block: shorter launches
     (ko.MKM, 5, [2, 4, 2, 4, 8, 2], np.float32, None),
     (ko.MKM, 8, [4] * 6, np.float64, 1),          # -> 64x64^2: the fp64 pair kernel
     (ko.MKM, 2, [8] * 5, np.float64, 2),          # -> 8, 64x64^2: pair kernel + leading 8x8
@@ -489,3 +489,30 @@ def test_small_factors_are_merged_into_their_kronecker_products(fk, mm, M, Ps, d
     # per-batch factors are not merged (one product per batch element would be needed): still correct
     check(fk, mm, M, Ps, Ps, dt, alpha=1.0, beta=1.0, seed=205, batch=2)
     assert sum(hi - lo + 1 for lo, hi, _ in fk.last_plan()) == len(Ps)
+
+
+FUSED_SMALL = [
+    # M, Ps, Qs                               shapes without a matrix-core kernel: several factors per launch through LDS
+    (10, [3] * 7, [3] * 7),                   # K = 2187: two launches
+    (33, [5, 3, 7, 2], [5, 3, 7, 2]),         # distinct sizes, one launch, ragged row tile
+    (5, [3, 5, 2], [4, 2, 6]),                # rectangular factors: the piece grows and shrinks between the steps
+    (3, [6] * 5, [6] * 5),                    # even, not a power of two
+    (40, [2, 3, 2, 3, 2, 3, 2, 3], [3, 2, 3, 2, 3, 2, 3, 2]),
+    (7, [13, 11, 9], [9, 11, 13]),            # P up to 16
+    (4, [3] * 10, [3] * 10),                  # reference tests/src/general-tests-NN.cpp shape family, K = 59049
+    (50, [5, 5], [2, 3]),
+]
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+@pytest.mark.parametrize("mm", [ko.MKM, ko.KMM])
+@pytest.mark.parametrize("M,Ps,Qs", FUSED_SMALL)
+def test_small_factors_of_any_shape_are_fused_through_lds(fk, mm, M, Ps, Qs, dt):
+    check(fk, mm, M, Ps, Qs, dt, alpha=1.5, beta=0.5, seed=301)
+    plan = fk.last_plan()
+    assert len(plan) < len(Ps) and any("small_fused" in k for _, _, k in plan), plan
+    check(fk, mm, M, Ps, Qs, dt, alpha=1.0, beta=0.0, seed=302, opFs=ko.OP_T)
+    check(fk, mm, M, Ps, Qs, dt, alpha=2.0, beta=1.0, seed=303, batch=3)          # per-batch factors
+    check(fk, mm, M, Ps, Qs, dt, alpha=1.0, beta=0.0, seed=304, batch=2, share_f=True)
+    if np.prod([max(p, q) for p, q in zip(Ps, Qs)]) < 50000:
+        check(fk, mm, M, Ps, Qs, dt, alpha=1.0, beta=1.0, seed=305, integer=True)
