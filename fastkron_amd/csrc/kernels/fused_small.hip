@@ -1,4 +1,4 @@
-// Several small factors of any shape (P <= 16, any Q) in one launch: the fused sliced multiply for the shapes the
+// Several small factors of any shape (P <= 8, any Q) in one launch: the fused sliced multiply for the shapes the
 // matrix-core kernels do not take (3x3, 5x5, 6x6, 7x5 ..., 2x2 where merging does not apply), MKM or KMM layout,
 // fp32 or fp64.
 //
@@ -29,7 +29,7 @@
 namespace fk {
 
 constexpr int kFsThreads = 512;
-constexpr uint32_t kFsMaxP = 16;
+constexpr uint32_t kFsMaxP = 8;             // larger factors run faster one at a time on the matrix cores
 constexpr size_t kFsBufBytes = 32768;        // per LDS buffer; two buffers: two workgroups fit a CU (measured best)
 
 struct FusedTile {
@@ -210,7 +210,6 @@ __global__ __launch_bounds__(kFsThreads, 4) void kron_fused_small_kernel(const S
 #define FS_CASE(PV) case PV: fsLocalStep<T, PV, MODE>(src, dst, F, a.f_sp[j], a.f_sq[j], a.q[j], t.A[j], t.magicA[j], nsl, t.tmShift, tid); break;
     switch (a.p[j]) {
       FS_CASE(1) FS_CASE(2) FS_CASE(3) FS_CASE(4) FS_CASE(5) FS_CASE(6) FS_CASE(7) FS_CASE(8)
-      FS_CASE(9) FS_CASE(10) FS_CASE(11) FS_CASE(12) FS_CASE(13) FS_CASE(14) FS_CASE(15) FS_CASE(16)
       default: break;
     }
 #undef FS_CASE

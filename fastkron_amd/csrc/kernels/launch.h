@@ -32,6 +32,10 @@ hipError_t launchPairMfma(const StepArgs& a, DType dt, hipStream_t stream);
 bool stepMfmaSupported(const StepArgs& a, DType dt);
 hipError_t launchStepMfma(const StepArgs& a, DType dt, hipStream_t stream);
 
+// One step with a factor of any shape up to 128x128 on the matrix cores (zero padded), fp64 or fp32, any layout.
+bool stepAnyMfmaSupported(const StepArgs& a, DType dt);
+hipError_t launchStepAnyMfma(const StepArgs& a, DType dt, hipStream_t stream);
+
 // One step with a 64x64 fp64 factor on the KMM layout (4x4x4 matrix-core instruction, 64-column tiles).
 bool kmm64F64Supported(const StepArgs& a);
 hipError_t launchKmm64F64(const StepArgs& a, hipStream_t stream);
@@ -44,7 +48,7 @@ hipError_t launchKmm4x6(const StepArgs& a, hipStream_t stream);
 bool kmmRegSupported(const StepArgs& a);
 hipError_t launchKmmReg(const StepArgs& a, hipStream_t stream);
 
-// Several small factors of any shape (P <= 16) fused through LDS, MKM or KMM layout, fp32 or fp64.
+// Several small factors of any shape (P <= 8) fused through LDS, MKM or KMM layout, fp32 or fp64.
 // fusedSmallFits: whether a group of factors (p[0], q[0] applied first) on Kin input columns has a tile.
 bool fusedSmallFits(uint32_t nf, const uint32_t* p, const uint32_t* q, uint64_t Kin, uint32_t M, bool kmm, DType dt);
 bool fusedSmallSupported(const StepArgs& a, DType dt);

@@ -1,0 +1,229 @@
+// One sliced-multiply step with a factor of any shape up to 128 x 128 on the matrix cores, fp32 or fp64, MKM or
+// KMM layout, opX = T included: the sizes between the specialised kernels (24x24, 31x63, 50x50, 8x32, 100x100 ...).
+//
+//   out[m, q*S + s] = sum_p in[m, s*P + p] * F[p, q],   S = Kin / P
+//
+// The factor is padded with zeros to 4*pc rows (pc = ceil(P/4)) and 16*qb columns (qb = ceil(Q/16)) and staged in
+// LDS once per workgroup.  A tile is 16 lanes wide along the dimension that is contiguous in the output (slices of
+// one row in the MKM layout, rows of one slice in the KMM layout) and is computed transposed,
+// D[q][j] = sum_p F^T[q][p] * X^T[p][j], with V_MFMA_*_16X16X4:
+//   * B operand (lane = 16*k + j): lane group k covers the contraction indices p = k*pc + c, c < pc, so a lane
+//     reads pc elements that are consecutive in memory in the MKM layout; indices beyond P read as zero;
+//   * A operand (lane = 16*k + q): F[k*pc + c][16*ib + q] from LDS, one read per product (the k groups are offset
+//     by 16 elements so that the four groups hit different banks);
+//   * the accumulator rows are output columns q: every quarter wave stores 16 consecutive elements.
+// Waves are persistent and load the next tile before computing the current one.  pc is a runtime value below
+// the template bound PCMAX (4, 8, 16 or 32): the product loops are unrolled to PCMAX with wave-uniform guards.
+//
+// Plays the role of the reference's generated kernels for arbitrary factor shapes (reference
+// src/kernels/cuda/kernel.cuh:53-224, which computes on CUDA cores, and src/gen_tuner_kernels.py which instantiates
+// one kernel per shape); one kernel with zero padding is this library's way.
+// Algorithmic traffic per launch: read M*Kin, write M*Kout elements (+ M*Kout for Y on the launch that writes Z).
+#include <hip/hip_runtime.h>
+#include "../problem.h"
+#include "launch.h"
+
+namespace fk {
+
+typedef double sad4 __attribute__((ext_vector_type(4)));
+typedef float saf4 __attribute__((ext_vector_type(4)));
+
+template <typename T> struct SaMfma;
+template <> struct SaMfma<double> {
+  using Acc = sad4;
+  static __device__ __forceinline__ Acc mma(double a, double b, Acc c) {
+    return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0);
+  }
+  // row index (0..15) of accumulator register r in the lane group hi = lane >> 4
+  static __device__ __forceinline__ int row(int r, int hi) { return 4 * r + hi; }
+};
+template <> struct SaMfma<float> {
+  using Acc = saf4;
+  static __device__ __forceinline__ Acc mma(float a, float b, Acc c) {
+    return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ int row(int r, int hi) { return 4 * hi + r; }
+};
+
+constexpr int kSaWaves = 4;
+constexpr uint32_t kSaMaxDim = 128;
+
+// A "line" is what a tile's 16 lanes run along: the slices of one row (MKM) or the rows of one slice (KMM).
+// Element (line, j, p) of the input lives at line*inLine + j*inJ + p*inP, element (line, q, j) of the output at
+// line*outLine + q*outQ + j*outJ, likewise for Y.
+struct StepAnyGeom {
+  uint32_t P, Q, pc, qb, kStride;      // kStride: LDS elements between the rows of two lane groups
+  uint32_t nJ, jBlocks, totalTiles;
+  int64_t inLine, inJ, inP, outLine, outJ, outQ, yLine, yJ, yQ;
+};
+
+template <typename T, int PCMAX, bool HAS_Y>
+__global__ __launch_bounds__(256, 2) void kron_step_any_kernel(const StepArgs a, const StepAnyGeom g) {
+  using MF = SaMfma<T>;
+  using Acc = typename MF::Acc;
+  extern __shared__ __align__(16) unsigned char saLds[];
+  T* fl = (T*)saLds;
+  const int tid = threadIdx.x;
+  const int l = tid & 63;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lo = l & 15, hi = l >> 4;
+  const uint32_t bt = blockIdx.y;
+  const uint32_t pc = g.pc, Qp = g.qb * 16;
+
+  const T* inB = (const T*)a.in + (size_t)bt * a.in_batch;
+  T* outB = (T*)a.out + (size_t)bt * a.out_batch;
+  const T* YB = HAS_Y ? (const T*)a.y + (size_t)bt * a.y_batch : nullptr;
+  const T alpha = a.epilogue ? (T)a.alpha : (T)1, beta = (T)a.beta;
+
+  // the zero-padded factor: fl[k*kStride + c*Qp + q] = F[k*pc + c][q]
+  {
+    const T* F = (const T*)a.f[0] + (size_t)bt * a.f_batch[0];
+    const uint32_t perK = pc * Qp;
+    for (uint32_t idx = tid; idx < 4 * perK; idx += 256) {
+      const uint32_t k = idx / perK, rem = idx - k * perK, c = rem / Qp, q = rem - c * Qp;
+      const uint32_t p = k * pc + c;
+      T v = (T)0;
+      if (p < g.P && q < g.Q) v = F[(int64_t)p * a.f_sp[0] + (int64_t)q * a.f_sq[0]];
+      fl[k * g.kStride + c * Qp + q] = v;
+    }
+  }
+  __syncthreads();
+
+  const uint32_t nWaves = gridDim.x * kSaWaves;
+  const uint32_t wave = blockIdx.x * kSaWaves + w;
+  const uint32_t p0 = hi * pc;                        // first contraction index of this lane group
+  const T* fa = fl + hi * g.kStride + lo;
+
+  auto loadTile = [&](uint32_t t, T (&x)[PCMAX]) {
+    const uint32_t line = t / g.jBlocks, j0 = (t - line * g.jBlocks) * 16;
+    const uint32_t j = (j0 + lo < g.nJ) ? j0 + lo : j0;                 // clamped: computed, not stored
+    const T* xp = inB + (int64_t)line * g.inLine + (int64_t)j * g.inJ + (int64_t)p0 * g.inP;
+    const uint32_t nvalid = p0 < g.P ? g.P - p0 : 0u;                   // contraction indices of this lane group below P
+#pragma unroll
+    for (int c = 0; c < PCMAX; c++) {
+      if (c < (int)pc) {
+        x[c] = (T)0;                                                    // indices beyond P count as zero and are not read
+        if ((uint32_t)c < nvalid) x[c] = xp[(int64_t)c * g.inP];
+      }
+    }
+  };
+
+  T xn[PCMAX];
+  if (wave < g.totalTiles) loadTile(wave, xn);
+  for (uint32_t t = wave; t < g.totalTiles; t += nWaves) {
+    T x[PCMAX];
+#pragma unroll
+    for (int c = 0; c < PCMAX; c++) x[c] = xn[c];
+    if (t + nWaves < g.totalTiles) loadTile(t + nWaves, xn);           // the next tile streams in under the products
+
+    const uint32_t line = t / g.jBlocks, j = (t - line * g.jBlocks) * 16 + lo;
+    const bool jOk = j < g.nJ;
+    T* out = outB + (int64_t)line * g.outLine + (int64_t)j * g.outJ;
+    const T* Y = HAS_Y ? YB + (int64_t)line * g.yLine + (int64_t)j * g.yJ : nullptr;
+    for (uint32_t ib = 0; ib < g.qb; ib++) {
+      Acc acc = (Acc){0, 0, 0, 0};
+#pragma unroll
+      for (int c = 0; c < PCMAX; c++)
+        if (c < (int)pc) acc = MF::mma(fa[c * Qp + 16 * ib], x[c], acc);
+      T yv[4];
+      if (HAS_Y) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          const uint32_t q = 16 * ib + MF::row(r, hi);
+          yv[r] = (jOk && q < g.Q) ? Y[(int64_t)q * g.yQ] : (T)0;
+        }
+      }
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const uint32_t q = 16 * ib + MF::row(r, hi);
+        if (!(jOk && q < g.Q)) continue;
+        T v = acc[r] * alpha;
+        if (HAS_Y) v += beta * yv[r];
+        out[(int64_t)q * g.outQ] = v;
+      }
+    }
+  }
+}
+
+static bool saOutRowsContiguous(const StepArgs& a) { return a.out_ldm == 1 && a.out_ldc != 1; }
+
+static bool stepAnyGeometry(const StepArgs& a, DType dt, StepAnyGeom* g) {
+  if (a.nf != 1 || a.M == 0) return false;
+  const uint32_t P = a.p[0], Q = a.q[0];
+  if (P == 0 || Q == 0 || P > kSaMaxDim || Q > kSaMaxDim || a.Kin % P) return false;
+  const uint64_t S = a.Kin / P;
+  if (S >= (1ull << 31)) return false;
+  g->P = P; g->Q = Q; g->pc = (P + 3) / 4; g->qb = (Q + 15) / 16;
+  g->kStride = g->pc * g->qb * 16 + 16;
+  uint64_t nLines;
+  if (saOutRowsContiguous(a)) {        // KMM: lanes along the rows of one slice
+    nLines = S; g->nJ = a.M;
+    g->inLine = (int64_t)P * a.in_ldc;  g->inJ = a.in_ldm;  g->inP = a.in_ldc;
+    g->outLine = a.out_ldc;             g->outJ = a.out_ldm; g->outQ = (int64_t)S * a.out_ldc;
+    g->yLine = a.y_ldc;                 g->yJ = a.y_ldm;     g->yQ = (int64_t)S * a.y_ldc;
+  } else {                             // MKM: lanes along the slices of one row
+    nLines = a.M; g->nJ = (uint32_t)S;
+    g->inLine = a.in_ldm;   g->inJ = (int64_t)P * a.in_ldc; g->inP = a.in_ldc;
+    g->outLine = a.out_ldm; g->outJ = a.out_ldc;            g->outQ = (int64_t)S * a.out_ldc;
+    g->yLine = a.y_ldm;     g->yJ = a.y_ldc;                g->yQ = (int64_t)S * a.y_ldc;
+  }
+  g->jBlocks = (g->nJ + 15) / 16;
+  const uint64_t tiles = nLines * g->jBlocks;
+  if (tiles >= (1ull << 31)) return false;
+  g->totalTiles = (uint32_t)tiles;
+  (void)dt;
+  return a.batch <= 65535;
+}
+
+bool stepAnyMfmaSupported(const StepArgs& a, DType dt) {
+  StepAnyGeom g;
+  return stepAnyGeometry(a, dt, &g);
+}
+
+template <typename T, int PCMAX>
+static hipError_t launchStepAnyT(const StepArgs& a, const StepAnyGeom& g, hipStream_t stream) {
+  const size_t ldsBytes = (size_t)4 * g.kStride * sizeof(T);
+  static bool attrSet = false;
+  if (!attrSet) {
+    hipError_t e = hipFuncSetAttribute((const void*)kron_step_any_kernel<T, PCMAX, true>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 140 * 1024);
+    if (e != hipSuccess) return e;
+    e = hipFuncSetAttribute((const void*)kron_step_any_kernel<T, PCMAX, false>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, 140 * 1024);
+    if (e != hipSuccess) return e;
+    attrSet = true;
+  }
+  static int cus = 0;
+  if (!cus) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    cus = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+              ? prop.multiProcessorCount : 256;
+  }
+  // persistent workgroups: two per CU when the factor's LDS copy allows it, fewer when there is not enough work
+  uint32_t wgs = (uint32_t)cus * (ldsBytes <= 72 * 1024 ? 2 : 1);
+  if (a.batch > 1) wgs = (wgs + a.batch - 1) / a.batch;
+  const uint32_t need = (g.totalTiles + kSaWaves - 1) / kSaWaves;
+  if (wgs > need) wgs = need;
+  if (wgs == 0) wgs = 1;
+  dim3 grid(wgs, a.batch), block(256);
+  if (a.y && a.epilogue) hipLaunchKernelGGL((kron_step_any_kernel<T, PCMAX, true>), grid, block, ldsBytes, stream, a, g);
+  else                   hipLaunchKernelGGL((kron_step_any_kernel<T, PCMAX, false>), grid, block, ldsBytes, stream, a, g);
+  return hipGetLastError();
+}
+
+template <typename T>
+static hipError_t launchStepAnyD(const StepArgs& a, const StepAnyGeom& g, hipStream_t stream) {
+  if (g.pc <= 4)  return launchStepAnyT<T, 4>(a, g, stream);
+  if (g.pc <= 8)  return launchStepAnyT<T, 8>(a, g, stream);
+  if (g.pc <= 16) return launchStepAnyT<T, 16>(a, g, stream);
+  return launchStepAnyT<T, 32>(a, g, stream);
+}
+
+hipError_t launchStepAnyMfma(const StepArgs& a, DType dt, hipStream_t stream) {
+  StepAnyGeom g;
+  if (!stepAnyGeometry(a, dt, &g)) return hipErrorInvalidValue;
+  return dt == DType::F32 ? launchStepAnyD<float>(a, g, stream) : launchStepAnyD<double>(a, g, stream);
+}
+
+}  // namespace fk

@@ -498,7 +498,7 @@ FUSED_SMALL = [
     (5, [3, 5, 2], [4, 2, 6]),                # rectangular factors: the piece grows and shrinks between the steps
     (3, [6] * 5, [6] * 5),                    # even, not a power of two
     (40, [2, 3, 2, 3, 2, 3, 2, 3], [3, 2, 3, 2, 3, 2, 3, 2]),
-    (7, [13, 11, 9], [9, 11, 13]),            # P up to 16
+    (7, [7, 5, 8], [5, 8, 3]),                # P up to 8, any Q
     (4, [3] * 10, [3] * 10),                  # reference tests/src/general-tests-NN.cpp shape family, K = 59049
     (50, [5, 5], [2, 3]),
 ]
@@ -516,3 +516,29 @@ def test_small_factors_of_any_shape_are_fused_through_lds(fk, mm, M, Ps, Qs, dt)
     check(fk, mm, M, Ps, Qs, dt, alpha=1.0, beta=0.0, seed=304, batch=2, share_f=True)
     if np.prod([max(p, q) for p, q in zip(Ps, Qs)]) < 50000:
         check(fk, mm, M, Ps, Qs, dt, alpha=1.0, beta=1.0, seed=305, integer=True)
+
+
+ANY_SHAPE = [
+    # M, Ps, Qs: one factor per launch on the matrix cores, zero padded to multiples of 4 (P) and 16 (Q)
+    (20, [31, 31], [31, 31]),
+    (5, [31, 33], [63, 37]),            # ragged in every dimension: P % 4, Q % 16, slices % 16
+    (16, [50, 50], [50, 50]),
+    (3, [100], [128]),
+    (33, [127], [9]),                   # a single output block, mostly padding
+    (4, [30, 64], [64, 30]),
+    (2, [128, 36], [36, 128]),
+]
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+@pytest.mark.parametrize("mm", [ko.MKM, ko.KMM])
+@pytest.mark.parametrize("M,Ps,Qs", ANY_SHAPE)
+def test_any_shape_step_on_the_matrix_cores(fk, mm, M, Ps, Qs, dt):
+    check(fk, mm, M, Ps, Qs, dt, alpha=1.5, beta=0.5, seed=401)
+    assert any("anyxany" in k for _, _, k in fk.last_plan()), fk.last_plan()
+    check(fk, mm, M, Ps, Qs, dt, alpha=1.0, beta=0.0, seed=402, opFs=ko.OP_T)
+    check(fk, mm, M, Ps, Qs, dt, alpha=1.0, beta=0.0, seed=403, opX=ko.OP_T)       # X stored transposed
+    assert any("anyxany" in k for _, _, k in fk.last_plan()), fk.last_plan()
+    check(fk, mm, M, Ps, Qs, dt, alpha=2.0, beta=1.0, seed=404, batch=3)
+    check(fk, mm, M, Ps, Qs, dt, alpha=1.0, beta=1.0, seed=405, integer=True)
+    check(fk, mm, M, Ps, Qs, dt, alpha=1.0, beta=0.0, seed=406, use_temp2=False)
