@@ -68,7 +68,8 @@ int ko_gekmm_sizes(uint32_t M, uint32_t N, const uint32_t* Ps, const uint32_t* Q
   for (uint32_t i = 0; i < N; i++) { K *= Ps[i]; L *= Qs[i]; }
   *yElems = (size_t)M * L;
   if (N == 1) { *tmpElems = (size_t)M * (K > L ? K : L); return 0; }
-  uint64_t* w = (uint64_t*)malloc(sizeof(uint64_t) * N);
+  uint64_t* w = (uint64_t*)calloc(N, sizeof(uint64_t));
+  if (!w) return 4;
   step_widths(N, Ps, Qs, w);
   uint64_t mx = 0;
   for (uint32_t i = 0; i < N; i++) if (w[i] > mx) mx = w[i];
@@ -80,7 +81,8 @@ int ko_gekmm_sizes(uint32_t M, uint32_t N, const uint32_t* Ps, const uint32_t* Q
 int ko_gekmm_sizes_forward(uint32_t M, uint32_t N, const uint32_t* Ps, const uint32_t* Qs,
                            size_t* yElems, size_t* intermediateElems) {
   if (!yElems || !intermediateElems || N == 0) return 4;
-  uint64_t* w = (uint64_t*)malloc(sizeof(uint64_t) * N);
+  uint64_t* w = (uint64_t*)calloc(N, sizeof(uint64_t));
+  if (!w) return 4;
   step_widths(N, Ps, Qs, w);
   *yElems = (size_t)M * w[0];
   for (uint32_t i = 1; i < N; i++) intermediateElems[i - 1] = (size_t)M * w[i];
