@@ -54,7 +54,7 @@ __device__ __forceinline__ void k6Contract3(float (&x)[64], const float (&fa)[3]
 
 template <bool HAS_Y>
 __global__ __launch_bounds__(512, 2) void kron_kmm4x6_kernel(const StepArgs a, const uint32_t mTiles) {
-  extern __shared__ float lds[];
+  extern __shared__ __align__(16) float lds[];
   const int tid = threadIdx.x;
   const int l = tid & 63;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);

@@ -14,11 +14,13 @@
 //            layout (lane 16*k+i) of a second product that contracts the *row* index i of the first;
 //            the factor operand of the second product is loaded with its rows permuted (4*k + r)
 //            to match.  No data movement between the two steps.
-//   exch. 1  transpose (k1,k2) <-> (q3,q4) through LDS, in two halves of 128 KB, XOR-swizzled so that
-//            both the ds_write_b32 and the ds_read_b32 side hit 64 distinct banks.
+//   exch. 1  transpose (k1,k2) <-> (q3,q4) through LDS, in two halves of 128 KB: 16-byte writes (four blocks
+//            of a lane are four adjacent columns of its row), 4-byte reads, chunks XOR-swizzled so that both
+//            sides are free of bank conflicts.
 //   stage 2  contract k1 then k2 the same way.
 //   exch. 2  bring the result to the store layout (lane = 4 consecutive columns, 1 KB per wave store),
-//            again in two swizzled halves; ds_read_b128 on the way out.
+//            again in two swizzled halves; 16-byte LDS writes and reads (the LDS pipeline is bound by its
+//            instruction rate, about 3-4 cycles per wave instruction whatever the width).
 //
 // Algorithmic traffic: 4*65536 bytes read + 4*65536 bytes written per row (+ Y when beta != 0).
 #include <hip/hip_runtime.h>
@@ -35,12 +37,15 @@ typedef float f4 __attribute__((ext_vector_type(4)));
 
 constexpr int kRowLen = 65536;
 constexpr int kLdsWords = 32768;           // 128 KB: one half of a row
-constexpr int kPF = 5;                     // blocks (of 16) of the next item loaded one item ahead
+#ifndef ROW16_KPF
+#define ROW16_KPF 5
+#endif
+constexpr int kPF = ROW16_KPF;                     // blocks (of 16) of the next item loaded one item ahead
 
 template <bool HAS_Y>
 __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a, const uint32_t blocksPerBatch,
                                                                const uint32_t totalItems) {
-  extern __shared__ float lds[];
+  extern __shared__ __align__(16) float lds[];
   const int tid = threadIdx.x;
   const int l0 = tid & 63;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);      // wave-uniform: keeps row addresses in SGPRs
@@ -104,6 +109,22 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a,
       for (int t = 0; t < 16 - kPF; t++) xb[t] = *(const f4*)(xp + t * 256);
     }
 
+    // LDS column of (k1 = w, k2 = t) is w*16 + t: the four blocks t = 4g .. 4g+3 of a lane are one 16-byte chunk
+    // of its row.  The chunk index is XORed with q3 = i so that the 64 rows of a wave-level write spread over
+    // the banks.
+    auto writeGroup = [&](const int g, const int h) {
+#pragma unroll
+      for (int rr = 0; rr < 2; rr++) {
+        f4 v;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          const int t = 4 * g + e;
+          v[e] = (t < kPF) ? xa[t < kPF ? t : 0][2 * h + rr] : xb[t < kPF ? 0 : t - kPF][2 * h + rr];
+        }
+        *(f4*)&lds[((kb * 2 + rr) * 16 + i) * 256 + (((w * 4 + g) ^ i) << 2)] = v;
+      }
+    };
+
     // ---- stage 1: contract k3 (first product) and k4 (second product), block by block.  The half of
     //      the result with bit 1 of q3 clear goes to LDS at once, under the products of the next blocks. ----
     {
@@ -128,9 +149,7 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a,
           // e[r] = Y[k1=w][k2=t0+t][q4=4kb+r][q3=i]: from here to the second exchange q3 and q4 appear with their
           // roles swapped with respect to the comments below (the first exchange treats them alike)
           x[t] = e;
-#pragma unroll
-          for (int rr = 0; rr < 2; rr++)
-            lds[((kb * 2 + rr) * 16 + i) * 256 + ((w * 16 + t0 + t) ^ l)] = e[rr];
+          if (((t0 + t) & 3) == 3) writeGroup((t0 + t) >> 2, 0);
         }
       };
       stage1(xa, kPF, 0);
@@ -145,21 +164,16 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a,
       if (h) {
         __syncthreads();
 #pragma unroll
-        for (int t = 0; t < 16; t++)
-#pragma unroll
-          for (int rr = 0; rr < 2; rr++) {
-            const int row = (kb * 2 + rr) * 16 + i;
-            lds[row * 256 + ((w * 16 + t) ^ l)] = (t < kPF) ? xa[t < kPF ? t : 0][2 + rr] : xb[t < kPF ? 0 : t - kPF][2 + rr];
-          }
+        for (int g = 0; g < 4; g++) writeGroup(g, 1);
       }
       __syncthreads();
 #pragma unroll
       for (int u = 0; u < 16; u++) {
         if (((u >> 1) & 1) != h) continue;
         const int row = ((u >> 2) * 2 + (u & 1)) * 16 + w;
-        const int swz = w + 16 * (u >> 2);
+        // column (k1 = 4c + kb, k2 = i) = c*64 + l: chunk c*16 + l/4, XORed with the row's q3 = w as written
 #pragma unroll
-        for (int c = 0; c < 4; c++) z[u][c] = lds[row * 256 + ((c * 64 + l) ^ swz)];
+        for (int c = 0; c < 4; c++) z[u][c] = lds[row * 256 + ((((c * 16 + (l >> 2)) ^ w) << 2) | (l & 3))];
       }
     }
     __syncthreads();
@@ -194,9 +208,16 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a,
         for (int r = 0; r < 4; r++) e = MFMA16(d[r], FD[r], e);
 #pragma unroll
         for (int r = 0; r < 4; r++) z[u][r] = e[r];       // = Z[q1=4kb+r][q2=i][q3=u][q4=w]
+        // four consecutive columns (w*16 + u, u = 4g .. 4g+3) of a row go out as one 16-byte write; the chunk
+        // index is XORed with q2 so that the lanes of a write (same chunk, 64 rows) spread over the banks
+        if ((u & 3) == 3) {
+          const int g = u >> 2;
 #pragma unroll
-        for (int rr = 0; rr < 2; rr++)
-          lds[((kb * 2 + rr) * 16 + i) * 256 + ((w * 16 + u) ^ (i * 4) ^ kb)] = e[rr];   // column q3*16 + q4 = w*16 + u
+          for (int rr = 0; rr < 2; rr++) {
+            const f4 v = {z[4 * g][rr], z[4 * g + 1][rr], z[4 * g + 2][rr], z[4 * g + 3][rr]};
+            *(f4*)&lds[((kb * 2 + rr) * 16 + i) * 256 + (((w * 4 + g) ^ i) << 2)] = v;
+          }
+        }
       }
     }
 
@@ -209,11 +230,12 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a,
       if (h) {
         __syncthreads();
 #pragma unroll
-        for (int u = 0; u < 16; u++)
+        for (int g = 0; g < 4; g++)
 #pragma unroll
           for (int rr = 0; rr < 2; rr++) {
             const int row = (kb * 2 + rr) * 16 + i;
-            lds[row * 256 + ((w * 16 + u) ^ (i * 4) ^ kb)] = z[u][2 + rr];
+            const f4 v = {z[4 * g][2 + rr], z[4 * g + 1][2 + rr], z[4 * g + 2][2 + rr], z[4 * g + 3][2 + rr]};
+            *(f4*)&lds[row * 256 + (((w * 4 + g) ^ i) << 2)] = v;
           }
       }
       __syncthreads();
@@ -226,10 +248,7 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a,
         for (int k = 0; k < 4; k++) {
           const int q1hi = 2 * g + (k >> 1), rr = k & 1;
           const int row = (q1hi * 2 + rr) * 16 + w;
-          const f4 v = *(const f4*)&lds[row * 256 + ((l * 4) ^ (w * 4))];
-          f4 p;                                           // word e of v is column 4l + (e ^ q1hi)
-          p[0] = v[0 ^ q1hi]; p[1] = v[1 ^ q1hi]; p[2] = v[2 ^ q1hi]; p[3] = v[3 ^ q1hi];
-          o[k] = p;
+          o[k] = *(const f4*)&lds[row * 256 + ((l * 4) ^ (w * 4))];     // chunk l of the row of (q1, q2 = w)
           if (HAS_Y) yv[k] = *(const f4*)(Y + (4 * q1hi + 2 * h + rr) * 4096 + w * 256 + l * 4);
         }
 #pragma unroll

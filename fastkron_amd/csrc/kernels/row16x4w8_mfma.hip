@@ -46,7 +46,7 @@ constexpr int kW8Early = 16;                // (v,t) register blocks of the next
 template <bool HAS_Y>
 __global__ __launch_bounds__(512, 2) void kron_row16x4w8_kernel(const StepArgs a, const uint32_t blocksPerBatch,
                                                                 const uint32_t totalItems) {
-  extern __shared__ float lds[];
+  extern __shared__ __align__(16) float lds[];
   const int tid = threadIdx.x;
   const int l0 = tid & 63;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);      // wave-uniform: keeps row addresses in SGPRs

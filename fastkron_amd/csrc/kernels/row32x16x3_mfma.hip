@@ -29,7 +29,7 @@ constexpr int kRow32LdsWords = 8192;
 
 template <bool HAS_Y>
 __global__ __launch_bounds__(512, 4) void kron_row32x16x3_kernel(const StepArgs a) {
-  extern __shared__ float lds[];
+  extern __shared__ __align__(16) float lds[];
   const int tid = threadIdx.x;
   const int l = tid & 63;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);      // wave-uniform: keeps row addresses in SGPRs

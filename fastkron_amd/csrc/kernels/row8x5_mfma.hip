@@ -75,7 +75,7 @@ __device__ __forceinline__ void contractSecond(float (&x)[8][8], const float (&f
 
 template <bool HAS_Y>
 __global__ __launch_bounds__(512, 4) void kron_row8x5_kernel(const StepArgs a) {
-  extern __shared__ float lds[];
+  extern __shared__ __align__(16) float lds[];
   float* fl = lds + 16384;                       // factors: fl[f*64 + p*8 + q], f = 0 is F1
   const int tid = threadIdx.x;
   const int l = tid & 63;
@@ -126,13 +126,19 @@ __global__ __launch_bounds__(512, 4) void kron_row8x5_kernel(const StepArgs a) {
 #pragma unroll
   for (int h = 0; h < 2; h++) {
     if (h) __syncthreads();
+    // id & 15 = (j & 1)*8 + w: two base addresses (even and odd j) plus constant offsets, so that the writes
+    // pair up into two-address LDS instructions
+    {
+      float* const base0 = lds + w * 64 + ((((l >> 2) ^ w) << 2) | (l & 3));
+      float* const base1 = lds + w * 64 + ((((l >> 2) ^ (w + 8)) << 2) | (l & 3));
 #pragma unroll
-    for (int i = 0; i < 4; i++)
+      for (int i = 0; i < 4; i++)
 #pragma unroll
-      for (int j = 0; j < 8; j++) {
-        const int id = i * 64 + j * 8 + w;
-        lds[id * 64 + ((((l >> 2) ^ (id & 15)) << 2) | (l & 3))] = x[4 * h + i][j];
-      }
+        for (int jj = 0; jj < 8; jj++) {
+          const int j = (jj < 4) ? 2 * jj : 2 * (jj - 4) + 1;          // even columns, then odd ones
+          ((j & 1) ? base1 : base0)[(i * 64 + j * 8) * 64] = x[4 * h + i][j];
+        }
+    }
     __syncthreads();
     if ((w >> 2) == h) {
       const int id = (w & 3) * 64 + l;
