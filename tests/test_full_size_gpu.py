@@ -83,3 +83,34 @@ def test_full_size_configuration(fk, name, mm, M, Ps, Qs, dt, alpha, beta, batch
         want = _oracle(mm, 1, Ps, Qs, xsum, fb, ysum, alpha, beta, np.float64)
         err = normwise(zsum, want)
         assert err <= TOL[dt], f"batch {b}: checksum over all chains off by {err:.3e}"
+
+
+@pytest.mark.parametrize("mm,M,Ps,dt", [
+    (ko.MKM, 2064, [16] * 5, np.float32),      # 2.16e9 elements: whole-block kernel on virtual rows + leading launch
+    (ko.MKM, 1040, [3] * 13, np.float32),      # 1.66e9 elements through the LDS-fused kernel
+    (ko.KMM, 4160, [64] * 3, np.float64),      # 1.09e9 doubles (8.7 GB per buffer) in the KMM layout
+])
+def test_element_offsets_beyond_32_bits(fk, mm, M, Ps, dt):
+    """Buffers whose element or byte offsets do not fit 32 bits: operands are generated on the device, a few
+    chains (the last ones included) are checked against the oracle."""
+    import torch
+    K = int(np.prod(Ps))
+    tdt = torch.float32 if dt == np.float32 else torch.float64
+    g = torch.Generator(device="cuda").manual_seed(5)
+    X = torch.rand(M * K, device="cuda", dtype=tdt, generator=g) - 0.5
+    Fs = [torch.rand(p * p, device="cuda", dtype=tdt, generator=g) - 0.5 for p in Ps]
+    Z = torch.empty(M * K, device="cuda", dtype=tdt)
+    t1, t2 = torch.empty_like(Z), torch.empty_like(Z)
+    fn = fk.xgemkm if mm == ko.MKM else fk.xgekmm
+    assert fn(M, Ps, Ps, X, Fs, Z, 1.0, 0.0, None, t1, t2) == 0
+    torch.cuda.synchronize()
+    picks = [0, 1, M // 2, M - 2, M - 1]
+    if mm == ko.MKM:
+        xs, zs = X.view(M, K)[picks].cpu().numpy(), Z.view(M, K)[picks].cpu().numpy()
+    else:
+        xs = X.view(K, M)[:, picks].contiguous().cpu().numpy()
+        zs = Z.view(K, M)[:, picks].contiguous().cpu().numpy()
+    del X, Z, t1, t2
+    want = _oracle(mm, len(picks), Ps, Ps, xs, [f.cpu().numpy() for f in Fs], None, 1.0, 0.0, dt)
+    err = normwise(np.ascontiguousarray(zs).reshape(-1), want)
+    assert err <= TOL[dt], err
