@@ -200,8 +200,19 @@ static hipError_t launchStepAnyT(const StepArgs& a, const StepAnyGeom& g, hipStr
     cus = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
               ? prop.multiProcessorCount : 256;
   }
-  // persistent workgroups: two per CU when the factor's LDS copy allows it, fewer when there is not enough work
-  uint32_t wgs = (uint32_t)cus * (ldsBytes <= 72 * 1024 ? 2 : 1);
+  // persistent workgroups, as many per CU as registers and the factor's LDS copy allow: a wave has one tile in
+  // flight, so the bytes in flight per CU (what hides the HBM latency) grow with the number of resident waves
+  static size_t occLds = ~(size_t)0;
+  static int occ = 1;
+  if (occLds != ldsBytes) {
+    int n = 0;
+    const void* fn = (a.y && a.epilogue) ? (const void*)kron_step_any_kernel<T, PCMAX, true>
+                                         : (const void*)kron_step_any_kernel<T, PCMAX, false>;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, fn, 256, ldsBytes) != hipSuccess || n < 1) n = 1;
+    occ = n > 8 ? 8 : n;
+    occLds = ldsBytes;
+  }
+  uint32_t wgs = (uint32_t)cus * (uint32_t)occ;
   if (a.batch > 1) wgs = (wgs + a.batch - 1) / a.batch;
   const uint32_t need = (g.totalTiles + kSaWaves - 1) / kSaWaves;
   if (wgs > need) wgs = need;
