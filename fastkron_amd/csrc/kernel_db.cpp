@@ -129,6 +129,23 @@ static bool row8CanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, u
 static hipError_t row8Launch(const KernelInfo&, const StepArgs& a, hipStream_t s) { return launchRow8x5(a, s); }
 static bool row8Check(const KernelInfo&, const StepArgs& a) { return row8x5Supported(a); }
 
+// ---- wave-per-block kernel for two or three fused 16x16 fp64 factors ----
+static bool row16x3F64CanRun(const KernelInfo&, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
+                             const DeviceInfo&) {
+  const uint32_t nf = hi - lo + 1;
+  if (p.dt != DType::F64 || p.mm != MMType::MKM || nf < 2 || nf > 3 || p.forward) return false;
+  uint64_t kk = 1;
+  for (uint32_t i = lo; i <= hi; i++) {
+    if (p.P[i] != 16 || p.Q[i] != 16) return false;
+    if (p.batch > 1 && p.strideF[i] != 0) return false;     // the factors are staged once per workgroup
+    kk *= 16;
+  }
+  if (p.colsBefore(hi) != kk || (nf == 2 && p.M % 16)) return false;
+  return !(first && p.opX == 2);
+}
+static hipError_t row16x3F64Launch(const KernelInfo&, const StepArgs& a, hipStream_t s) { return launchRow16x3F64(a, s); }
+static bool row16x3F64Check(const KernelInfo&, const StepArgs& a) { return row16x3F64Supported(a); }
+
 // ---- whole-row kernel for three fused 32x16 fp32 factors ----
 static bool row32CanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
                         const DeviceInfo&) {
@@ -226,6 +243,14 @@ void registerRowKernels(std::vector<KernelInfo>& out) {
   k32.dt = DType::F32; k32.P = 32; k32.Q = 16; k32.fused = 3; k32.tileM = 1; k32.tileK = 32768; k32.threads = 512;
   k32.variant = 0; k32.canRun = row32CanRun; k32.launch = row32Launch; k32.check = row32Check;
   out.push_back(k32);
+
+  {
+    KernelInfo kd3{};
+    kd3.name = "mkm_hip_gfx950_256_d_16x16_16x16_3_1x4096_mfma16x16x4_NN_strided_0_3";
+    kd3.dt = DType::F64; kd3.P = 16; kd3.Q = 16; kd3.fused = 3; kd3.tileM = 1; kd3.tileK = 4096; kd3.threads = 256;
+    kd3.variant = 0; kd3.canRun = row16x3F64CanRun; kd3.launch = row16x3F64Launch; kd3.check = row16x3F64Check;
+    out.push_back(kd3);
+  }
 
   {
     KernelInfo k6{};

@@ -1,0 +1,200 @@
+// Three fused 16x16 fp64 factors on contiguous blocks of 16^3 = 4096 doubles (dgemkm with 16x16^3, or the three
+// trailing factors of a longer chain applied block by block): one wave owns a block, keeps it in registers and
+// needs neither an LDS exchange nor a barrier.
+//
+//   Z[q1,q2,q3] = alpha * sum_{k1,k2,k3} X[k1,k2,k3] F1[k1,q1] F2[k2,q2] F3[k3,q3]  (+ beta*Y)
+//
+//   k3, k2   for every k1: V_MFMA_F64_16X16X4_F64 twice, chained in registers.  The first product contracts k3 with
+//            the 256 values X[k1,:,:] as A operand (lane = (k2, 4 consecutive k3): two 16-byte loads, 2 KB contiguous
+//            per wave) and leaves D[k2][q3] in register k2/4 of lane 16*(k2%4) + q3, which is the B-operand layout
+//            of a product that contracts k2; its A operand is F2 with the rows permuted to match (4r + lane/16).
+//   k1       the 16 results of a lane for its (q2, q3) sit in 16 x 4 registers: the last contraction runs over the
+//            register index on the vector ALU (fp64 FMA runs at the matrix rate on this chip), F1 read from LDS as
+//            broadcast 16-byte pairs.
+//   store    per q1 a lane holds four doubles, rows q2 = 4r + lane/16: every quarter wave writes a 128-byte line.
+// With two factors the leading digit is a row index (16 consecutive rows form a block) and F1 is the identity.
+//
+// The reference has no fp64 kernel that fuses this shape in one launch: its tile must fit 48 KB of shared memory
+// (reference src/gen_tuner_kernels.py:10,366) and it runs one or two factors per launch.
+// Algorithmic traffic: 8*4096 bytes read + 8*4096 bytes written per block (+ Y when beta != 0).
+#include <hip/hip_runtime.h>
+#include "../problem.h"
+#include "launch.h"
+
+namespace fk {
+
+typedef double r3d4 __attribute__((ext_vector_type(4)));
+typedef double r3d2 __attribute__((ext_vector_type(2)));
+
+#define R3MFMA(a, b, c) __builtin_amdgcn_mfma_f64_16x16x4f64((a), (b), (c), 0, 0, 0)
+
+constexpr int kR3Block = 4096;
+constexpr int kR3Waves = 4;
+constexpr int kR3Ahead = 2;            // k1 slices of the next block requested before the last contraction
+constexpr int kR3Win = 2;              // further slices in flight while a block is contracted
+
+template <bool HAS_Y>
+__global__ __launch_bounds__(256, 2) void kron_row16x3_f64_kernel(const StepArgs a, const uint32_t blocksPerBatch,
+                                                                  const uint32_t totalBlocks) {
+  __shared__ __align__(16) double f1s[256];          // F1 transposed: f1s[q1*16 + k1]
+  const int tid = threadIdx.x;
+  const int l0 = tid & 63;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lo = l0 & 15, hi = l0 >> 4;
+
+  // a.f[0] is the last factor F3, a.f[1] = F2, a.f[2] = F1 (identity when only two factors are fused).
+  // Factors shared by the whole launch only: per-batch factors are left to other kernels.
+  {
+    const int q1 = tid >> 4, k1 = tid & 15;
+    double v = (q1 == k1) ? 1.0 : 0.0;
+    if (a.nf == 3) v = ((const double*)a.f[2])[(int64_t)k1 * a.f_sp[2] + (int64_t)q1 * a.f_sq[2]];
+    f1s[tid] = v;
+  }
+  // operands of the two products: F3[4*hi + c][lo] and F2[4*r + hi][lo]
+  double f3[4], f2[4];
+  {
+    const double* F3 = (const double*)a.f[0];
+    const double* F2 = (const double*)a.f[1];
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+      f3[c] = F3[(int64_t)(4 * hi + c) * a.f_sp[0] + (int64_t)lo * a.f_sq[0]];
+      f2[c] = F2[(int64_t)(4 * c + hi) * a.f_sp[1] + (int64_t)lo * a.f_sq[1]];
+    }
+  }
+  __syncthreads();
+
+  const uint32_t nWaves = gridDim.x * kR3Waves;
+  uint32_t blk = blockIdx.x * kR3Waves + w;
+  if (blk >= totalBlocks) return;
+
+  auto blockPtr = [&](uint32_t b) {
+    return (const double*)a.in + (size_t)(b / blocksPerBatch) * a.in_batch + (size_t)(b % blocksPerBatch) * kR3Block;
+  };
+  // x[c] = X[k1][k2 = lo][k3 = 4*hi + c]
+  auto loadSlice = [&](const double* X, int k1, double (&x)[4]) {
+    const double* xp = X + k1 * 256 + lo * 16 + hi * 4;
+    const r3d2 v0 = *(const r3d2*)xp, v1 = *(const r3d2*)(xp + 2);
+    x[0] = v0[0]; x[1] = v0[1]; x[2] = v1[0]; x[3] = v1[1];
+  };
+
+  double xa[kR3Ahead][4];                            // the first slices of the block about to be processed
+  {
+    const double* X = blockPtr(blk);
+#pragma unroll
+    for (int k = 0; k < kR3Ahead; k++) loadSlice(X, k, xa[k]);
+  }
+
+  auto processBlock = [&](const uint32_t blk) {
+    const double* X = blockPtr(blk);
+    const size_t bt = blk / blocksPerBatch, m = blk % blocksPerBatch;
+    double* Z = (double*)a.out + bt * a.out_batch + m * kR3Block;
+    const double* Y = HAS_Y ? (const double*)a.y + bt * a.y_batch + m * kR3Block : nullptr;
+
+    // ---- k3 and k2, slice by slice; z[k1][r] = T[k1][q2 = 4r + hi][q3 = lo] ----
+    double z[16][4];
+    double xb[kR3Win][4];                            // rolling window of slices in flight
+#pragma unroll
+    for (int k = 0; k < kR3Win; k++) loadSlice(X, kR3Ahead + k, xb[k]);
+#pragma unroll
+    for (int k1 = 0; k1 < 16; k1++) {
+      double x[4];
+#pragma unroll
+      for (int c = 0; c < 4; c++)
+        x[c] = (k1 < kR3Ahead) ? xa[k1 < kR3Ahead ? k1 : 0][c] : xb[(k1 - kR3Ahead) % kR3Win][c];
+      if (k1 >= kR3Ahead && k1 + kR3Win < 16) loadSlice(X, k1 + kR3Win, xb[(k1 - kR3Ahead) % kR3Win]);
+      r3d4 d = {0, 0, 0, 0};
+#pragma unroll
+      for (int c = 0; c < 4; c++) d = R3MFMA(x[c], f3[c], d);          // d[k2][q3]
+      r3d4 e = {0, 0, 0, 0};
+#pragma unroll
+      for (int r = 0; r < 4; r++) e = R3MFMA(f2[r], d[r], e);          // e[q2][q3]
+#pragma unroll
+      for (int r = 0; r < 4; r++) z[k1][r] = e[r];
+      __builtin_amdgcn_sched_barrier(0);             // keeps the loads of later slices from being hoisted up here
+    }
+
+    // ---- the first slices of the wave's next block stream in under the last contraction ----
+    {
+      const uint32_t nx = blk + nWaves;
+      const double* Xn = blockPtr(nx < totalBlocks ? nx : blk);
+#pragma unroll
+      for (int k = 0; k < kR3Ahead; k++) loadSlice(Xn, k, xa[k]);
+    }
+
+    // ---- k1 on the vector ALU, one q1 at a time, and the stores ----
+    const double alpha = a.epilogue ? a.alpha : 1.0, beta = a.beta;
+    double* zp = Z + hi * 16 + lo;
+    const double* yp = HAS_Y ? Y + hi * 16 + lo : nullptr;
+#pragma unroll 1
+    for (int q1 = 0; q1 < 16; q1++) {
+      double yv[4];
+      if (HAS_Y) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) yv[r] = yp[q1 * 256 + r * 64];
+      }
+      double acc[4] = {0, 0, 0, 0};
+#pragma unroll
+      for (int k = 0; k < 16; k += 2) {
+        const r3d2 f = *(const r3d2*)&f1s[q1 * 16 + k];
+#pragma unroll
+        for (int r = 0; r < 4; r++) acc[r] += f[0] * z[k][r];
+#pragma unroll
+        for (int r = 0; r < 4; r++) acc[r] += f[1] * z[k + 1][r];
+      }
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        double v = acc[r] * alpha;
+        if (HAS_Y) v += beta * yv[r];
+        zp[q1 * 256 + r * 64] = v;                   // Z[q1][q2 = 4r + hi][q3 = lo]
+      }
+    }
+  };
+
+  // The first block is peeled off the loop: the wait for the slices requested ahead is counted in younger memory
+  // operations, and entering the loop only from a complete block lets that count include the block's stores.
+  processBlock(blk);
+  for (blk += nWaves; blk < totalBlocks; blk += nWaves) processBlock(blk);
+}
+
+bool row16x3F64Supported(const StepArgs& a) {
+  if (a.nf != 2 && a.nf != 3) return false;
+  uint64_t k = 1;
+  for (uint32_t j = 0; j < a.nf; j++) {
+    if (a.p[j] != 16 || a.q[j] != 16 || (a.batch > 1 && a.f_batch[j] != 0)) return false;
+    k *= 16;
+  }
+  if (a.Kin != k || a.Kout != k) return false;
+  if (a.in_ldc != 1 || a.out_ldc != 1 || (a.y && a.y_ldc != 1)) return false;
+  // the rows of a block must be contiguous, and M must be a whole number of blocks
+  if ((uint64_t)a.in_ldm != k || (uint64_t)a.out_ldm != k || (a.y && (uint64_t)a.y_ldm != k)) return false;
+  if (a.nf == 2 && a.M % 16) return false;
+  // 16-byte loads
+  if (((uintptr_t)a.in & 15) || (a.in_batch & 1)) return false;
+  const uint64_t blocks = (uint64_t)(a.nf == 2 ? a.M / 16 : a.M) * a.batch;
+  return blocks < (1ull << 32);
+}
+
+hipError_t launchRow16x3F64(const StepArgs& a, hipStream_t stream) {
+  if (!row16x3F64Supported(a)) return hipErrorInvalidValue;
+  static int cus = 0;
+  if (!cus) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    cus = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+              ? prop.multiProcessorCount : 256;
+  }
+  const uint32_t blocksPerBatch = a.nf == 2 ? a.M / 16 : a.M;
+  const uint64_t total = (uint64_t)blocksPerBatch * a.batch;
+  // persistent waves: two workgroups of four waves per CU (two waves per SIMD at up to 256 registers)
+  uint32_t wgs = (uint32_t)cus * 2;
+  const uint64_t need = (total + kR3Waves - 1) / kR3Waves;
+  if (wgs > need) wgs = (uint32_t)need;
+  dim3 grid(wgs), block(256);
+  if (a.y && a.epilogue)
+    hipLaunchKernelGGL(kron_row16x3_f64_kernel<true>, grid, block, 0, stream, a, blocksPerBatch, (uint32_t)total);
+  else
+    hipLaunchKernelGGL(kron_row16x3_f64_kernel<false>, grid, block, 0, stream, a, blocksPerBatch, (uint32_t)total);
+  return hipGetLastError();
+}
+
+}  // namespace fk

@@ -542,3 +542,23 @@ def test_any_shape_step_on_the_matrix_cores(fk, mm, M, Ps, Qs, dt):
     check(fk, mm, M, Ps, Qs, dt, alpha=2.0, beta=1.0, seed=404, batch=3)
     check(fk, mm, M, Ps, Qs, dt, alpha=1.0, beta=1.0, seed=405, integer=True)
     check(fk, mm, M, Ps, Qs, dt, alpha=1.0, beta=0.0, seed=406, use_temp2=False)
+
+
+@pytest.mark.parametrize("M,Ps,launches", [
+    (5, [16] * 3, 1),               # a block per row
+    (32, [16, 16], 1),              # two factors: 16 rows per block, identity in the leading slot
+    (3, [16] * 4, 2),               # three trailing factors in place on 48 virtual rows + one leading launch
+    (1, [16] * 5, 3),
+    (2, [4, 8, 16, 16, 16], None),  # merged leading factors
+])
+def test_fp64_16x16_block_kernel(fk, M, Ps, launches):
+    """fp64 chains of 16x16 factors: three factors per launch on blocks of 4096 doubles held in one wave's registers."""
+    check(fk, ko.MKM, M, Ps, Ps, np.float64, alpha=1.5, beta=0.5, seed=501)
+    plan = fk.last_plan()
+    assert any("_d_16x16_16x16_3_" in k for _, _, k in plan), plan
+    if launches is not None:
+        assert len(plan) == launches, plan
+    check(fk, ko.MKM, M, Ps, Ps, np.float64, alpha=1.0, beta=0.0, seed=502, opFs=ko.OP_T)
+    check(fk, ko.MKM, M, Ps, Ps, np.float64, alpha=1.0, beta=1.0, seed=503, batch=3, share_f=True)
+    check(fk, ko.MKM, M, Ps, Ps, np.float64, alpha=2.0, beta=0.0, seed=504, batch=2)          # per-batch factors: other kernels
+    check(fk, ko.MKM, M, Ps, Ps, np.float64, alpha=1.0, beta=1.0, seed=505, integer=True)
