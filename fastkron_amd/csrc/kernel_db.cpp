@@ -54,12 +54,12 @@ static hipError_t fusedSmallLaunch(const KernelInfo& k, const StepArgs& a, hipSt
 }
 static bool fusedSmallCheck(const KernelInfo& k, const StepArgs& a) { return fusedSmallSupported(a, k.dt); }
 
-// ---- one factor of any shape up to 128x128 on the matrix cores (zero padded) ----
+// ---- one factor of any shape up to 256x512 on the matrix cores (zero padded) ----
 static bool stepAnyCanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, uint32_t hi, bool, bool,
                           const DeviceInfo&) {
   if (k.dt != p.dt || lo != hi) return false;
   const uint32_t P = p.P[lo], Q = p.Q[lo];
-  if (P > 128 || Q > 128) return false;
+  if (P > 256 || Q > 512) return false;
   // Small factors are bound by memory on the plain kernel already; the padded tiles pay off from these sizes on
   // (measured per layout and type: e.g. fp32 MKM 18x18, fp64 MKM 12x12, fp32 KMM 31x31, fp64 KMM 20x20).
   const bool kmm = p.mm == MMType::KMM && p.M > 1;
@@ -74,7 +74,7 @@ static bool stepAnyCheck(const KernelInfo& k, const StepArgs& a) { return stepAn
 void registerGenericKernels(std::vector<KernelInfo>& out) {
   for (DType dt : {DType::F32, DType::F64}) {
     KernelInfo k{};
-    k.name = std::string("gekmm_hip_gfx950_256_") + (dt == DType::F32 ? "f" : "d") + "_anyxany_128x128_1_16xany_mfma16x16x4";
+    k.name = std::string("gekmm_hip_gfx950_256_") + (dt == DType::F32 ? "f" : "d") + "_anyxany_256x512_1_16xany_mfma16x16x4";
     k.dt = dt; k.P = 1; k.Q = 1; k.fused = 1; k.tileM = 0; k.tileK = 0; k.threads = 256; k.variant = 0;
     k.canRun = stepAnyCanRun; k.launch = stepAnyLaunch; k.check = stepAnyCheck;
     out.push_back(k);

@@ -36,7 +36,7 @@ hipError_t launchStepMfma(const StepArgs& a, DType dt, hipStream_t stream);
 bool row16x3F64Supported(const StepArgs& a);
 hipError_t launchRow16x3F64(const StepArgs& a, hipStream_t stream);
 
-// One step with a factor of any shape up to 128x128 on the matrix cores (zero padded), fp64 or fp32, any layout.
+// One step with a factor of any shape up to 256x512 on the matrix cores (zero padded), fp64 or fp32, any layout.
 bool stepAnyMfmaSupported(const StepArgs& a, DType dt);
 hipError_t launchStepAnyMfma(const StepArgs& a, DType dt, hipStream_t stream);
 

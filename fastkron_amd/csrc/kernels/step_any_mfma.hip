@@ -1,5 +1,6 @@
-// One sliced-multiply step with a factor of any shape up to 128 x 128 on the matrix cores, fp32 or fp64, MKM or
-// KMM layout, opX = T included: the sizes between the specialised kernels (24x24, 31x63, 50x50, 8x32, 100x100 ...).
+// One sliced-multiply step with a factor of any shape up to 256 x 512 on the matrix cores, fp32 or fp64, MKM or
+// KMM layout, opX = T included: the sizes between the specialised kernels (24x24, 31x63, 50x50, 8x32, 100x100,
+// 200x200 ...).
 //
 //   out[m, q*S + s] = sum_p in[m, s*P + p] * F[p, q],   S = Kin / P
 //
@@ -13,7 +14,9 @@
 //     by 16 elements so that the four groups hit different banks);
 //   * the accumulator rows are output columns q: every quarter wave stores 16 consecutive elements.
 // Waves are persistent and load the next tile before computing the current one.  pc is a runtime value below
-// the template bound PCMAX (4, 8, 16 or 32): the product loops are unrolled to PCMAX with wave-uniform guards.
+// the template bound PCMAX (4 ... 64): the product loops are unrolled to PCMAX with wave-uniform guards.  A factor
+// whose padded copy does not fit 64 KB of LDS is split into slabs of output columns, one slab per workgroup
+// (grid z); the slabs of a tile re-read its input through the caches.
 //
 // Plays the role of the reference's generated kernels for arbitrary factor shapes (reference
 // src/kernels/cuda/kernel.cuh:53-224, which computes on CUDA cores, and src/gen_tuner_kernels.py which instantiates
@@ -46,18 +49,20 @@ template <> struct SaMfma<float> {
 };
 
 constexpr int kSaWaves = 4;
-constexpr uint32_t kSaMaxDim = 128;
+constexpr uint32_t kSaMaxP = 256, kSaMaxQ = 512;
+constexpr size_t kSaLdsTarget = 65536;     // per workgroup: two workgroups per CU
 
 // A "line" is what a tile's 16 lanes run along: the slices of one row (MKM) or the rows of one slice (KMM).
 // Element (line, j, p) of the input lives at line*inLine + j*inJ + p*inP, element (line, q, j) of the output at
 // line*outLine + q*outQ + j*outJ, likewise for Y.
 struct StepAnyGeom {
-  uint32_t P, Q, pc, qb, kStride;      // kStride: LDS elements between the rows of two lane groups
+  uint32_t P, Q, pc, pcPad, qb, kStride;   // pcPad: pc rounded up to 4; kStride: LDS elements between lane groups
+  uint32_t qbSlab, nSlabs;             // 16-column blocks per slab of output columns, slabs per factor
   uint32_t nJ, jBlocks, totalTiles;
   int64_t inLine, inJ, inP, outLine, outJ, outQ, yLine, yJ, yQ;
 };
 
-template <typename T, int PCMAX, bool HAS_Y>
+template <typename T, int PCMAX, bool HAS_Y, bool PREFETCH>
 __global__ __launch_bounds__(256, 2) void kron_step_any_kernel(const StepArgs a, const StepAnyGeom g) {
   using MF = SaMfma<T>;
   using Acc = typename MF::Acc;
@@ -68,22 +73,24 @@ __global__ __launch_bounds__(256, 2) void kron_step_any_kernel(const StepArgs a,
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lo = l & 15, hi = l >> 4;
   const uint32_t bt = blockIdx.y;
-  const uint32_t pc = g.pc, Qp = g.qb * 16;
+  const uint32_t pc = g.pc, Qp = g.qbSlab * 16;          // columns of this workgroup's slab of the factor
+  const uint32_t ib0 = blockIdx.z * g.qbSlab;
+  const uint32_t nb = g.qb - ib0 < g.qbSlab ? g.qb - ib0 : g.qbSlab;
 
   const T* inB = (const T*)a.in + (size_t)bt * a.in_batch;
   T* outB = (T*)a.out + (size_t)bt * a.out_batch;
   const T* YB = HAS_Y ? (const T*)a.y + (size_t)bt * a.y_batch : nullptr;
   const T alpha = a.epilogue ? (T)a.alpha : (T)1, beta = (T)a.beta;
 
-  // the zero-padded factor: fl[k*kStride + c*Qp + q] = F[k*pc + c][q]
+  // the zero-padded slab of the factor: fl[k*kStride + c*Qp + q] = F[k*pc + c][16*ib0 + q]
   {
     const T* F = (const T*)a.f[0] + (size_t)bt * a.f_batch[0];
-    const uint32_t perK = pc * Qp;
+    const uint32_t perK = g.pcPad * Qp;                // rows pc .. pcPad-1 of a lane group are zero
     for (uint32_t idx = tid; idx < 4 * perK; idx += 256) {
       const uint32_t k = idx / perK, rem = idx - k * perK, c = rem / Qp, q = rem - c * Qp;
-      const uint32_t p = k * pc + c;
+      const uint32_t p = k * pc + c, qq = 16 * ib0 + q;
       T v = (T)0;
-      if (p < g.P && q < g.Q) v = F[(int64_t)p * a.f_sp[0] + (int64_t)q * a.f_sq[0]];
+      if (c < pc && p < g.P && qq < g.Q) v = F[(int64_t)p * a.f_sp[0] + (int64_t)qq * a.f_sq[0]];
       fl[k * g.kStride + c * Qp + q] = v;
     }
   }
@@ -98,33 +105,47 @@ __global__ __launch_bounds__(256, 2) void kron_step_any_kernel(const StepArgs a,
     const uint32_t line = t / g.jBlocks, j0 = (t - line * g.jBlocks) * 16;
     const uint32_t j = (j0 + lo < g.nJ) ? j0 + lo : j0;                 // clamped: computed, not stored
     const T* xp = inB + (int64_t)line * g.inLine + (int64_t)j * g.inJ + (int64_t)p0 * g.inP;
-    const uint32_t nvalid = p0 < g.P ? g.P - p0 : 0u;                   // contraction indices of this lane group below P
+    uint32_t nvalid = p0 < g.P ? g.P - p0 : 0u;                         // contraction indices of this lane group below P
+    nvalid = nvalid < pc ? nvalid : pc;
 #pragma unroll
     for (int c = 0; c < PCMAX; c++) {
-      if (c < (int)pc) {
+      if (c < (int)g.pcPad) {
         x[c] = (T)0;                                                    // indices beyond P count as zero and are not read
         if ((uint32_t)c < nvalid) x[c] = xp[(int64_t)c * g.inP];
       }
     }
   };
 
-  T xn[PCMAX];
-  if (wave < g.totalTiles) loadTile(wave, xn);
+  T xn[PREFETCH ? PCMAX : 1];
+  if (PREFETCH && wave < g.totalTiles) loadTile(wave, (T(&)[PCMAX])xn);
   for (uint32_t t = wave; t < g.totalTiles; t += nWaves) {
     T x[PCMAX];
+    if (PREFETCH) {
 #pragma unroll
-    for (int c = 0; c < PCMAX; c++) x[c] = xn[c];
-    if (t + nWaves < g.totalTiles) loadTile(t + nWaves, xn);           // the next tile streams in under the products
+      for (int c = 0; c < PCMAX; c++) x[c] = xn[PREFETCH ? c : 0];
+      if (t + nWaves < g.totalTiles) loadTile(t + nWaves, (T(&)[PCMAX])xn);   // the next tile streams in under the products
+    } else {
+      loadTile(t, x);
+    }
 
     const uint32_t line = t / g.jBlocks, j = (t - line * g.jBlocks) * 16 + lo;
     const bool jOk = j < g.nJ;
     T* out = outB + (int64_t)line * g.outLine + (int64_t)j * g.outJ;
     const T* Y = HAS_Y ? YB + (int64_t)line * g.yLine + (int64_t)j * g.yJ : nullptr;
-    for (uint32_t ib = 0; ib < g.qb; ib++) {
+    for (uint32_t ibl = 0; ibl < nb; ibl++) {
+      const uint32_t ib = ib0 + ibl;
       Acc acc = (Acc){0, 0, 0, 0};
+      // four products per wave-uniform guard: straight-line groups let the operand reads run ahead of the products
 #pragma unroll
-      for (int c = 0; c < PCMAX; c++)
-        if (c < (int)pc) acc = MF::mma(fa[c * Qp + 16 * ib], x[c], acc);
+      for (int c0 = 0; c0 < PCMAX; c0 += 4) {
+        if (c0 < (int)g.pcPad) {
+          T f[4];
+#pragma unroll
+          for (int c = 0; c < 4; c++) f[c] = fa[(c0 + c) * Qp + 16 * ibl];
+#pragma unroll
+          for (int c = 0; c < 4; c++) acc = MF::mma(f[c], x[c0 + c], acc);
+        }
+      }
       T yv[4];
       if (HAS_Y) {
 #pragma unroll
@@ -150,11 +171,17 @@ static bool saOutRowsContiguous(const StepArgs& a) { return a.out_ldm == 1 && a.
 static bool stepAnyGeometry(const StepArgs& a, DType dt, StepAnyGeom* g) {
   if (a.nf != 1 || a.M == 0) return false;
   const uint32_t P = a.p[0], Q = a.q[0];
-  if (P == 0 || Q == 0 || P > kSaMaxDim || Q > kSaMaxDim || a.Kin % P) return false;
+  if (P == 0 || Q == 0 || P > kSaMaxP || Q > kSaMaxQ || a.Kin % P) return false;
   const uint64_t S = a.Kin / P;
   if (S >= (1ull << 31)) return false;
   g->P = P; g->Q = Q; g->pc = (P + 3) / 4; g->qb = (Q + 15) / 16;
-  g->kStride = g->pc * g->qb * 16 + 16;
+  // slabs of output columns so that the padded copy of a slab fits the LDS target
+  g->pcPad = (g->pc + 3) / 4 * 4;
+  uint32_t slab = (uint32_t)(kSaLdsTarget / (4 * (size_t)g->pcPad * 16 * dtypeSize(dt)));
+  if (slab < 1) slab = 1;
+  if (slab > g->qb) slab = g->qb;
+  g->qbSlab = slab; g->nSlabs = (g->qb + slab - 1) / slab;
+  g->kStride = g->pcPad * slab * 16 + 16;
   uint64_t nLines;
   if (saOutRowsContiguous(a)) {        // KMM: lanes along the rows of one slice
     nLines = S; g->nJ = a.M;
@@ -171,8 +198,7 @@ static bool stepAnyGeometry(const StepArgs& a, DType dt, StepAnyGeom* g) {
   const uint64_t tiles = nLines * g->jBlocks;
   if (tiles >= (1ull << 31)) return false;
   g->totalTiles = (uint32_t)tiles;
-  (void)dt;
-  return a.batch <= 65535;
+  return a.batch <= 65535 && g->nSlabs <= 65535;
 }
 
 bool stepAnyMfmaSupported(const StepArgs& a, DType dt) {
@@ -182,13 +208,15 @@ bool stepAnyMfmaSupported(const StepArgs& a, DType dt) {
 
 template <typename T, int PCMAX>
 static hipError_t launchStepAnyT(const StepArgs& a, const StepAnyGeom& g, hipStream_t stream) {
+  // the tile of the next iteration is held in registers too unless the two copies would not fit (fp64, P > 128)
+  constexpr bool PF = PCMAX * sizeof(T) <= 256;
   const size_t ldsBytes = (size_t)4 * g.kStride * sizeof(T);
   static bool attrSet = false;
   if (!attrSet) {
-    hipError_t e = hipFuncSetAttribute((const void*)kron_step_any_kernel<T, PCMAX, true>,
+    hipError_t e = hipFuncSetAttribute((const void*)kron_step_any_kernel<T, PCMAX, true, PF>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, 140 * 1024);
     if (e != hipSuccess) return e;
-    e = hipFuncSetAttribute((const void*)kron_step_any_kernel<T, PCMAX, false>,
+    e = hipFuncSetAttribute((const void*)kron_step_any_kernel<T, PCMAX, false, PF>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, 140 * 1024);
     if (e != hipSuccess) return e;
     attrSet = true;
@@ -206,29 +234,33 @@ static hipError_t launchStepAnyT(const StepArgs& a, const StepAnyGeom& g, hipStr
   static int occ = 1;
   if (occLds != ldsBytes) {
     int n = 0;
-    const void* fn = (a.y && a.epilogue) ? (const void*)kron_step_any_kernel<T, PCMAX, true>
-                                         : (const void*)kron_step_any_kernel<T, PCMAX, false>;
+    const void* fn = (a.y && a.epilogue) ? (const void*)kron_step_any_kernel<T, PCMAX, true, PF>
+                                         : (const void*)kron_step_any_kernel<T, PCMAX, false, PF>;
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, fn, 256, ldsBytes) != hipSuccess || n < 1) n = 1;
     occ = n > 8 ? 8 : n;
     occLds = ldsBytes;
   }
   uint32_t wgs = (uint32_t)cus * (uint32_t)occ;
-  if (a.batch > 1) wgs = (wgs + a.batch - 1) / a.batch;
+  const uint32_t share = a.batch * g.nSlabs;                  // the other two grid dimensions
+  if (share > 1) wgs = (wgs + share - 1) / share;
   const uint32_t need = (g.totalTiles + kSaWaves - 1) / kSaWaves;
   if (wgs > need) wgs = need;
   if (wgs == 0) wgs = 1;
-  dim3 grid(wgs, a.batch), block(256);
-  if (a.y && a.epilogue) hipLaunchKernelGGL((kron_step_any_kernel<T, PCMAX, true>), grid, block, ldsBytes, stream, a, g);
-  else                   hipLaunchKernelGGL((kron_step_any_kernel<T, PCMAX, false>), grid, block, ldsBytes, stream, a, g);
+  dim3 grid(wgs, a.batch, g.nSlabs), block(256);
+  if (a.y && a.epilogue)
+    hipLaunchKernelGGL((kron_step_any_kernel<T, PCMAX, true, PF>), grid, block, ldsBytes, stream, a, g);
+  else
+    hipLaunchKernelGGL((kron_step_any_kernel<T, PCMAX, false, PF>), grid, block, ldsBytes, stream, a, g);
   return hipGetLastError();
 }
 
 template <typename T>
 static hipError_t launchStepAnyD(const StepArgs& a, const StepAnyGeom& g, hipStream_t stream) {
-  if (g.pc <= 4)  return launchStepAnyT<T, 4>(a, g, stream);
-  if (g.pc <= 8)  return launchStepAnyT<T, 8>(a, g, stream);
-  if (g.pc <= 16) return launchStepAnyT<T, 16>(a, g, stream);
-  return launchStepAnyT<T, 32>(a, g, stream);
+  if (g.pcPad <= 4)  return launchStepAnyT<T, 4>(a, g, stream);
+  if (g.pcPad <= 8)  return launchStepAnyT<T, 8>(a, g, stream);
+  if (g.pcPad <= 16) return launchStepAnyT<T, 16>(a, g, stream);
+  if (g.pcPad <= 32) return launchStepAnyT<T, 32>(a, g, stream);
+  return launchStepAnyT<T, 64>(a, g, stream);
 }
 
 hipError_t launchStepAnyMfma(const StepArgs& a, DType dt, hipStream_t stream) {

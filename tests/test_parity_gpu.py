@@ -527,6 +527,9 @@ ANY_SHAPE = [
     (33, [127], [9]),                   # a single output block, mostly padding
     (4, [30, 64], [64, 30]),
     (2, [128, 36], [36, 128]),
+    (3, [129, 200], [200, 129]),        # beyond 128: more lane registers, the factor in slabs of output columns
+    (2, [255], [297]),
+    (4, [17], [512]),
 ]
 
 
