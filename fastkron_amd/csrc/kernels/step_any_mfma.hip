@@ -58,6 +58,7 @@ constexpr size_t kSaLdsTarget = 65536;     // per workgroup: two workgroups per 
 struct StepAnyGeom {
   uint32_t P, Q, pc, pcPad, qb, kStride;   // pcPad: pc rounded up to 4; kStride: LDS elements between lane groups
   uint32_t qbSlab, nSlabs;             // 16-column blocks per slab of output columns, slabs per factor
+  uint32_t vecLoad;                    // elements per vector load of the input (0: element by element)
   uint32_t nJ, jBlocks, totalTiles;
   int64_t inLine, inJ, inP, outLine, outJ, outQ, yLine, yJ, yQ;
 };
@@ -107,6 +108,37 @@ __global__ __launch_bounds__(256, 2) void kron_step_any_kernel(const StepArgs a,
     const T* xp = inB + (int64_t)line * g.inLine + (int64_t)j * g.inJ + (int64_t)p0 * g.inP;
     uint32_t nvalid = p0 < g.P ? g.P - p0 : 0u;                         // contraction indices of this lane group below P
     nvalid = nvalid < pc ? nvalid : pc;
+    if (g.vecLoad) {
+      // P is a multiple of 4 (no ragged lane group), the pc elements of a lane are contiguous and aligned:
+      // 16- or 8-byte loads
+      constexpr int VE = 16 / sizeof(T);
+      typedef T VT __attribute__((ext_vector_type(VE)));
+      typedef T V2 __attribute__((ext_vector_type(2)));
+      if (g.vecLoad >= (uint32_t)VE) {
+#pragma unroll
+        for (int c = 0; c < PCMAX; c += VE) {
+          if (c < (int)pc) {
+            const VT v = *(const VT*)(xp + c);
+#pragma unroll
+            for (int e = 0; e < VE; e++) x[c + e] = v[e];
+          } else if (c < (int)g.pcPad) {
+#pragma unroll
+            for (int e = 0; e < VE; e++) x[c + e] = (T)0;
+          }
+        }
+      } else {
+#pragma unroll
+        for (int c = 0; c < PCMAX; c += 2) {
+          if (c < (int)pc) {
+            const V2 v = *(const V2*)(xp + c);
+            x[c] = v[0]; x[c + 1] = v[1];
+          } else if (c < (int)g.pcPad) {
+            x[c] = (T)0; x[c + 1] = (T)0;
+          }
+        }
+      }
+      return;
+    }
 #pragma unroll
     for (int c = 0; c < PCMAX; c++) {
       if (c < (int)g.pcPad) {
@@ -193,6 +225,16 @@ static bool stepAnyGeometry(const StepArgs& a, DType dt, StepAnyGeom* g) {
     g->inLine = a.in_ldm;   g->inJ = (int64_t)P * a.in_ldc; g->inP = a.in_ldc;
     g->outLine = a.out_ldm; g->outJ = a.out_ldc;            g->outQ = (int64_t)S * a.out_ldc;
     g->yLine = a.y_ldm;     g->yJ = a.y_ldc;                g->yQ = (int64_t)S * a.y_ldc;
+  }
+  // vector loads: contiguous input, no ragged lane group, every lane's run aligned to the vector
+  g->vecLoad = 0;
+  if (g->inP == 1 && P % 4 == 0) {
+    const uint32_t es = (uint32_t)dtypeSize(dt);
+    for (uint32_t ve = 16 / es; ve >= 2; ve /= 2) {
+      const bool ok = g->pc % ve == 0 && g->inLine % ve == 0 && g->inJ % ve == 0 && (a.in_batch % ve) == 0 &&
+                      ((uintptr_t)a.in % (ve * es)) == 0;
+      if (ok) { g->vecLoad = ve; break; }
+    }
   }
   g->jBlocks = (g->nJ + 15) / 16;
   const uint64_t tiles = nLines * g->jBlocks;
