@@ -396,15 +396,26 @@ fastKronError Handle::execute(const KronProblem& p, const Plan& plan, void* temp
     if (logLevel() >= 2)
       printf("[fastkron]   launch %zu: factors [%u,%u] Kin=%llu Kout=%llu kernel %s\n", l, s.lo, s.hi,
              (unsigned long long)a.Kin, (unsigned long long)a.Kout, k.name.c_str());
-    if (dryRun) {
-      if (k.check && !k.check(k, a)) return fastKronKernelNotFound;
-      in = a.out; inBatch = a.out_batch;
-      continue;
-    }
-    hipError_t he = k.launch(k, a, stream_);
-    if (he != hipSuccess) {
-      fprintf(stderr, "[fastkron] launch of %s failed: %s\n", k.name.c_str(), hipGetErrorString(he));
-      return fastKronInvalidArgument;                 // reference cuda_kernel_db.cu:296-301
+    // The batch index is a grid dimension (at most 65535): larger batches go out in chunks of that many.
+    constexpr uint32_t kMaxGridBatch = 65535;
+    const size_t es = dtypeSize(p.dt);
+    for (uint32_t b0 = 0; b0 < a.batch; b0 += kMaxGridBatch) {
+      StepArgs c = a;
+      c.batch = a.batch - b0 < kMaxGridBatch ? a.batch - b0 : kMaxGridBatch;
+      c.in = (const char*)a.in + (size_t)b0 * a.in_batch * es;
+      c.out = (char*)a.out + (size_t)b0 * a.out_batch * es;
+      if (a.y) c.y = (const char*)a.y + (size_t)b0 * a.y_batch * es;
+      for (uint32_t j = 0; j < a.nf && j < kMaxFused; j++)
+        c.f[j] = (const char*)a.f[j] + (size_t)b0 * a.f_batch[j] * es;
+      if (dryRun) {
+        if (k.check && !k.check(k, c)) return fastKronKernelNotFound;
+        break;                                        // every chunk has the same strides and alignment class
+      }
+      hipError_t he = k.launch(k, c, stream_);
+      if (he != hipSuccess) {
+        fprintf(stderr, "[fastkron] launch of %s failed: %s\n", k.name.c_str(), hipGetErrorString(he));
+        return fastKronInvalidArgument;               // reference cuda_kernel_db.cu:296-301
+      }
     }
     in = a.out; inBatch = a.out_batch;
   }

@@ -565,3 +565,11 @@ def test_fp64_16x16_block_kernel(fk, M, Ps, launches):
     check(fk, ko.MKM, M, Ps, Ps, np.float64, alpha=1.0, beta=1.0, seed=503, batch=3, share_f=True)
     check(fk, ko.MKM, M, Ps, Ps, np.float64, alpha=2.0, beta=0.0, seed=504, batch=2)          # per-batch factors: other kernels
     check(fk, ko.MKM, M, Ps, Ps, np.float64, alpha=1.0, beta=1.0, seed=505, integer=True)
+
+
+@pytest.mark.parametrize("mm", [ko.MKM, ko.KMM])
+def test_more_batches_than_a_grid_dimension_holds(fk, mm):
+    """70000 small problems in one strided-batched call: the batch index is a grid dimension of at most 65535,
+    so the launches go out in chunks."""
+    check(fk, mm, 2, [4, 3], [3, 4], np.float32, alpha=1.5, beta=0.5, seed=601, batch=70000)
+    check(fk, mm, 3, [2, 2, 2], [2, 2, 2], np.float64, alpha=1.0, beta=0.0, seed=602, batch=66000, share_f=True)
