@@ -7,9 +7,9 @@
 //   phase A  lane = (m, 3 bits of (k1,k2,k3)), wave = the other 3 bits, registers = (k4,k5,k6): the three fast
 //            digits are contracted in registers with V_MFMA_F32_4X4X1_16B_F32 (16 independent 4x4 outer products
 //            per instruction: every lane gets its own outputs, D[i][lane] += F[4qq+i][p] * x_lane[p]);
-//   exchange one pass through LDS (128 KB + padding: index m*4168 + a*65 + b, a = (k1,k2,k3), b = (q4,q5,q6);
-//            the paddings make both the write, lanes along (m, a), and the read, lanes along (m, b), hit every
-//            bank exactly twice per 64-lane access);
+//   exchange one pass through LDS (128 KB + padding: index m*4164 + a*65 + b, a = (k1,k2,k3), b = (q4,q5,q6);
+//            the paddings spread both the write, lanes along (m, a), and the read, lanes along (m, b), over
+//            the banks: strides chosen by measuring the paired 4-byte accesses the compiler emits);
 //   phase B  registers = (k1,k2,k3), contracted the same way; the digits end up in place, so the result is in
 //            its final order;
 //   store    alpha / beta*Y applied; Y is requested at kernel start, right behind X.
@@ -31,7 +31,8 @@ typedef float k6f4 __attribute__((ext_vector_type(4)));
 #define K6MFMA(a, b, c) __builtin_amdgcn_mfma_f32_4x4x1f32((a), (b), (c), 0, 0, 0)
 
 constexpr int kK6Rows = 4096;               // 4^6
-constexpr int kK6MStride = 64 * 65 + 8;     // LDS words per column m: 64 rows a of 65 words, + 8
+constexpr int kK6MStride = 64 * 65 + 4;     // LDS words per column m: 64 rows a of 65 words, + 4 (measured: the
+                                            // fastest column stride for both sides of the exchange is 4 mod 8)
 constexpr size_t kK6LdsBytes = 8 * kK6MStride * sizeof(float);
 
 // Contract the three digits held in the registers of x (digit j has register stride 4^j) with the factors
