@@ -40,6 +40,7 @@ struct KernelInfo {
   uint32_t tileM, tileK;  // rows and input columns per workgroup (0: not tiled that way)
   uint32_t threads;
   uint32_t variant;       // kernel-family specific
+  bool     tunerOnly;     // a candidate for the tuner, never chosen by the online selection
   CanRunFn canRun;
   LaunchFn launch;
   CheckFn  check;

@@ -336,7 +336,11 @@ def test_long_chains_split_into_row_kernel_plus_leading_kmm(fk, M, Ps):
 @pytest.mark.parametrize("M,Ps", [(64, [8]), (70, [8] * 3), (64, [16]), (100, [16, 16]), (64, [4]), (80, [4, 4]), (64, [4] * 4)])
 def test_kmm_register_kernel_more_tiles(fk, M, Ps):
     check(fk, ko.KMM, M, Ps, Ps, np.float32, alpha=1.5, beta=0.5, seed=111)
-    assert all("mfma4x4x1" in k for _, _, k in fk.last_plan()), fk.last_plan()
+    # groups of 4x4 / 8x8 factors run on the register kernel; single factors are left to the plain kernel
+    plan = fk.last_plan()
+    assert all("mfma4x4x1" in k or hi == lo for lo, hi, k in plan), plan
+    if len(Ps) >= 2 and Ps[0] < 16:
+        assert any("mfma4x4x1" in k for _, _, k in plan), plan
     check(fk, ko.KMM, M, Ps, Ps, np.float32, alpha=1.0, beta=0.0, seed=112, batch=3)
 
 
@@ -360,7 +364,7 @@ def test_chains_split_into_pair_kernel_plus_leading_kmm_step(fk, M, Ps, dt):
     matrix-core steps across the blocks."""
     check(fk, ko.MKM, M, Ps, Ps, dt, alpha=1.5, beta=0.5, seed=131)
     plan = fk.last_plan()
-    assert len(plan) == len(Ps) - 1 and plan[0][2].startswith("mkm_") and all(k.startswith("kmm_") for _, _, k in plan[1:]), plan
+    assert len(plan) == len(Ps) - 1 and plan[0][2].startswith("mkm_") and all("kmm_" in k for _, _, k in plan[1:]), plan
     check(fk, ko.MKM, M, Ps, Ps, dt, alpha=1.0, beta=0.0, seed=132, opFs=ko.OP_T)
     check(fk, ko.MKM, M, Ps, Ps, dt, alpha=1.0, beta=1.0, seed=133, batch=2, share_f=True)
     check(fk, ko.MKM, M, Ps, Ps, dt, alpha=1.0, beta=1.0, seed=134, batch=2)
@@ -373,7 +377,9 @@ def test_kmm_layout_mfma_step_kernel(fk, M, Ps, dt):
     """GeKMM with 16..128-wide square factors on the matrix cores, tiles of 16 consecutive columns of X,
     including column counts that are not a multiple of 16."""
     check(fk, ko.KMM, M, Ps, Ps, dt, alpha=1.5, beta=0.5, seed=141)
-    assert all(k.startswith("kmm_") and "generic" not in k for _, _, k in fk.last_plan()), fk.last_plan()
+    # (fp32 16x16 is the exception: the plain kernel is faster there)
+    assert all((k.startswith("kmm_") and "generic" not in k) or (dt == np.float32 and Ps[lo] == 16)
+               for lo, _, k in fk.last_plan()), fk.last_plan()
     check(fk, ko.KMM, M, Ps, Ps, dt, alpha=1.0, beta=0.0, seed=142, opFs=ko.OP_T)
     check(fk, ko.KMM, M, Ps, Ps, dt, alpha=1.0, beta=1.0, seed=143, batch=2)
     check(fk, ko.KMM, M, Ps, Ps, dt, alpha=1.0, beta=0.0, seed=144, integer=True)

@@ -131,8 +131,8 @@ def test_gradient_of_x_only_is_one_fused_call(mm):
     w = torch.randint(0, 3, z.shape, generator=torch.Generator().manual_seed(5)).float().cuda()
     (z * w).sum().backward()
     plan = fk.default_handle().last_plan()
-    assert all("generic" not in k for _, _, k in plan), plan
     if mm == "mkm":
+        assert all("generic" not in k for _, _, k in plan), plan
         assert len(plan) == 1, plan                                    # the backward call: four fused 16x16 factors
     kron = fs[0]
     for f in fs[1:]:
