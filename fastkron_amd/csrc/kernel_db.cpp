@@ -47,6 +47,12 @@ static bool fusedSmallCanRun(const KernelInfo& k, const KronProblem& p, uint32_t
   uint32_t ps[kMaxFused], qs[kMaxFused];
   for (uint32_t j = 0; j < nf; j++) { ps[j] = p.P[hi - j]; qs[j] = p.Q[hi - j]; }
   const bool kmm = p.mm == MMType::KMM && p.M > 1;
+  // In the KMM layout the plain kernel already runs every factor at about 5 TB/s: fusing pays off only for
+  // groups of three or more factors of at most 6 rows (measured against tuned plans).
+  if (kmm) {
+    if (nf < 3) return false;
+    for (uint32_t j = 0; j < nf; j++) if (ps[j] > 6) return false;
+  }
   return fusedSmallFits(nf, ps, qs, p.colsBefore(hi), p.M, kmm, p.dt);
 }
 static hipError_t fusedSmallLaunch(const KernelInfo& k, const StepArgs& a, hipStream_t s) {
@@ -313,7 +319,8 @@ void registerRowKernels(std::vector<KernelInfo>& out) {
     kd.threads = 256; kd.variant = variant;
     kd.canRun = stepF64CanRun; kd.launch = stepF64Launch; kd.check = stepF64Check;
     // fp32 16x16 in the KMM layout: the plain kernel's 256-byte accesses along M beat the 64-byte tile rows
-    kd.tunerOnly = (variant == 1 && dt == DType::F32 && P == 16);
+    // and for 128x128 the padded step (factor in LDS instead of split over wave tasks) is a third faster
+    kd.tunerOnly = (variant == 1 && dt == DType::F32 && (P == 16 || P == 128));
     out.push_back(kd);
   }
 }

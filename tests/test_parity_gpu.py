@@ -378,7 +378,7 @@ def test_kmm_layout_mfma_step_kernel(fk, M, Ps, dt):
     including column counts that are not a multiple of 16."""
     check(fk, ko.KMM, M, Ps, Ps, dt, alpha=1.5, beta=0.5, seed=141)
     # (fp32 16x16 is the exception: the plain kernel is faster there)
-    assert all((k.startswith("kmm_") and "generic" not in k) or (dt == np.float32 and Ps[lo] == 16)
+    assert all(("kmm_" in k and "generic" not in k) or (dt == np.float32 and Ps[lo] == 16)
                for lo, _, k in fk.last_plan()), fk.last_plan()
     check(fk, ko.KMM, M, Ps, Ps, dt, alpha=1.0, beta=0.0, seed=142, opFs=ko.OP_T)
     check(fk, ko.KMM, M, Ps, Ps, dt, alpha=1.0, beta=1.0, seed=143, batch=2)
@@ -516,7 +516,10 @@ FUSED_SMALL = [
 def test_small_factors_of_any_shape_are_fused_through_lds(fk, mm, M, Ps, Qs, dt):
     check(fk, mm, M, Ps, Qs, dt, alpha=1.5, beta=0.5, seed=301)
     plan = fk.last_plan()
-    assert len(plan) < len(Ps) and any("small_fused" in k for _, _, k in plan), plan
+    # (in the KMM layout only groups of three or more factors of at most 6 rows are fused: the plain kernel is
+    # as fast as the fused one beyond that)
+    if mm == ko.MKM or (len(Ps) >= 3 and max(Ps) <= 6):
+        assert len(plan) < len(Ps) and any("small_fused" in k for _, _, k in plan), plan
     check(fk, mm, M, Ps, Qs, dt, alpha=1.0, beta=0.0, seed=302, opFs=ko.OP_T)
     check(fk, mm, M, Ps, Qs, dt, alpha=2.0, beta=1.0, seed=303, batch=3)          # per-batch factors
     check(fk, mm, M, Ps, Qs, dt, alpha=1.0, beta=0.0, seed=304, batch=2, share_f=True)
