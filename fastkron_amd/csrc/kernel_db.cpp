@@ -200,6 +200,16 @@ static bool kmm64CanRun(const KernelInfo&, const KronProblem& p, uint32_t lo, ui
 static hipError_t kmm64Launch(const KernelInfo&, const StepArgs& a, hipStream_t s) { return launchKmm64F64(a, s); }
 static bool kmm64Check(const KernelInfo&, const StepArgs& a) { return kmm64F64Supported(a); }
 
+// ---- KMM layout: two fused 16x16 factors ----
+static bool kmm16x2CanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
+                          const DeviceInfo&) {
+  if (p.dt != k.dt || p.mm != MMType::KMM || p.M < 2 || hi - lo + 1 != 2 || p.forward) return false;
+  for (uint32_t i = lo; i <= hi; i++) if (p.P[i] != 16 || p.Q[i] != 16) return false;
+  return !(first && p.opX == 2);
+}
+static hipError_t kmm16x2Launch(const KernelInfo& k, const StepArgs& a, hipStream_t s) { return launchKmm16x2(a, k.dt, s); }
+static bool kmm16x2Check(const KernelInfo& k, const StepArgs& a) { return kmm16x2Supported(a, k.dt); }
+
 // ---- KMM layout: six fused 4x4 fp32 factors covering all 4096 rows ----
 static bool kmm4x6CanRun(const KernelInfo&, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
                          const DeviceInfo& dev) {
@@ -250,6 +260,15 @@ void registerRowKernels(std::vector<KernelInfo>& out) {
   k32.dt = DType::F32; k32.P = 32; k32.Q = 16; k32.fused = 3; k32.tileM = 1; k32.tileK = 32768; k32.threads = 512;
   k32.variant = 0; k32.canRun = row32CanRun; k32.launch = row32Launch; k32.check = row32Check;
   out.push_back(k32);
+
+  for (DType dt : {DType::F32, DType::F64}) {
+    KernelInfo k2{};
+    k2.name = std::string("kmm_hip_gfx950_256_") + (dt == DType::F32 ? "f" : "d") +
+              "_16x16_16x16_2_16x256_mfma16x16x4_NN_strided_0_3";
+    k2.dt = dt; k2.P = 16; k2.Q = 16; k2.fused = 2; k2.tileM = 16; k2.tileK = 256; k2.threads = 256; k2.variant = 0;
+    k2.canRun = kmm16x2CanRun; k2.launch = kmm16x2Launch; k2.check = kmm16x2Check;
+    out.push_back(k2);
+  }
 
   {
     KernelInfo kd3{};

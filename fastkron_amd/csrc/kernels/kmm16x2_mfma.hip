@@ -1,0 +1,194 @@
+// Two fused 16x16 factors in the KMM layout (element (m, col) at m + col*M, the M index contiguous), fp32 or fp64:
+// half the launches and half the HBM passes of sgekmm / dgekmm chains of 16x16 factors, and of the leading
+// factors of long GeMKM chains (which run as KMM problems over contiguous blocks).
+//
+//   out[(q0, q1, s), m] = sum_{k0,k1} in[(s, k0, k1), m] * F0[k0,q0] * F1[k1,q1]      (s: slice, S = Kin / 256)
+//
+// A wave owns a tile of one slice and 16 consecutive m: 256 x 16 elements, kept in registers; no LDS exchange,
+// no barrier.
+//   k1   for each k0 one V_MFMA_*_16X16X4 group, computed transposed: D[q1][m] = sum_k1 F1^T[q1][k1] X[k1][m].
+//        B operand lane = 16*k + m reads rows k1 = 4*c + k (16 consecutive m per quarter wave and product), the A
+//        operand is F1 in registers.  The results z[k0][r] = T[k0][q1 = row(r, lane/16)][m = lane%16] stay in
+//        16 x 4 registers.
+//   k0   contracted over the register index on the vector ALU, F0 read from LDS as broadcast pairs.
+//   store  per q0 a lane holds four values, rows q1 = row(r, lane/16): every quarter wave writes 16 consecutive m.
+//
+// The reference's GPU kernels fuse factors through shared memory on CUDA cores (reference
+// src/kernels/cuda/kernel.cuh:165-219); its x86 KMM kernels vectorise along M as this one does (reference
+// src/kernels/cpu/kernel.h:124-126).
+// Algorithmic traffic per launch: read M*Kin, write M*Kin elements (+ M*Kin for Y on the launch that writes Z).
+#include <hip/hip_runtime.h>
+#include "../problem.h"
+#include "launch.h"
+
+namespace fk {
+
+typedef double k2d4 __attribute__((ext_vector_type(4)));
+typedef float k2f4 __attribute__((ext_vector_type(4)));
+
+template <typename T> struct K2Mfma;
+template <> struct K2Mfma<double> {
+  using Acc = k2d4;
+  static __device__ __forceinline__ Acc mma(double a, double b, Acc c) {
+    return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ int row(int r, int hi) { return 4 * r + hi; }
+};
+template <> struct K2Mfma<float> {
+  using Acc = k2f4;
+  static __device__ __forceinline__ Acc mma(float a, float b, Acc c) {
+    return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ int row(int r, int hi) { return 4 * hi + r; }
+};
+
+constexpr int kK2Waves = 4;
+constexpr int kK2Win = 3;              // k0 slices of a tile in flight
+
+template <typename T, bool HAS_Y>
+__global__ __launch_bounds__(256, 2) void kron_kmm16x2_kernel(const StepArgs a, const uint32_t mTiles,
+                                                              const uint32_t totalTiles) {
+  using MF = K2Mfma<T>;
+  using Acc = typename MF::Acc;
+  typedef T V2 __attribute__((ext_vector_type(2)));
+  __shared__ __align__(16) T f0s[256];              // F0 transposed: f0s[q0*16 + k0]
+  const int tid = threadIdx.x;
+  const int l0 = tid & 63;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lo = l0 & 15, hi = l0 >> 4;
+  const uint32_t bt = blockIdx.y;
+  const uint64_t S = a.Kin / 256;
+  const uint64_t M = a.M;
+
+  // a.f[0] is the later factor F1 (contracts the fast digit k1), a.f[1] = F0
+  {
+    const T* F0 = (const T*)a.f[1] + (size_t)bt * a.f_batch[1];
+    const int q0 = tid >> 4, k0 = tid & 15;
+    f0s[tid] = F0[(int64_t)k0 * a.f_sp[1] + (int64_t)q0 * a.f_sq[1]];
+  }
+  T f1[4];                                          // A operand: F1[k1 = 4*c + hi][q1 = lo]
+  {
+    const T* F1 = (const T*)a.f[0] + (size_t)bt * a.f_batch[0];
+#pragma unroll
+    for (int c = 0; c < 4; c++) f1[c] = F1[(int64_t)(4 * c + hi) * a.f_sp[0] + (int64_t)lo * a.f_sq[0]];
+  }
+  __syncthreads();
+
+  const T* inB = (const T*)a.in + (size_t)bt * a.in_batch;
+  T* outB = (T*)a.out + (size_t)bt * a.out_batch;
+  const T* YB = HAS_Y ? (const T*)a.y + (size_t)bt * a.y_batch : nullptr;
+  const T alpha = a.epilogue ? (T)a.alpha : (T)1, beta = (T)a.beta;
+
+  const uint32_t nWaves = gridDim.x * kK2Waves;
+  // x[c] = X[(s, k0, k1 = 4*c + hi), m]; columns beyond M are clamped to the tile's first one (computed, not stored)
+  // The rows are read in the order (k0, c): row k0*16 + 4*c + hi, four rows further with every load, so one
+  // running pointer serves the whole tile.
+  const uint64_t rowStep = 4 * (uint64_t)a.in_ldc;
+  auto loadSlice = [&](const T*& xp, T (&x)[4]) {
+#pragma unroll
+    for (int c = 0; c < 4; c++) { x[c] = *xp; xp += rowStep; }
+  };
+
+  for (uint32_t t = blockIdx.x * kK2Waves + w; t < totalTiles; t += nWaves) {
+    const uint64_t s = t / mTiles;
+    const uint32_t m0 = (uint32_t)(t - s * mTiles) * 16;
+    const bool mOk = m0 + lo < M;
+    const uint32_t m = mOk ? m0 + lo : m0;
+    const T* xp = inB + m + (s * 256 + hi) * (uint64_t)a.in_ldc;
+
+    T z[16][4];
+    T xw[kK2Win][4];
+#pragma unroll
+    for (int k = 0; k < kK2Win; k++) loadSlice(xp, xw[k]);
+#pragma unroll
+    for (int k0 = 0; k0 < 16; k0++) {
+      T x[4];
+#pragma unroll
+      for (int c = 0; c < 4; c++) x[c] = xw[k0 % kK2Win][c];
+      if (k0 + kK2Win < 16) loadSlice(xp, xw[k0 % kK2Win]);
+      Acc d = (Acc){0, 0, 0, 0};
+#pragma unroll
+      for (int c = 0; c < 4; c++) d = MF::mma(f1[c], x[c], d);         // d[q1][m]
+#pragma unroll
+      for (int r = 0; r < 4; r++) z[k0][r] = d[r];
+      __builtin_amdgcn_sched_barrier(0);             // keeps the loads of later slices from being hoisted up here
+    }
+
+    // ---- k0 on the vector ALU, one q0 at a time, and the stores ----
+    // output row (q0, q1 = row(r, hi)): a running pointer per lane, 16 rows further with every q0
+    const uint64_t oq = S * (uint64_t)a.out_ldc, yq = HAS_Y ? S * (uint64_t)a.y_ldc : 0;   // stride of one output row q
+    const uint64_t rs = (uint64_t)(MF::row(1, 0) - MF::row(0, 0));                        // rows between two registers
+    T* op = outB + m + s * (uint64_t)a.out_ldc + (uint64_t)MF::row(0, hi) * oq;
+    const T* yp = HAS_Y ? YB + m + s * (uint64_t)a.y_ldc + (uint64_t)MF::row(0, hi) * yq : nullptr;
+#pragma unroll 1
+    for (int q0 = 0; q0 < 16; q0++) {
+      T yv[4];
+      if (HAS_Y) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) yv[r] = mOk ? yp[r * rs * yq] : (T)0;
+        yp += 16 * yq;
+      }
+      T acc[4] = {0, 0, 0, 0};
+#pragma unroll
+      for (int k = 0; k < 16; k += 2) {
+        const V2 f = *(const V2*)&f0s[q0 * 16 + k];
+#pragma unroll
+        for (int r = 0; r < 4; r++) acc[r] += f[0] * z[k][r];
+#pragma unroll
+        for (int r = 0; r < 4; r++) acc[r] += f[1] * z[k + 1][r];
+      }
+      if (mOk) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          T v = acc[r] * alpha;
+          if (HAS_Y) v += beta * yv[r];
+          op[r * rs * oq] = v;
+        }
+      }
+      op += 16 * oq;
+    }
+  }
+}
+
+bool kmm16x2Supported(const StepArgs& a, DType dt) {
+  if (a.nf != 2) return false;
+  for (uint32_t j = 0; j < 2; j++) if (a.p[j] != 16 || a.q[j] != 16) return false;
+  if (a.Kin % 256 || a.Kout != a.Kin) return false;
+  // the M index contiguous in the input, the output and Y
+  if (a.in_ldm != 1 || a.out_ldm != 1 || (a.y && a.y_ldm != 1)) return false;
+  const uint64_t tiles = (a.Kin / 256) * ((a.M + 15) / 16);
+  (void)dt;
+  return tiles < (1ull << 31) && a.batch <= 65535;
+}
+
+template <typename T>
+static hipError_t launchKmm16x2T(const StepArgs& a, hipStream_t stream) {
+  static int cus = 0;
+  if (!cus) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    cus = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+              ? prop.multiProcessorCount : 256;
+  }
+  const uint32_t mTiles = (a.M + 15) / 16;
+  const uint32_t totalTiles = (uint32_t)((a.Kin / 256) * mTiles);
+  // persistent waves: two workgroups of four waves per CU (two waves per SIMD)
+  uint32_t wgs = (uint32_t)cus * 2;
+  if (a.batch > 1) wgs = (wgs + a.batch - 1) / a.batch;
+  const uint32_t need = (totalTiles + kK2Waves - 1) / kK2Waves;
+  if (wgs > need) wgs = need;
+  if (wgs == 0) wgs = 1;
+  dim3 grid(wgs, a.batch), block(256);
+  if (a.y && a.epilogue)
+    hipLaunchKernelGGL((kron_kmm16x2_kernel<T, true>), grid, block, 0, stream, a, mTiles, totalTiles);
+  else
+    hipLaunchKernelGGL((kron_kmm16x2_kernel<T, false>), grid, block, 0, stream, a, mTiles, totalTiles);
+  return hipGetLastError();
+}
+
+hipError_t launchKmm16x2(const StepArgs& a, DType dt, hipStream_t stream) {
+  if (!kmm16x2Supported(a, dt)) return hipErrorInvalidValue;
+  return dt == DType::F32 ? launchKmm16x2T<float>(a, stream) : launchKmm16x2T<double>(a, stream);
+}
+
+}  // namespace fk

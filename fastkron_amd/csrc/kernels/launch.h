@@ -40,6 +40,11 @@ hipError_t launchRow16x3F64(const StepArgs& a, hipStream_t stream);
 bool stepAnyMfmaSupported(const StepArgs& a, DType dt);
 hipError_t launchStepAnyMfma(const StepArgs& a, DType dt, hipStream_t stream);
 
+// Two fused 16x16 factors on the KMM layout, fp32 or fp64: matrix cores for one digit, vector FMAs over the
+// register index for the other; 256 x 16 tiles in registers.
+bool kmm16x2Supported(const StepArgs& a, DType dt);
+hipError_t launchKmm16x2(const StepArgs& a, DType dt, hipStream_t stream);
+
 // One step with a 64x64 fp64 factor on the KMM layout (4x4x4 matrix-core instruction, 64-column tiles).
 bool kmm64F64Supported(const StepArgs& a);
 hipError_t launchKmm64F64(const StepArgs& a, hipStream_t stream);

@@ -338,7 +338,7 @@ def test_kmm_register_kernel_more_tiles(fk, M, Ps):
     check(fk, ko.KMM, M, Ps, Ps, np.float32, alpha=1.5, beta=0.5, seed=111)
     # groups of 4x4 / 8x8 factors run on the register kernel; single factors are left to the plain kernel
     plan = fk.last_plan()
-    assert all("mfma4x4x1" in k or hi == lo for lo, hi, k in plan), plan
+    assert all("mfma4x4x1" in k or hi == lo or "_16x16_16x16_2_" in k for lo, hi, k in plan), plan
     if len(Ps) >= 2 and Ps[0] < 16:
         assert any("mfma4x4x1" in k for _, _, k in plan), plan
     check(fk, ko.KMM, M, Ps, Ps, np.float32, alpha=1.0, beta=0.0, seed=112, batch=3)
@@ -560,7 +560,7 @@ def test_any_shape_step_on_the_matrix_cores(fk, mm, M, Ps, Qs, dt):
     (5, [16] * 3, 1),               # a block per row
     (32, [16, 16], 1),              # two factors: 16 rows per block, identity in the leading slot
     (3, [16] * 4, 2),               # three trailing factors in place on 48 virtual rows + one leading launch
-    (1, [16] * 5, 3),
+    (1, [16] * 5, 2),               # the two leading factors as one KMM-layout pair launch
     (2, [4, 8, 16, 16, 16], None),  # merged leading factors
 ])
 def test_fp64_16x16_block_kernel(fk, M, Ps, launches):
@@ -582,3 +582,16 @@ def test_more_batches_than_a_grid_dimension_holds(fk, mm):
     so the launches go out in chunks."""
     check(fk, mm, 2, [4, 3], [3, 4], np.float32, alpha=1.5, beta=0.5, seed=601, batch=70000)
     check(fk, mm, 3, [2, 2, 2], [2, 2, 2], np.float64, alpha=1.0, beta=0.0, seed=602, batch=66000, share_f=True)
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+@pytest.mark.parametrize("M,Ps,launches", [(16, [16, 16], 1), (37, [16] * 4, 2), (100, [16] * 3, 2), (5, [3, 16, 16], 2),
+                                           (2048, [16, 16], 1)])
+def test_kmm_layout_pair_of_16x16_factors(fk, M, Ps, launches, dt):
+    """GeKMM chains of 16x16 factors: two factors per launch, tiles of 16 columns of X including ragged ones."""
+    check(fk, ko.KMM, M, Ps, Ps, dt, alpha=1.5, beta=0.5, seed=701)
+    plan = fk.last_plan()
+    assert any("_16x16_16x16_2_16x256_" in k for _, _, k in plan) and len(plan) == launches, plan
+    check(fk, ko.KMM, M, Ps, Ps, dt, alpha=1.0, beta=0.0, seed=702, opFs=ko.OP_T)
+    check(fk, ko.KMM, M, Ps, Ps, dt, alpha=1.0, beta=1.0, seed=703, batch=3)
+    check(fk, ko.KMM, M, Ps, Ps, dt, alpha=1.0, beta=0.0, seed=704, integer=True)
