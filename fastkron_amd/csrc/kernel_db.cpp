@@ -135,11 +135,11 @@ static bool row8CanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, u
 static hipError_t row8Launch(const KernelInfo&, const StepArgs& a, hipStream_t s) { return launchRow8x5(a, s); }
 static bool row8Check(const KernelInfo&, const StepArgs& a) { return row8x5Supported(a); }
 
-// ---- wave-per-block kernel for two or three fused 16x16 fp64 factors ----
-static bool row16x3F64CanRun(const KernelInfo&, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
-                             const DeviceInfo&) {
+// ---- wave-per-block kernel for two or three fused 16x16 factors ----
+static bool row16x3CanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
+                          const DeviceInfo&) {
   const uint32_t nf = hi - lo + 1;
-  if (p.dt != DType::F64 || p.mm != MMType::MKM || nf < 2 || nf > 3 || p.forward) return false;
+  if (p.dt != k.dt || p.mm != MMType::MKM || nf < 2 || nf > 3 || p.forward) return false;
   uint64_t kk = 1;
   for (uint32_t i = lo; i <= hi; i++) {
     if (p.P[i] != 16 || p.Q[i] != 16) return false;
@@ -149,8 +149,8 @@ static bool row16x3F64CanRun(const KernelInfo&, const KronProblem& p, uint32_t l
   if (p.colsBefore(hi) != kk || (nf == 2 && p.M % 16)) return false;
   return !(first && p.opX == 2);
 }
-static hipError_t row16x3F64Launch(const KernelInfo&, const StepArgs& a, hipStream_t s) { return launchRow16x3F64(a, s); }
-static bool row16x3F64Check(const KernelInfo&, const StepArgs& a) { return row16x3F64Supported(a); }
+static hipError_t row16x3Launch(const KernelInfo& k, const StepArgs& a, hipStream_t s) { return launchRow16x3(a, k.dt, s); }
+static bool row16x3Check(const KernelInfo& k, const StepArgs& a) { return row16x3Supported(a, k.dt); }
 
 // ---- whole-row kernel for three fused 32x16 fp32 factors ----
 static bool row32CanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
@@ -239,6 +239,17 @@ static bool kmmRegCheck(const KernelInfo&, const StepArgs& a) { return kmmRegSup
 
 void registerRowKernels(std::vector<KernelInfo>& out) {
   // grammar: <mm>_<backend>_<arch>_<threads>_<type>_<PxQ>_<TilePxTileQ>_<fused>_<TileMxTileK>_<regs>_<ops>_<batch>_<p2p>_<opt>
+  // two or three 16x16 factors: one wave per 4096-element block (measured faster than the workgroup kernel below on
+  // three factors, 4.6 against 4.1 TB/s in fp32, and free of its row-count conditions)
+  for (DType dt : {DType::F64, DType::F32}) {
+    KernelInfo kd3{};
+    kd3.name = std::string("mkm_hip_gfx950_256_") + (dt == DType::F64 ? "d" : "f") +
+               "_16x16_16x16_3_1x4096_mfma16x16x4_NN_strided_0_3";
+    kd3.dt = dt; kd3.P = 16; kd3.Q = 16; kd3.fused = 3; kd3.tileM = 1; kd3.tileK = 4096; kd3.threads = 256;
+    kd3.variant = 0; kd3.canRun = row16x3CanRun; kd3.launch = row16x3Launch; kd3.check = row16x3Check;
+    out.push_back(kd3);
+  }
+
   // two builds of the 16x16 whole-block kernel: 16 waves (preferred online), 8 waves with the whole next block
   // prefetched (a candidate for the tuner)
   for (uint32_t threads : {1024u, 512u}) {
@@ -268,14 +279,6 @@ void registerRowKernels(std::vector<KernelInfo>& out) {
     k2.dt = dt; k2.P = 16; k2.Q = 16; k2.fused = 2; k2.tileM = 16; k2.tileK = 256; k2.threads = 256; k2.variant = 0;
     k2.canRun = kmm16x2CanRun; k2.launch = kmm16x2Launch; k2.check = kmm16x2Check;
     out.push_back(k2);
-  }
-
-  {
-    KernelInfo kd3{};
-    kd3.name = "mkm_hip_gfx950_256_d_16x16_16x16_3_1x4096_mfma16x16x4_NN_strided_0_3";
-    kd3.dt = DType::F64; kd3.P = 16; kd3.Q = 16; kd3.fused = 3; kd3.tileM = 1; kd3.tileK = 4096; kd3.threads = 256;
-    kd3.variant = 0; kd3.canRun = row16x3F64CanRun; kd3.launch = row16x3F64Launch; kd3.check = row16x3F64Check;
-    out.push_back(kd3);
   }
 
   {

@@ -32,9 +32,9 @@ hipError_t launchPairMfma(const StepArgs& a, DType dt, hipStream_t stream);
 bool stepMfmaSupported(const StepArgs& a, DType dt);
 hipError_t launchStepMfma(const StepArgs& a, DType dt, hipStream_t stream);
 
-// Two or three fused 16x16 fp64 factors on blocks of 4096 doubles (MKM layout), one wave per block.
-bool row16x3F64Supported(const StepArgs& a);
-hipError_t launchRow16x3F64(const StepArgs& a, hipStream_t stream);
+// Two or three fused 16x16 factors on blocks of 4096 elements (MKM layout), fp64 or fp32, one wave per block.
+bool row16x3Supported(const StepArgs& a, DType dt);
+hipError_t launchRow16x3(const StepArgs& a, DType dt, hipStream_t stream);
 
 // One step with a factor of any shape up to 256x512 on the matrix cores (zero padded), fp64 or fp32, any layout.
 bool stepAnyMfmaSupported(const StepArgs& a, DType dt);

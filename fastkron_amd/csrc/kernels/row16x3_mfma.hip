@@ -1,6 +1,6 @@
-// Three fused 16x16 fp64 factors on contiguous blocks of 16^3 = 4096 doubles (dgemkm with 16x16^3, or the three
-// trailing factors of a longer chain applied block by block): one wave owns a block, keeps it in registers and
-// needs neither an LDS exchange nor a barrier.
+// Three fused 16x16 factors on contiguous blocks of 16^3 = 4096 elements (dgemkm with 16x16^3, or the three
+// trailing factors of a longer chain applied block by block; fp32 where the 16x16^4 workgroup kernel does not
+// apply): one wave owns a block, keeps it in registers and needs neither an LDS exchange nor a barrier.
 //
 //   Z[q1,q2,q3] = alpha * sum_{k1,k2,k3} X[k1,k2,k3] F1[k1,q1] F2[k2,q2] F3[k3,q3]  (+ beta*Y)
 //
@@ -24,19 +24,38 @@
 namespace fk {
 
 typedef double r3d4 __attribute__((ext_vector_type(4)));
-typedef double r3d2 __attribute__((ext_vector_type(2)));
+typedef float r3f4 __attribute__((ext_vector_type(4)));
 
-#define R3MFMA(a, b, c) __builtin_amdgcn_mfma_f64_16x16x4f64((a), (b), (c), 0, 0, 0)
+// accumulator layouts of the two 16x16x4 instructions: row(r, hi) = output row held by register r in the lane
+// group hi = lane / 16
+template <typename T> struct R3Mfma;
+template <> struct R3Mfma<double> {
+  using Acc = r3d4;
+  static __device__ __forceinline__ Acc mma(double a, double b, Acc c) {
+    return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ int row(int r, int hi) { return 4 * r + hi; }
+};
+template <> struct R3Mfma<float> {
+  using Acc = r3f4;
+  static __device__ __forceinline__ Acc mma(float a, float b, Acc c) {
+    return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ int row(int r, int hi) { return 4 * hi + r; }
+};
 
 constexpr int kR3Block = 4096;
 constexpr int kR3Waves = 4;
 constexpr int kR3Ahead = 2;            // k1 slices of the next block requested before the last contraction
 constexpr int kR3Win = 2;              // further slices in flight while a block is contracted
 
-template <bool HAS_Y>
-__global__ __launch_bounds__(256, 2) void kron_row16x3_f64_kernel(const StepArgs a, const uint32_t blocksPerBatch,
-                                                                  const uint32_t totalBlocks) {
-  __shared__ __align__(16) double f1s[256];          // F1 transposed: f1s[q1*16 + k1]
+template <typename T, bool HAS_Y>
+__global__ __launch_bounds__(256, 2) void kron_row16x3_kernel(const StepArgs a, const uint32_t blocksPerBatch,
+                                                              const uint32_t totalBlocks) {
+  using MF = R3Mfma<T>;
+  using Acc = typename MF::Acc;
+  typedef T V2 __attribute__((ext_vector_type(2)));
+  __shared__ __align__(16) T f1s[256];               // F1 transposed: f1s[q1*16 + k1]
   const int tid = threadIdx.x;
   const int l0 = tid & 63;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -46,19 +65,20 @@ __global__ __launch_bounds__(256, 2) void kron_row16x3_f64_kernel(const StepArgs
   // Factors shared by the whole launch only: per-batch factors are left to other kernels.
   {
     const int q1 = tid >> 4, k1 = tid & 15;
-    double v = (q1 == k1) ? 1.0 : 0.0;
-    if (a.nf == 3) v = ((const double*)a.f[2])[(int64_t)k1 * a.f_sp[2] + (int64_t)q1 * a.f_sq[2]];
+    T v = (q1 == k1) ? (T)1 : (T)0;
+    if (a.nf == 3) v = ((const T*)a.f[2])[(int64_t)k1 * a.f_sp[2] + (int64_t)q1 * a.f_sq[2]];
     f1s[tid] = v;
   }
-  // operands of the two products: F3[4*hi + c][lo] and F2[4*r + hi][lo]
-  double f3[4], f2[4];
+  // operands of the two products: F3[4*hi + c][lo] and F2[row(r, hi)][lo] (the rows the first product leaves
+  // in register r of this lane group)
+  T f3[4], f2[4];
   {
-    const double* F3 = (const double*)a.f[0];
-    const double* F2 = (const double*)a.f[1];
+    const T* F3 = (const T*)a.f[0];
+    const T* F2 = (const T*)a.f[1];
 #pragma unroll
     for (int c = 0; c < 4; c++) {
       f3[c] = F3[(int64_t)(4 * hi + c) * a.f_sp[0] + (int64_t)lo * a.f_sq[0]];
-      f2[c] = F2[(int64_t)(4 * c + hi) * a.f_sp[1] + (int64_t)lo * a.f_sq[1]];
+      f2[c] = F2[(int64_t)MF::row(c, hi) * a.f_sp[1] + (int64_t)lo * a.f_sq[1]];
     }
   }
   __syncthreads();
@@ -68,46 +88,51 @@ __global__ __launch_bounds__(256, 2) void kron_row16x3_f64_kernel(const StepArgs
   if (blk >= totalBlocks) return;
 
   auto blockPtr = [&](uint32_t b) {
-    return (const double*)a.in + (size_t)(b / blocksPerBatch) * a.in_batch + (size_t)(b % blocksPerBatch) * kR3Block;
+    return (const T*)a.in + (size_t)(b / blocksPerBatch) * a.in_batch + (size_t)(b % blocksPerBatch) * kR3Block;
   };
-  // x[c] = X[k1][k2 = lo][k3 = 4*hi + c]
-  auto loadSlice = [&](const double* X, int k1, double (&x)[4]) {
-    const double* xp = X + k1 * 256 + lo * 16 + hi * 4;
-    const r3d2 v0 = *(const r3d2*)xp, v1 = *(const r3d2*)(xp + 2);
-    x[0] = v0[0]; x[1] = v0[1]; x[2] = v1[0]; x[3] = v1[1];
+  // x[c] = X[k1][k2 = lo][k3 = 4*hi + c]: 16-byte loads
+  auto loadSlice = [&](const T* X, int k1, T (&x)[4]) {
+    const T* xp = X + k1 * 256 + lo * 16 + hi * 4;
+    if (sizeof(T) == 8) {
+      const V2 v0 = *(const V2*)xp, v1 = *(const V2*)(xp + 2);
+      x[0] = v0[0]; x[1] = v0[1]; x[2] = v1[0]; x[3] = v1[1];
+    } else {
+      const Acc v = *(const Acc*)xp;
+      x[0] = v[0]; x[1] = v[1]; x[2] = v[2]; x[3] = v[3];
+    }
   };
 
-  double xa[kR3Ahead][4];                            // the first slices of the block about to be processed
+  T xa[kR3Ahead][4];                                 // the first slices of the block about to be processed
   {
-    const double* X = blockPtr(blk);
+    const T* X = blockPtr(blk);
 #pragma unroll
     for (int k = 0; k < kR3Ahead; k++) loadSlice(X, k, xa[k]);
   }
 
   auto processBlock = [&](const uint32_t blk) {
-    const double* X = blockPtr(blk);
+    const T* X = blockPtr(blk);
     const size_t bt = blk / blocksPerBatch, m = blk % blocksPerBatch;
-    double* Z = (double*)a.out + bt * a.out_batch + m * kR3Block;
-    const double* Y = HAS_Y ? (const double*)a.y + bt * a.y_batch + m * kR3Block : nullptr;
+    T* Z = (T*)a.out + bt * a.out_batch + m * kR3Block;
+    const T* Y = HAS_Y ? (const T*)a.y + bt * a.y_batch + m * kR3Block : nullptr;
 
-    // ---- k3 and k2, slice by slice; z[k1][r] = T[k1][q2 = 4r + hi][q3 = lo] ----
-    double z[16][4];
-    double xb[kR3Win][4];                            // rolling window of slices in flight
+    // ---- k3 and k2, slice by slice; z[k1][r] = T[k1][q2 = row(r, hi)][q3 = lo] ----
+    T z[16][4];
+    T xb[kR3Win][4];                                 // rolling window of slices in flight
 #pragma unroll
     for (int k = 0; k < kR3Win; k++) loadSlice(X, kR3Ahead + k, xb[k]);
 #pragma unroll
     for (int k1 = 0; k1 < 16; k1++) {
-      double x[4];
+      T x[4];
 #pragma unroll
       for (int c = 0; c < 4; c++)
         x[c] = (k1 < kR3Ahead) ? xa[k1 < kR3Ahead ? k1 : 0][c] : xb[(k1 - kR3Ahead) % kR3Win][c];
       if (k1 >= kR3Ahead && k1 + kR3Win < 16) loadSlice(X, k1 + kR3Win, xb[(k1 - kR3Ahead) % kR3Win]);
-      r3d4 d = {0, 0, 0, 0};
+      Acc d = (Acc){0, 0, 0, 0};
 #pragma unroll
-      for (int c = 0; c < 4; c++) d = R3MFMA(x[c], f3[c], d);          // d[k2][q3]
-      r3d4 e = {0, 0, 0, 0};
+      for (int c = 0; c < 4; c++) d = MF::mma(x[c], f3[c], d);         // d[k2][q3]
+      Acc e = (Acc){0, 0, 0, 0};
 #pragma unroll
-      for (int r = 0; r < 4; r++) e = R3MFMA(f2[r], d[r], e);          // e[q2][q3]
+      for (int r = 0; r < 4; r++) e = MF::mma(f2[r], d[r], e);         // e[q2][q3]
 #pragma unroll
       for (int r = 0; r < 4; r++) z[k1][r] = e[r];
       __builtin_amdgcn_sched_barrier(0);             // keeps the loads of later slices from being hoisted up here
@@ -116,26 +141,26 @@ __global__ __launch_bounds__(256, 2) void kron_row16x3_f64_kernel(const StepArgs
     // ---- the first slices of the wave's next block stream in under the last contraction ----
     {
       const uint32_t nx = blk + nWaves;
-      const double* Xn = blockPtr(nx < totalBlocks ? nx : blk);
+      const T* Xn = blockPtr(nx < totalBlocks ? nx : blk);
 #pragma unroll
       for (int k = 0; k < kR3Ahead; k++) loadSlice(Xn, k, xa[k]);
     }
 
     // ---- k1 on the vector ALU, one q1 at a time, and the stores ----
-    const double alpha = a.epilogue ? a.alpha : 1.0, beta = a.beta;
-    double* zp = Z + hi * 16 + lo;
-    const double* yp = HAS_Y ? Y + hi * 16 + lo : nullptr;
+    const T alpha = a.epilogue ? (T)a.alpha : (T)1, beta = (T)a.beta;
+    T* zp = Z + lo;
+    const T* yp = HAS_Y ? Y + lo : nullptr;
 #pragma unroll 1
     for (int q1 = 0; q1 < 16; q1++) {
-      double yv[4];
+      T yv[4];
       if (HAS_Y) {
 #pragma unroll
-        for (int r = 0; r < 4; r++) yv[r] = yp[q1 * 256 + r * 64];
+        for (int r = 0; r < 4; r++) yv[r] = yp[q1 * 256 + MF::row(r, hi) * 16];
       }
-      double acc[4] = {0, 0, 0, 0};
+      T acc[4] = {0, 0, 0, 0};
 #pragma unroll
       for (int k = 0; k < 16; k += 2) {
-        const r3d2 f = *(const r3d2*)&f1s[q1 * 16 + k];
+        const V2 f = *(const V2*)&f1s[q1 * 16 + k];
 #pragma unroll
         for (int r = 0; r < 4; r++) acc[r] += f[0] * z[k][r];
 #pragma unroll
@@ -143,9 +168,9 @@ __global__ __launch_bounds__(256, 2) void kron_row16x3_f64_kernel(const StepArgs
       }
 #pragma unroll
       for (int r = 0; r < 4; r++) {
-        double v = acc[r] * alpha;
+        T v = acc[r] * alpha;
         if (HAS_Y) v += beta * yv[r];
-        zp[q1 * 256 + r * 64] = v;                   // Z[q1][q2 = 4r + hi][q3 = lo]
+        zp[q1 * 256 + MF::row(r, hi) * 16] = v;      // Z[q1][q2 = row(r, hi)][q3 = lo]
       }
     }
   };
@@ -156,7 +181,7 @@ __global__ __launch_bounds__(256, 2) void kron_row16x3_f64_kernel(const StepArgs
   for (blk += nWaves; blk < totalBlocks; blk += nWaves) processBlock(blk);
 }
 
-bool row16x3F64Supported(const StepArgs& a) {
+bool row16x3Supported(const StepArgs& a, DType dt) {
   if (a.nf != 2 && a.nf != 3) return false;
   uint64_t k = 1;
   for (uint32_t j = 0; j < a.nf; j++) {
@@ -169,13 +194,13 @@ bool row16x3F64Supported(const StepArgs& a) {
   if ((uint64_t)a.in_ldm != k || (uint64_t)a.out_ldm != k || (a.y && (uint64_t)a.y_ldm != k)) return false;
   if (a.nf == 2 && a.M % 16) return false;
   // 16-byte loads
-  if (((uintptr_t)a.in & 15) || (a.in_batch & 1)) return false;
+  if (((uintptr_t)a.in & 15) || (a.in_batch * dtypeSize(dt)) % 16) return false;
   const uint64_t blocks = (uint64_t)(a.nf == 2 ? a.M / 16 : a.M) * a.batch;
   return blocks < (1ull << 32);
 }
 
-hipError_t launchRow16x3F64(const StepArgs& a, hipStream_t stream) {
-  if (!row16x3F64Supported(a)) return hipErrorInvalidValue;
+hipError_t launchRow16x3(const StepArgs& a, DType dt, hipStream_t stream) {
+  if (!row16x3Supported(a, dt)) return hipErrorInvalidValue;
   static int cus = 0;
   if (!cus) {
     int dev = 0;
@@ -190,10 +215,15 @@ hipError_t launchRow16x3F64(const StepArgs& a, hipStream_t stream) {
   const uint64_t need = (total + kR3Waves - 1) / kR3Waves;
   if (wgs > need) wgs = (uint32_t)need;
   dim3 grid(wgs), block(256);
-  if (a.y && a.epilogue)
-    hipLaunchKernelGGL(kron_row16x3_f64_kernel<true>, grid, block, 0, stream, a, blocksPerBatch, (uint32_t)total);
-  else
-    hipLaunchKernelGGL(kron_row16x3_f64_kernel<false>, grid, block, 0, stream, a, blocksPerBatch, (uint32_t)total);
+  const bool y = a.y && a.epilogue;
+  const uint32_t tb = (uint32_t)total;
+  if (dt == DType::F64) {
+    if (y) hipLaunchKernelGGL((kron_row16x3_kernel<double, true>), grid, block, 0, stream, a, blocksPerBatch, tb);
+    else   hipLaunchKernelGGL((kron_row16x3_kernel<double, false>), grid, block, 0, stream, a, blocksPerBatch, tb);
+  } else {
+    if (y) hipLaunchKernelGGL((kron_row16x3_kernel<float, true>), grid, block, 0, stream, a, blocksPerBatch, tb);
+    else   hipLaunchKernelGGL((kron_row16x3_kernel<float, false>), grid, block, 0, stream, a, blocksPerBatch, tb);
+  }
   return hipGetLastError();
 }
 

@@ -302,15 +302,19 @@ def test_tuned_plans_persist_to_a_file(tmp_path):
         h2.close()
 
 
-@pytest.mark.parametrize("M,Ps,tag", [(8, [8] * 4, "1x32768"), (128, [8] * 3, "1x32768"), (1024, [8] * 2, "1x32768"),
-                                      (16, [16] * 3, "1x65536"), (512, [16] * 2, "1x65536"), (32, [16] * 3, "1x65536")])
-def test_row_kernels_with_fewer_factors(fk, M, Ps, tag):
+@pytest.mark.parametrize("M,Ps,tag,tag_b", [(8, [8] * 4, "1x32768", "1x32768"), (128, [8] * 3, "1x32768", "1x32768"),
+                                            (1024, [8] * 2, "1x32768", "1x32768"), (16, [16] * 3, "1x4096", "1x65536"),
+                                            (512, [16] * 2, "1x4096", "1x65536"), (32, [16] * 3, "1x4096", "1x65536")])
+def test_row_kernels_with_fewer_factors(fk, M, Ps, tag, tag_b):
     """Shorter chains of 8x8 / 16x16 factors reuse the whole-row kernels: 8^(5-N) (16^(4-N)) consecutive rows
-    form one contiguous block and the missing leading factors are identities."""
+    form one contiguous block and the missing leading factors are identities.  Two or three 16x16 factors shared
+    by the batch go to the wave-per-block kernel instead; with per-batch factors the workgroup kernel runs them."""
     check(fk, ko.MKM, M, Ps, Ps, np.float32, alpha=1.5, beta=0.5, seed=91)
     plan = fk.last_plan()
     assert len(plan) == 1 and tag in plan[0][2], plan
     check(fk, ko.MKM, M, Ps, Ps, np.float32, alpha=1.0, beta=0.0, seed=92, batch=2)
+    plan = fk.last_plan()
+    assert len(plan) == 1 and tag_b in plan[0][2], plan
 
 
 def test_row_kernels_need_whole_blocks(fk):
@@ -595,3 +599,16 @@ def test_kmm_layout_pair_of_16x16_factors(fk, M, Ps, launches, dt):
     check(fk, ko.KMM, M, Ps, Ps, dt, alpha=1.0, beta=0.0, seed=702, opFs=ko.OP_T)
     check(fk, ko.KMM, M, Ps, Ps, dt, alpha=1.0, beta=1.0, seed=703, batch=3)
     check(fk, ko.KMM, M, Ps, Ps, dt, alpha=1.0, beta=0.0, seed=704, integer=True)
+
+
+@pytest.mark.parametrize("M,Ps", [(5, [16] * 3), (7, [16, 16, 16]), (48, [16, 16]), (3, [2, 8, 16, 16])])
+def test_fp32_16x16_wave_per_block_kernel_where_the_workgroup_kernel_needs_whole_blocks(fk, M, Ps):
+    """fp32 16x16^3 with a row count that is no multiple of 16: one wave per 4096-element block instead of the
+    workgroup kernel that packs 16 rows into a 16^4 block."""
+    check(fk, ko.MKM, M, Ps, Ps, np.float32, alpha=1.5, beta=0.5, seed=801)
+    plan = fk.last_plan()
+    if M % 16:
+        assert any("_f_16x16_16x16_3_1x4096_" in k for _, _, k in plan), plan
+    check(fk, ko.MKM, M, Ps, Ps, np.float32, alpha=1.0, beta=0.0, seed=802, opFs=ko.OP_T)
+    check(fk, ko.MKM, M, Ps, Ps, np.float32, alpha=1.0, beta=1.0, seed=803, batch=2, share_f=True)
+    check(fk, ko.MKM, M, Ps, Ps, np.float32, alpha=1.0, beta=0.0, seed=804, integer=True)
