@@ -46,8 +46,9 @@ template <> struct R3Mfma<float> {
 
 constexpr int kR3Block = 4096;
 constexpr int kR3Waves = 4;
-constexpr int kR3Ahead = 2;            // k1 slices of the next block requested before the last contraction
-constexpr int kR3Win = 2;              // further slices in flight while a block is contracted
+// k1 slices of the next block requested before the last contraction / further slices in flight while a block is
+// contracted: as many as the registers allow at two waves per SIMD
+template <typename T> struct R3Depth { static constexpr int ahead = sizeof(T) == 4 ? 4 : 2, win = sizeof(T) == 4 ? 4 : 2; };
 
 template <typename T, bool HAS_Y>
 __global__ __launch_bounds__(256, 2) void kron_row16x3_kernel(const StepArgs a, const uint32_t blocksPerBatch,
@@ -55,6 +56,7 @@ __global__ __launch_bounds__(256, 2) void kron_row16x3_kernel(const StepArgs a, 
   using MF = R3Mfma<T>;
   using Acc = typename MF::Acc;
   typedef T V2 __attribute__((ext_vector_type(2)));
+  constexpr int kR3Ahead = R3Depth<T>::ahead, kR3Win = R3Depth<T>::win;
   __shared__ __align__(16) T f1s[256];               // F1 transposed: f1s[q1*16 + k1]
   const int tid = threadIdx.x;
   const int l0 = tid & 63;
@@ -210,7 +212,7 @@ hipError_t launchRow16x3(const StepArgs& a, DType dt, hipStream_t stream) {
   }
   const uint32_t blocksPerBatch = a.nf == 2 ? a.M / 16 : a.M;
   const uint64_t total = (uint64_t)blocksPerBatch * a.batch;
-  // persistent waves: two workgroups of four waves per CU (two waves per SIMD at up to 256 registers)
+  // persistent waves: two workgroups of four waves per CU (more resident waves measured slightly slower)
   uint32_t wgs = (uint32_t)cus * 2;
   const uint64_t need = (total + kR3Waves - 1) / kR3Waves;
   if (wgs > need) wgs = (uint32_t)need;
