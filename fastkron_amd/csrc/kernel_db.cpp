@@ -135,18 +135,20 @@ static bool row8CanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, u
 static hipError_t row8Launch(const KernelInfo&, const StepArgs& a, hipStream_t s) { return launchRow8x5(a, s); }
 static bool row8Check(const KernelInfo&, const StepArgs& a) { return row8x5Supported(a); }
 
-// ---- wave-per-block kernel for two or three fused 16x16 factors ----
+// ---- wave-per-block kernel for two or three fused PxP factors, 9 <= P <= 16 ----
 static bool row16x3CanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
                           const DeviceInfo&) {
   const uint32_t nf = hi - lo + 1;
   if (p.dt != k.dt || p.mm != MMType::MKM || nf < 2 || nf > 3 || p.forward) return false;
+  const uint32_t P = p.P[hi];
+  if (P < 9 || P > 16) return false;
   uint64_t kk = 1;
   for (uint32_t i = lo; i <= hi; i++) {
-    if (p.P[i] != 16 || p.Q[i] != 16) return false;
+    if (p.P[i] != P || p.Q[i] != P) return false;
     if (p.batch > 1 && p.strideF[i] != 0) return false;     // the factors are staged once per workgroup
-    kk *= 16;
+    kk *= P;
   }
-  if (p.colsBefore(hi) != kk || (nf == 2 && p.M % 16)) return false;
+  if (p.colsBefore(hi) != kk || (nf == 2 && p.M % P)) return false;
   return !(first && p.opX == 2);
 }
 static hipError_t row16x3Launch(const KernelInfo& k, const StepArgs& a, hipStream_t s) { return launchRow16x3(a, k.dt, s); }
@@ -240,11 +242,11 @@ static bool kmmRegCheck(const KernelInfo&, const StepArgs& a) { return kmmRegSup
 void registerRowKernels(std::vector<KernelInfo>& out) {
   // grammar: <mm>_<backend>_<arch>_<threads>_<type>_<PxQ>_<TilePxTileQ>_<fused>_<TileMxTileK>_<regs>_<ops>_<batch>_<p2p>_<opt>
   // two or three 16x16 factors: one wave per 4096-element block (measured faster than the workgroup kernel below on
-  // three factors, 4.6 against 4.1 TB/s in fp32, and free of its row-count conditions)
+  // three factors, 4.6 against 4.1 TB/s in fp32, and free of its row-count conditions); 9x9 ... 15x15 zero-padded
   for (DType dt : {DType::F64, DType::F32}) {
     KernelInfo kd3{};
     kd3.name = std::string("mkm_hip_gfx950_256_") + (dt == DType::F64 ? "d" : "f") +
-               "_16x16_16x16_3_1x4096_mfma16x16x4_NN_strided_0_3";
+               "_16x16_16x16_3_1x4096_mfma16x16x4_NN_strided_0_3";      // also 9x9 ... 15x15, padded to this tile
     kd3.dt = dt; kd3.P = 16; kd3.Q = 16; kd3.fused = 3; kd3.tileM = 1; kd3.tileK = 4096; kd3.threads = 256;
     kd3.variant = 0; kd3.canRun = row16x3CanRun; kd3.launch = row16x3Launch; kd3.check = row16x3Check;
     out.push_back(kd3);

@@ -44,13 +44,14 @@ template <> struct R3Mfma<float> {
   static __device__ __forceinline__ int row(int r, int hi) { return 4 * hi + r; }
 };
 
-constexpr int kR3Block = 4096;
 constexpr int kR3Waves = 4;
 // k1 slices of the next block requested before the last contraction / further slices in flight while a block is
 // contracted: as many as the registers allow at two waves per SIMD
 template <typename T> struct R3Depth { static constexpr int ahead = sizeof(T) == 4 ? 4 : 2, win = sizeof(T) == 4 ? 4 : 2; };
 
-template <typename T, bool HAS_Y>
+// EXACT: 16x16 factors (vector loads, no masks).  Otherwise PxP factors with 9 <= P <= 15 on blocks of P^3
+// elements: the matrix-core operands are zero-padded to 16 and the lanes / registers beyond P are masked.
+template <typename T, bool HAS_Y, bool EXACT>
 __global__ __launch_bounds__(256, 2) void kron_row16x3_kernel(const StepArgs a, const uint32_t blocksPerBatch,
                                                               const uint32_t totalBlocks) {
   using MF = R3Mfma<T>;
@@ -62,13 +63,16 @@ __global__ __launch_bounds__(256, 2) void kron_row16x3_kernel(const StepArgs a, 
   const int l0 = tid & 63;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lo = l0 & 15, hi = l0 >> 4;
+  const int P = EXACT ? 16 : (int)a.p[0];            // factor size; P2, P3: strides of k2 / k1 and the block length
+  const int P2 = P * P, P3 = P2 * P;
 
   // a.f[0] is the last factor F3, a.f[1] = F2, a.f[2] = F1 (identity when only two factors are fused).
   // Factors shared by the whole launch only: per-batch factors are left to other kernels.
   {
     const int q1 = tid >> 4, k1 = tid & 15;
-    T v = (q1 == k1) ? (T)1 : (T)0;
-    if (a.nf == 3) v = ((const T*)a.f[2])[(int64_t)k1 * a.f_sp[2] + (int64_t)q1 * a.f_sq[2]];
+    const bool in = EXACT || (q1 < P && k1 < P);
+    T v = (in && q1 == k1) ? (T)1 : (T)0;
+    if (a.nf == 3 && in) v = ((const T*)a.f[2])[(int64_t)k1 * a.f_sp[2] + (int64_t)q1 * a.f_sq[2]];
     f1s[tid] = v;
   }
   // operands of the two products: F3[4*hi + c][lo] and F2[row(r, hi)][lo] (the rows the first product leaves
@@ -79,8 +83,9 @@ __global__ __launch_bounds__(256, 2) void kron_row16x3_kernel(const StepArgs a, 
     const T* F2 = (const T*)a.f[1];
 #pragma unroll
     for (int c = 0; c < 4; c++) {
-      f3[c] = F3[(int64_t)(4 * hi + c) * a.f_sp[0] + (int64_t)lo * a.f_sq[0]];
-      f2[c] = F2[(int64_t)MF::row(c, hi) * a.f_sp[1] + (int64_t)lo * a.f_sq[1]];
+      f3[c] = f2[c] = (T)0;
+      if (EXACT || (4 * hi + c < P && lo < P)) f3[c] = F3[(int64_t)(4 * hi + c) * a.f_sp[0] + (int64_t)lo * a.f_sq[0]];
+      if (EXACT || (MF::row(c, hi) < P && lo < P)) f2[c] = F2[(int64_t)MF::row(c, hi) * a.f_sp[1] + (int64_t)lo * a.f_sq[1]];
     }
   }
   __syncthreads();
@@ -90,12 +95,18 @@ __global__ __launch_bounds__(256, 2) void kron_row16x3_kernel(const StepArgs a, 
   if (blk >= totalBlocks) return;
 
   auto blockPtr = [&](uint32_t b) {
-    return (const T*)a.in + (size_t)(b / blocksPerBatch) * a.in_batch + (size_t)(b % blocksPerBatch) * kR3Block;
+    return (const T*)a.in + (size_t)(b / blocksPerBatch) * a.in_batch + (size_t)(b % blocksPerBatch) * P3;
   };
-  // x[c] = X[k1][k2 = lo][k3 = 4*hi + c]: 16-byte loads
+  // x[c] = X[k1][k2 = lo][k3 = 4*hi + c]: 16-byte loads (element by element, masked, for P < 16)
   auto loadSlice = [&](const T* X, int k1, T (&x)[4]) {
-    const T* xp = X + k1 * 256 + lo * 16 + hi * 4;
-    if (sizeof(T) == 8) {
+    const T* xp = X + k1 * P2 + lo * P + hi * 4;
+    if (!EXACT) {
+#pragma unroll
+      for (int c = 0; c < 4; c++) {
+        x[c] = (T)0;
+        if (k1 < P && lo < P && 4 * hi + c < P) x[c] = xp[c];
+      }
+    } else if (sizeof(T) == 8) {
       const V2 v0 = *(const V2*)xp, v1 = *(const V2*)(xp + 2);
       x[0] = v0[0]; x[1] = v0[1]; x[2] = v1[0]; x[3] = v1[1];
     } else {
@@ -114,8 +125,8 @@ __global__ __launch_bounds__(256, 2) void kron_row16x3_kernel(const StepArgs a, 
   auto processBlock = [&](const uint32_t blk) {
     const T* X = blockPtr(blk);
     const size_t bt = blk / blocksPerBatch, m = blk % blocksPerBatch;
-    T* Z = (T*)a.out + bt * a.out_batch + m * kR3Block;
-    const T* Y = HAS_Y ? (const T*)a.y + bt * a.y_batch + m * kR3Block : nullptr;
+    T* Z = (T*)a.out + bt * a.out_batch + m * P3;
+    const T* Y = HAS_Y ? (const T*)a.y + bt * a.y_batch + m * P3 : nullptr;
 
     // ---- k3 and k2, slice by slice; z[k1][r] = T[k1][q2 = row(r, hi)][q3 = lo] ----
     T z[16][4];
@@ -129,12 +140,14 @@ __global__ __launch_bounds__(256, 2) void kron_row16x3_kernel(const StepArgs a, 
       for (int c = 0; c < 4; c++)
         x[c] = (k1 < kR3Ahead) ? xa[k1 < kR3Ahead ? k1 : 0][c] : xb[(k1 - kR3Ahead) % kR3Win][c];
       if (k1 >= kR3Ahead && k1 + kR3Win < 16) loadSlice(X, k1 + kR3Win, xb[(k1 - kR3Ahead) % kR3Win]);
-      Acc d = (Acc){0, 0, 0, 0};
-#pragma unroll
-      for (int c = 0; c < 4; c++) d = MF::mma(x[c], f3[c], d);         // d[k2][q3]
       Acc e = (Acc){0, 0, 0, 0};
+      if (EXACT || k1 < P) {
+        Acc d = (Acc){0, 0, 0, 0};
 #pragma unroll
-      for (int r = 0; r < 4; r++) e = MF::mma(f2[r], d[r], e);         // e[q2][q3]
+        for (int c = 0; c < 4; c++) d = MF::mma(x[c], f3[c], d);       // d[k2][q3]
+#pragma unroll
+        for (int r = 0; r < 4; r++) e = MF::mma(f2[r], d[r], e);       // e[q2][q3]
+      }
 #pragma unroll
       for (int r = 0; r < 4; r++) z[k1][r] = e[r];
       __builtin_amdgcn_sched_barrier(0);             // keeps the loads of later slices from being hoisted up here
@@ -152,12 +165,14 @@ __global__ __launch_bounds__(256, 2) void kron_row16x3_kernel(const StepArgs a, 
     const T alpha = a.epilogue ? (T)a.alpha : (T)1, beta = (T)a.beta;
     T* zp = Z + lo;
     const T* yp = HAS_Y ? Y + lo : nullptr;
+    // (for P < 16: slices k1 >= P were not loaded, their z are exact zeros; rows and columns >= P are not stored)
 #pragma unroll 1
-    for (int q1 = 0; q1 < 16; q1++) {
+    for (int q1 = 0; q1 < P; q1++) {
       T yv[4];
       if (HAS_Y) {
 #pragma unroll
-        for (int r = 0; r < 4; r++) yv[r] = yp[q1 * 256 + MF::row(r, hi) * 16];
+        for (int r = 0; r < 4; r++)
+          yv[r] = (EXACT || (MF::row(r, hi) < P && lo < P)) ? yp[q1 * P2 + MF::row(r, hi) * P] : (T)0;
       }
       T acc[4] = {0, 0, 0, 0};
 #pragma unroll
@@ -172,7 +187,8 @@ __global__ __launch_bounds__(256, 2) void kron_row16x3_kernel(const StepArgs a, 
       for (int r = 0; r < 4; r++) {
         T v = acc[r] * alpha;
         if (HAS_Y) v += beta * yv[r];
-        zp[q1 * 256 + MF::row(r, hi) * 16] = v;      // Z[q1][q2 = row(r, hi)][q3 = lo]
+        if (EXACT || (MF::row(r, hi) < P && lo < P))
+          zp[q1 * P2 + MF::row(r, hi) * P] = v;      // Z[q1][q2 = row(r, hi)][q3 = lo]
       }
     }
   };
@@ -185,20 +201,31 @@ __global__ __launch_bounds__(256, 2) void kron_row16x3_kernel(const StepArgs a, 
 
 bool row16x3Supported(const StepArgs& a, DType dt) {
   if (a.nf != 2 && a.nf != 3) return false;
+  const uint32_t P = a.p[0];
+  if (P < 9 || P > 16) return false;
   uint64_t k = 1;
   for (uint32_t j = 0; j < a.nf; j++) {
-    if (a.p[j] != 16 || a.q[j] != 16 || (a.batch > 1 && a.f_batch[j] != 0)) return false;
-    k *= 16;
+    if (a.p[j] != P || a.q[j] != P || (a.batch > 1 && a.f_batch[j] != 0)) return false;
+    k *= P;
   }
   if (a.Kin != k || a.Kout != k) return false;
   if (a.in_ldc != 1 || a.out_ldc != 1 || (a.y && a.y_ldc != 1)) return false;
   // the rows of a block must be contiguous, and M must be a whole number of blocks
   if ((uint64_t)a.in_ldm != k || (uint64_t)a.out_ldm != k || (a.y && (uint64_t)a.y_ldm != k)) return false;
-  if (a.nf == 2 && a.M % 16) return false;
-  // 16-byte loads
-  if (((uintptr_t)a.in & 15) || (a.in_batch * dtypeSize(dt)) % 16) return false;
-  const uint64_t blocks = (uint64_t)(a.nf == 2 ? a.M / 16 : a.M) * a.batch;
+  if (a.nf == 2 && a.M % P) return false;
+  // 16-byte loads of the 16x16 form
+  if (P == 16 && (((uintptr_t)a.in & 15) || (a.in_batch * dtypeSize(dt)) % 16)) return false;
+  const uint64_t blocks = (uint64_t)(a.nf == 2 ? a.M / P : a.M) * a.batch;
   return blocks < (1ull << 32);
+}
+
+template <typename T, bool EXACT>
+static void launchRow16x3T(const StepArgs& a, dim3 grid, uint32_t blocksPerBatch, uint32_t total, hipStream_t stream) {
+  dim3 block(256);
+  if (a.y && a.epilogue)
+    hipLaunchKernelGGL((kron_row16x3_kernel<T, true, EXACT>), grid, block, 0, stream, a, blocksPerBatch, total);
+  else
+    hipLaunchKernelGGL((kron_row16x3_kernel<T, false, EXACT>), grid, block, 0, stream, a, blocksPerBatch, total);
 }
 
 hipError_t launchRow16x3(const StepArgs& a, DType dt, hipStream_t stream) {
@@ -210,21 +237,21 @@ hipError_t launchRow16x3(const StepArgs& a, DType dt, hipStream_t stream) {
     cus = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
               ? prop.multiProcessorCount : 256;
   }
-  const uint32_t blocksPerBatch = a.nf == 2 ? a.M / 16 : a.M;
+  const uint32_t P = a.p[0];
+  const uint32_t blocksPerBatch = a.nf == 2 ? a.M / P : a.M;
   const uint64_t total = (uint64_t)blocksPerBatch * a.batch;
   // persistent waves: two workgroups of four waves per CU (more resident waves measured slightly slower)
   uint32_t wgs = (uint32_t)cus * 2;
   const uint64_t need = (total + kR3Waves - 1) / kR3Waves;
   if (wgs > need) wgs = (uint32_t)need;
-  dim3 grid(wgs), block(256);
-  const bool y = a.y && a.epilogue;
+  dim3 grid(wgs);
   const uint32_t tb = (uint32_t)total;
   if (dt == DType::F64) {
-    if (y) hipLaunchKernelGGL((kron_row16x3_kernel<double, true>), grid, block, 0, stream, a, blocksPerBatch, tb);
-    else   hipLaunchKernelGGL((kron_row16x3_kernel<double, false>), grid, block, 0, stream, a, blocksPerBatch, tb);
+    if (P == 16) launchRow16x3T<double, true>(a, grid, blocksPerBatch, tb, stream);
+    else         launchRow16x3T<double, false>(a, grid, blocksPerBatch, tb, stream);
   } else {
-    if (y) hipLaunchKernelGGL((kron_row16x3_kernel<float, true>), grid, block, 0, stream, a, blocksPerBatch, tb);
-    else   hipLaunchKernelGGL((kron_row16x3_kernel<float, false>), grid, block, 0, stream, a, blocksPerBatch, tb);
+    if (P == 16) launchRow16x3T<float, true>(a, grid, blocksPerBatch, tb, stream);
+    else         launchRow16x3T<float, false>(a, grid, blocksPerBatch, tb, stream);
   }
   return hipGetLastError();
 }

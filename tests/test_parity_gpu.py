@@ -612,3 +612,20 @@ def test_fp32_16x16_wave_per_block_kernel_where_the_workgroup_kernel_needs_whole
     check(fk, ko.MKM, M, Ps, Ps, np.float32, alpha=1.0, beta=0.0, seed=802, opFs=ko.OP_T)
     check(fk, ko.MKM, M, Ps, Ps, np.float32, alpha=1.0, beta=1.0, seed=803, batch=2, share_f=True)
     check(fk, ko.MKM, M, Ps, Ps, np.float32, alpha=1.0, beta=0.0, seed=804, integer=True)
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+@pytest.mark.parametrize("M,Ps,launches", [(5, [10] * 3, 1), (7, [12] * 3, 1), (24, [12, 12], 1), (3, [9] * 3, 1),
+                                           (2, [15] * 3, 1), (3, [10] * 4, 2), (2, [12] * 5, None), (4, [13] * 3, 1)])
+def test_wave_per_block_kernel_with_factors_of_9_to_15(fk, M, Ps, launches, dt):
+    """Two or three PxP factors with 9 <= P <= 15 on blocks of P^3 elements: the 16x16x3 wave-per-block kernel with
+    zero-padded operands and masked lanes; longer chains apply the three trailing factors block by block."""
+    check(fk, ko.MKM, M, Ps, Ps, dt, alpha=1.5, beta=0.5, seed=901)
+    plan = fk.last_plan()
+    assert any("_16x16_16x16_3_1x4096_" in k for _, _, k in plan), plan
+    if launches is not None:
+        assert len(plan) == launches, plan
+    check(fk, ko.MKM, M, Ps, Ps, dt, alpha=1.0, beta=0.0, seed=902, opFs=ko.OP_T)
+    check(fk, ko.MKM, M, Ps, Ps, dt, alpha=1.0, beta=1.0, seed=903, batch=3, share_f=True)
+    check(fk, ko.MKM, M, Ps, Ps, dt, alpha=2.0, beta=0.0, seed=904, batch=2)
+    check(fk, ko.MKM, M, Ps, Ps, dt, alpha=1.0, beta=1.0, seed=905, integer=True)
