@@ -206,7 +206,9 @@ static bool kmm64Check(const KernelInfo&, const StepArgs& a) { return kmm64F64Su
 static bool kmm16x2CanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
                           const DeviceInfo&) {
   if (p.dt != k.dt || p.mm != MMType::KMM || p.M < 2 || hi - lo + 1 != 2 || p.forward) return false;
-  for (uint32_t i = lo; i <= hi; i++) if (p.P[i] != 16 || p.Q[i] != 16) return false;
+  const uint32_t P = p.P[hi];
+  if (P < 9 || P > 16) return false;                       // 9 ... 15: zero-padded to the 16x16 tile
+  for (uint32_t i = lo; i <= hi; i++) if (p.P[i] != P || p.Q[i] != P) return false;
   return !(first && p.opX == 2);
 }
 static hipError_t kmm16x2Launch(const KernelInfo& k, const StepArgs& a, hipStream_t s) { return launchKmm16x2(a, k.dt, s); }

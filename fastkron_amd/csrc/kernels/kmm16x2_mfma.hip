@@ -45,7 +45,9 @@ template <> struct K2Mfma<float> {
 constexpr int kK2Waves = 4;
 constexpr int kK2Win = 3;              // k0 slices of a tile in flight
 
-template <typename T, bool HAS_Y>
+// EXACT: 16x16 factors.  Otherwise PxP factors with 9 <= P <= 15: matrix-core operands zero-padded to 16, rows and
+// registers beyond P masked.
+template <typename T, bool HAS_Y, bool EXACT>
 __global__ __launch_bounds__(256, 2) void kron_kmm16x2_kernel(const StepArgs a, const uint32_t mTiles,
                                                               const uint32_t totalTiles) {
   using MF = K2Mfma<T>;
@@ -57,20 +59,26 @@ __global__ __launch_bounds__(256, 2) void kron_kmm16x2_kernel(const StepArgs a, 
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lo = l0 & 15, hi = l0 >> 4;
   const uint32_t bt = blockIdx.y;
-  const uint64_t S = a.Kin / 256;
+  const int P = EXACT ? 16 : (int)a.p[0];
+  const uint64_t S = a.Kin / (uint64_t)(P * P);
   const uint64_t M = a.M;
 
   // a.f[0] is the later factor F1 (contracts the fast digit k1), a.f[1] = F0
   {
     const T* F0 = (const T*)a.f[1] + (size_t)bt * a.f_batch[1];
     const int q0 = tid >> 4, k0 = tid & 15;
-    f0s[tid] = F0[(int64_t)k0 * a.f_sp[1] + (int64_t)q0 * a.f_sq[1]];
+    T v = (T)0;
+    if (EXACT || (q0 < P && k0 < P)) v = F0[(int64_t)k0 * a.f_sp[1] + (int64_t)q0 * a.f_sq[1]];
+    f0s[tid] = v;
   }
   T f1[4];                                          // A operand: F1[k1 = 4*c + hi][q1 = lo]
   {
     const T* F1 = (const T*)a.f[0] + (size_t)bt * a.f_batch[0];
 #pragma unroll
-    for (int c = 0; c < 4; c++) f1[c] = F1[(int64_t)(4 * c + hi) * a.f_sp[0] + (int64_t)lo * a.f_sq[0]];
+    for (int c = 0; c < 4; c++) {
+      f1[c] = (T)0;
+      if (EXACT || (4 * c + hi < P && lo < P)) f1[c] = F1[(int64_t)(4 * c + hi) * a.f_sp[0] + (int64_t)lo * a.f_sq[0]];
+    }
   }
   __syncthreads();
 
@@ -81,12 +89,17 @@ __global__ __launch_bounds__(256, 2) void kron_kmm16x2_kernel(const StepArgs a, 
 
   const uint32_t nWaves = gridDim.x * kK2Waves;
   // x[c] = X[(s, k0, k1 = 4*c + hi), m]; columns beyond M are clamped to the tile's first one (computed, not stored)
-  // The rows are read in the order (k0, c): row k0*16 + 4*c + hi, four rows further with every load, so one
-  // running pointer serves the whole tile.
-  const uint64_t rowStep = 4 * (uint64_t)a.in_ldc;
+  // The rows are read in the order (k0, c): row k0*P + 4*c + hi, four rows further with every load and P - 16
+  // back at the end of a slice, so one running pointer serves the whole tile.  Rows 4*c + hi >= P are not read.
+  const int64_t rowStep = 4 * (int64_t)a.in_ldc, sliceFix = (int64_t)(P - 16) * (int64_t)a.in_ldc;
   auto loadSlice = [&](const T*& xp, T (&x)[4]) {
 #pragma unroll
-    for (int c = 0; c < 4; c++) { x[c] = *xp; xp += rowStep; }
+    for (int c = 0; c < 4; c++) {
+      x[c] = (T)0;
+      if (EXACT || 4 * c + hi < P) x[c] = *xp;
+      xp += rowStep;
+    }
+    if (!EXACT) xp += sliceFix;
   };
 
   for (uint32_t t = blockIdx.x * kK2Waves + w; t < totalTiles; t += nWaves) {
@@ -94,7 +107,7 @@ __global__ __launch_bounds__(256, 2) void kron_kmm16x2_kernel(const StepArgs a, 
     const uint32_t m0 = (uint32_t)(t - s * mTiles) * 16;
     const bool mOk = m0 + lo < M;
     const uint32_t m = mOk ? m0 + lo : m0;
-    const T* xp = inB + m + (s * 256 + hi) * (uint64_t)a.in_ldc;
+    const T* xp = inB + m + (s * (uint64_t)(P * P) + hi) * (uint64_t)a.in_ldc;
 
     T z[16][4];
     T xw[kK2Win][4];
@@ -105,10 +118,12 @@ __global__ __launch_bounds__(256, 2) void kron_kmm16x2_kernel(const StepArgs a, 
       T x[4];
 #pragma unroll
       for (int c = 0; c < 4; c++) x[c] = xw[k0 % kK2Win][c];
-      if (k0 + kK2Win < 16) loadSlice(xp, xw[k0 % kK2Win]);
+      if (k0 + kK2Win < (EXACT ? 16 : P)) loadSlice(xp, xw[k0 % kK2Win]);
       Acc d = (Acc){0, 0, 0, 0};
+      if (EXACT || k0 < P) {
 #pragma unroll
-      for (int c = 0; c < 4; c++) d = MF::mma(f1[c], x[c], d);         // d[q1][m]
+        for (int c = 0; c < 4; c++) d = MF::mma(f1[c], x[c], d);       // d[q1][m]
+      }
 #pragma unroll
       for (int r = 0; r < 4; r++) z[k0][r] = d[r];
       __builtin_amdgcn_sched_barrier(0);             // keeps the loads of later slices from being hoisted up here
@@ -121,12 +136,12 @@ __global__ __launch_bounds__(256, 2) void kron_kmm16x2_kernel(const StepArgs a, 
     T* op = outB + m + s * (uint64_t)a.out_ldc + (uint64_t)MF::row(0, hi) * oq;
     const T* yp = HAS_Y ? YB + m + s * (uint64_t)a.y_ldc + (uint64_t)MF::row(0, hi) * yq : nullptr;
 #pragma unroll 1
-    for (int q0 = 0; q0 < 16; q0++) {
+    for (int q0 = 0; q0 < P; q0++) {
       T yv[4];
       if (HAS_Y) {
 #pragma unroll
-        for (int r = 0; r < 4; r++) yv[r] = mOk ? yp[r * rs * yq] : (T)0;
-        yp += 16 * yq;
+        for (int r = 0; r < 4; r++) yv[r] = (mOk && (EXACT || MF::row(r, hi) < P)) ? yp[r * rs * yq] : (T)0;
+        yp += (uint64_t)P * yq;
       }
       T acc[4] = {0, 0, 0, 0};
 #pragma unroll
@@ -142,26 +157,28 @@ __global__ __launch_bounds__(256, 2) void kron_kmm16x2_kernel(const StepArgs a, 
         for (int r = 0; r < 4; r++) {
           T v = acc[r] * alpha;
           if (HAS_Y) v += beta * yv[r];
-          op[r * rs * oq] = v;
+          if (EXACT || MF::row(r, hi) < P) op[r * rs * oq] = v;
         }
       }
-      op += 16 * oq;
+      op += (uint64_t)P * oq;
     }
   }
 }
 
 bool kmm16x2Supported(const StepArgs& a, DType dt) {
   if (a.nf != 2) return false;
-  for (uint32_t j = 0; j < 2; j++) if (a.p[j] != 16 || a.q[j] != 16) return false;
-  if (a.Kin % 256 || a.Kout != a.Kin) return false;
+  const uint32_t P = a.p[0];
+  if (P < 9 || P > 16) return false;
+  for (uint32_t j = 0; j < 2; j++) if (a.p[j] != P || a.q[j] != P) return false;
+  if (a.Kin % (P * P) || a.Kout != a.Kin) return false;
   // the M index contiguous in the input, the output and Y
   if (a.in_ldm != 1 || a.out_ldm != 1 || (a.y && a.y_ldm != 1)) return false;
-  const uint64_t tiles = (a.Kin / 256) * ((a.M + 15) / 16);
+  const uint64_t tiles = (a.Kin / (P * P)) * ((a.M + 15) / 16);
   (void)dt;
   return tiles < (1ull << 31) && a.batch <= 65535;
 }
 
-template <typename T>
+template <typename T, bool EXACT>
 static hipError_t launchKmm16x2T(const StepArgs& a, hipStream_t stream) {
   static int cus = 0;
   if (!cus) {
@@ -170,8 +187,9 @@ static hipError_t launchKmm16x2T(const StepArgs& a, hipStream_t stream) {
     cus = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
               ? prop.multiProcessorCount : 256;
   }
+  const uint32_t P = a.p[0];
   const uint32_t mTiles = (a.M + 15) / 16;
-  const uint32_t totalTiles = (uint32_t)((a.Kin / 256) * mTiles);
+  const uint32_t totalTiles = (uint32_t)((a.Kin / (P * P)) * mTiles);
   // persistent waves: two workgroups of four waves per CU (two waves per SIMD)
   uint32_t wgs = (uint32_t)cus * 2;
   if (a.batch > 1) wgs = (wgs + a.batch - 1) / a.batch;
@@ -180,15 +198,17 @@ static hipError_t launchKmm16x2T(const StepArgs& a, hipStream_t stream) {
   if (wgs == 0) wgs = 1;
   dim3 grid(wgs, a.batch), block(256);
   if (a.y && a.epilogue)
-    hipLaunchKernelGGL((kron_kmm16x2_kernel<T, true>), grid, block, 0, stream, a, mTiles, totalTiles);
+    hipLaunchKernelGGL((kron_kmm16x2_kernel<T, true, EXACT>), grid, block, 0, stream, a, mTiles, totalTiles);
   else
-    hipLaunchKernelGGL((kron_kmm16x2_kernel<T, false>), grid, block, 0, stream, a, mTiles, totalTiles);
+    hipLaunchKernelGGL((kron_kmm16x2_kernel<T, false, EXACT>), grid, block, 0, stream, a, mTiles, totalTiles);
   return hipGetLastError();
 }
 
 hipError_t launchKmm16x2(const StepArgs& a, DType dt, hipStream_t stream) {
   if (!kmm16x2Supported(a, dt)) return hipErrorInvalidValue;
-  return dt == DType::F32 ? launchKmm16x2T<float>(a, stream) : launchKmm16x2T<double>(a, stream);
+  const bool exact = a.p[0] == 16;
+  if (dt == DType::F32) return exact ? launchKmm16x2T<float, true>(a, stream) : launchKmm16x2T<float, false>(a, stream);
+  return exact ? launchKmm16x2T<double, true>(a, stream) : launchKmm16x2T<double, false>(a, stream);
 }
 
 }  // namespace fk

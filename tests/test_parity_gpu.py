@@ -601,6 +601,22 @@ def test_kmm_layout_pair_of_16x16_factors(fk, M, Ps, launches, dt):
     check(fk, ko.KMM, M, Ps, Ps, dt, alpha=1.0, beta=0.0, seed=704, integer=True)
 
 
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+@pytest.mark.parametrize("M,Ps,launches", [(16, [12, 12], 1), (37, [9, 9], 1), (5, [15, 15], 1), (100, [10] * 4, 2),
+                                           (33, [13] * 3, 2), (1, [11, 11], None)])
+def test_kmm_layout_pair_of_factors_of_9_to_15(fk, M, Ps, launches, dt):
+    """GeKMM chains of PxP factors with 9 <= P <= 15: the 16x16 pair kernel with zero-padded operands and masked
+    rows; a single column of X (M = 1) takes another kernel."""
+    check(fk, ko.KMM, M, Ps, Ps, dt, alpha=1.5, beta=0.5, seed=711)
+    plan = fk.last_plan()
+    if launches is not None:
+        assert any("_16x16_16x16_2_16x256_" in k for _, _, k in plan) and len(plan) == launches, plan
+    check(fk, ko.KMM, M, Ps, Ps, dt, alpha=1.0, beta=0.0, seed=712, opFs=ko.OP_T)
+    check(fk, ko.KMM, M, Ps, Ps, dt, alpha=1.0, beta=1.0, seed=713, batch=3)
+    check(fk, ko.KMM, M, Ps, Ps, dt, alpha=2.0, beta=0.0, seed=714, opX=ko.OP_T)
+    check(fk, ko.KMM, M, Ps, Ps, dt, alpha=1.0, beta=0.0, seed=715, integer=True)
+
+
 @pytest.mark.parametrize("M,Ps", [(5, [16] * 3), (7, [16, 16, 16]), (48, [16, 16]), (3, [2, 8, 16, 16])])
 def test_fp32_16x16_wave_per_block_kernel_where_the_workgroup_kernel_needs_whole_blocks(fk, M, Ps):
     """fp32 16x16^3 with a row count that is no multiple of 16: one wave per 4096-element block instead of the
