@@ -10,6 +10,7 @@
 //
 //   load     wave w owns the block k1 = w (4096 contiguous elements): one 16-byte load per lane and
 //            256-element slice (k3 = lane%16, k4 = 4*(lane/16) + register), a window of kWin slices in flight
+//            (kCarry of them, the first of the next row, across the exchange)
 //   k4, k3   per slice, V_MFMA_F32_16X16X4_F32 chained in registers: the first product leaves D[i][j] in
 //            register i%4 of lane 16*(i/4)+j, which is exactly the A-operand layout (lane 16*k+i) of a
 //            second product that contracts the *row* index i of the first; the factor operand of the
@@ -18,7 +19,7 @@
 //            adds every slice's share to the lane's 16 x 4 accumulators, acc[q2][r] += F2[k2][q2] * T[k2][r].
 //            Up to here a wave works on its own: no barrier, no LDS traffic but operands, and every slice
 //            worked on frees the registers for the request of the slice kWin later, so the loads of a row
-//            are spread over this phase (and run on into the first kWin slices of the next row).
+//            are spread over this phase (and run on into the first kCarry slices of the next row).
 //   k1       the one digit that couples the waves: quarter by quarter (q2 = 4*qq .. 4*qq+3, 64 KB) through
 //            a double-buffered LDS exchange, 16-byte writes and reads; the quarter qq+1 is written between
 //            the same two barriers in which the quarter qq is consumed: one 16x16x4 product per 16 columns,
@@ -29,10 +30,11 @@
 // Vector memory instructions of a CU pass through one in-order pipeline: stores issued behind a burst of loads
 // wait for it, and so do the waves that issue them.  Hence the spreading above (a burst of 16 loads per lane
 // behind the last quarter, with the stores of two quarters behind it, costs 14 us per row), and the register
-// budget (64 accumulators + the window out of 128) is what limits the window.
+// budget (64 accumulators + the window out of 128) is what limits the window: one window slot that the compiler
+// has to spill right after its load makes the wave wait for that load, and costs 8 % of the launch.
 // The CUs start in lockstep and would alternate between a phase in which all of them wait for HBM and a phase in
-// which none uses it; a third of the workgroups each start kStaggerTicks later than the previous third (when a
-// workgroup has more than one row to work on), which interleaves the phases of neighbouring CUs.
+// which none uses it; the workgroups start in kStaggerGroups groups, kStaggerTicks apart (when a workgroup has more
+// than one row to work on), which interleaves the phases of neighbouring CUs.
 //
 // Algorithmic traffic: 4*65536 bytes read + 4*65536 bytes written per row (+ Y when beta != 0).
 #include <hip/hip_runtime.h>
@@ -47,9 +49,16 @@ typedef float f4 __attribute__((ext_vector_type(4)));
 #define MFMA4(a, b, c) __builtin_amdgcn_mfma_f32_4x4x1f32((a), (b), (c), 0, 0, 0)
 
 constexpr int kRowLen = 65536;
-constexpr int kWin = 4;                    // slices in flight per wave (registers: 64 accumulators + 4*kWin + operands)
-constexpr uint32_t kStaggerGroups = 3;     // measured: 3 groups 4 us apart; 2 or 4 groups lose (neighbouring CUs in phase)
-constexpr uint32_t kStaggerTicks = 400;    // of the 100 MHz wall clock
+#ifndef ROW16_WIN
+#define ROW16_WIN 6
+#endif
+#ifndef ROW16_CARRY
+#define ROW16_CARRY 2
+#endif
+constexpr int kWin = ROW16_WIN;            // slices in flight per wave while it works on slices (registers: 64 accumulators + 4*kWin + operands)
+constexpr int kCarry = ROW16_CARRY;        // slices of the next row in flight during the exchange (<= kWin)
+constexpr uint32_t kStaggerGroups = 5;     // measured: 5 groups 2.5 us apart or 3 groups 4 us apart; 2 or 4 groups lose to no stagger
+constexpr uint32_t kStaggerTicks = 250;    // of the 100 MHz wall clock
 constexpr int kQuarterWords = 16384;       // 64 KB: 16 rows k1 of 1024 columns (four values of q2)
 constexpr int kLdsWords = 2 * kQuarterWords + 5 * 256;   // two quarters + the four factors + F2 transposed
 
@@ -89,8 +98,8 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a,
 
   // An item is a block of 65536 contiguous elements: one row for four factors, 16^(4-nf) rows otherwise.
   // x[t][r] = X[k1=w][k2=t][k3=i][k4=4kb+r] (i = l%16, kb = l/16): 1 KB per wave instruction.
-  // kWin slices are in flight: slice t + kWin is requested when slice t has been read, the first kWin slices of
-  // the next item when the last kWin of this one have.
+  // kWin slices are in flight: slice t + kWin is requested when slice t has been read, and the first kCarry slices
+  // of the next item behind the last ones of this item; the other kWin - kCarry follow at the start of that item.
   f4 xw[kWin];
   // uniform part of a slice address (scalar registers) and the lane's part (one 32-bit register)
   auto slicePtr = [&](const uint32_t it) {
@@ -108,11 +117,11 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a,
   {
     const float* xp = slicePtr(item);
 #pragma unroll
-    for (int t = 0; t < kWin; t++) xw[t] = *(const f4*)(xp + (laneOff + t * 256));
+    for (int t = 0; t < kCarry; t++) xw[t] = *(const f4*)(xp + (laneOff + t * 256));
   }
   __syncthreads();
 
-  const float alpha = (float)a.alpha, beta = (float)a.beta;
+  const float alpha = a.epilogue ? (float)a.alpha : 1.f, beta = (float)a.beta;    // HAS_Y implies a.epilogue
   uint32_t batchOfFactors = item / blocksPerBatch;
 
   for (;;) {
@@ -122,8 +131,16 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a,
     asm volatile("" : "+v"(l));
     const int i = l & 15, kb = l >> 4;
     const uint32_t m = item % blocksPerBatch, b = item / blocksPerBatch;
-    float* Z = (float*)a.out + (size_t)b * a.out_batch + (size_t)m * kRowLen;
-    const float* Y = HAS_Y ? (const float*)a.y + (size_t)b * a.y_batch + (size_t)m * kRowLen : nullptr;
+    // row bases pinned to scalar registers: the stores then take one 32-bit lane offset each instead of an address pair
+    typedef __attribute__((address_space(1))) float GlobalFloat;
+    typedef __attribute__((address_space(1))) f4 GlobalF4;
+    auto uniformPtr = [](const void* p) {
+      const uintptr_t v = (uintptr_t)p;
+      const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+      return (GlobalFloat*)(((uintptr_t)hi << 32) | lo);
+    };
+    GlobalFloat* const Z = uniformPtr((float*)a.out + (size_t)b * a.out_batch + (size_t)m * kRowLen);
+    const GlobalFloat* const Y = HAS_Y ? uniformPtr((const float*)a.y + (size_t)b * a.y_batch + (size_t)m * kRowLen) : nullptr;
     if (perBatchFactors && b != batchOfFactors) {      // a new batch: restage its factors
       __syncthreads();                                 // every wave has read its last operand of the previous item
       stageFactors(b);
@@ -149,6 +166,8 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a,
         FB[c] = fl[0 * 256 + (4 * kb + c) * 16 + i];      // F4
       }
       const float* const xcur = slicePtr(item);
+#pragma unroll
+      for (int t = kCarry; t < kWin; t++) xw[t] = *(const f4*)(xcur + (laneOff + t * 256));
       // behind the last item the requests go to one cached kilobyte of the current row instead, and are dropped
       const float* const xnext = slicePtr(nx < totalItems ? nx : item);
       const int nextStride = nx < totalItems ? 256 : 0;
@@ -160,7 +179,7 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a,
         for (int r = 0; r < 4; r++) d = MFMA16(xw[t % kWin][r], FB[r], d);     // d[k3][q4]
         // the slot is free: request the slice that comes kWin later
         if (t + kWin < 16) xw[t % kWin] = *(const f4*)(xcur + (laneOff + (t + kWin) * 256));
-        else xw[t % kWin] = *(const f4*)(xnext + (laneOff + (t + kWin - 16) * nextStride));
+        else if (t + kWin - 16 < kCarry) xw[t % kWin] = *(const f4*)(xnext + (laneOff + (t + kWin - 16) * nextStride));
         f4 e = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int r = 0; r < 4; r++) e = MFMA16(d[r], FA[r], e);        // e[q4][q3]: e[r] = T[k2=t][q3=i][q4=4kb+r]
@@ -169,6 +188,14 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a,
 #pragma unroll
           for (int r = 0; r < 4; r++) acc[qq][r] = MFMA4(fa[qq], e[r], acc[qq][r]);
         __builtin_amdgcn_sched_barrier(0);
+      }
+      // slice j of the next item sits in the slot that fell free for it, (16 - kWin + j) % kWin: to slot j
+      if (16 % kWin) {
+        f4 nxt[kCarry];
+#pragma unroll
+        for (int j = 0; j < kCarry; j++) nxt[j] = xw[(16 - kWin + j) % kWin];
+#pragma unroll
+        for (int j = 0; j < kCarry; j++) xw[j] = nxt[j];
       }
     }
 
@@ -195,11 +222,11 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a,
     // quarter qq of the k1 contraction, read from buffer qq % 2, and its stores
     auto consume = [&](const int qq) {
       const float* const rb = rbase + (qq & 1) * kQuarterWords;
-      const int col = kb * 4 * 4096 + (4 * qq + q2l) * 256 + g * 64 + 4 * i;
+      const uint32_t col = kb * 4 * 4096 + (4 * qq + q2l) * 256 + g * 64 + 4 * i;   // unsigned: uniform base + 32-bit lane offset
       f4 yv[HAS_Y ? 4 : 1];
       if (HAS_Y) {
 #pragma unroll
-        for (int r = 0; r < 4; r++) yv[r] = *(const f4*)(Y + col + r * 4096);
+        for (int r = 0; r < 4; r++) yv[r] = *(const GlobalF4*)(Y + (col + r * 4096));
       }
       f4 D[4];
 #pragma unroll
@@ -212,12 +239,9 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a,
       }
 #pragma unroll
       for (int r = 0; r < 4; r++) {
-        f4 o = {D[0][r], D[1][r], D[2][r], D[3][r]};
-        if (a.epilogue) {
-          o = o * alpha;
-          if (HAS_Y) o = o + yv[r] * beta;
-        }
-        *(f4*)(Z + col + r * 4096) = o;
+        f4 o = (f4){D[0][r], D[1][r], D[2][r], D[3][r]} * alpha;
+        if (HAS_Y) o = o + yv[r] * beta;
+        *(GlobalF4*)(Z + (col + r * 4096)) = o;
       }
     };
 
