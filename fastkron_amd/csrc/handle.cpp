@@ -258,12 +258,13 @@ fastKronError Handle::trySplitLeadingTrailing(const KronProblem& p, void* temp1,
   if (p.mm != MMType::MKM || p.forward || p.opX != fastKronOp_N) return fastKronKernelNotFound;
   if (!temp1 || !temp2 || p.N < 3) return fastKronKernelNotFound;
   // trailing run of identical square factors that one whole-row kernel fuses:
-  // fp32 8x8 (five), 16x16 (four), 32x32 or 64x64 (two); fp64 16x16 (three), 32x32 or 64x64 (two);
+  // fp32 8x8 (five), 16x16 (four), 32x32 (three), 64x64 (two); fp64 16x16 (three), 32x32 or 64x64 (two);
   // 9x9 ... 15x15 (three, either type)
   const uint32_t tp = p.P[p.N - 1];
   if (p.Q[p.N - 1] != tp) return fastKronKernelNotFound;
   uint32_t maxT = 0;
-  if (tp == 32 || tp == 64)    maxT = 2;
+  if (tp == 32 && p.dt == DType::F32) maxT = 3;      // three 32x32 fp32 factors fused per 32768-column block
+  else if (tp == 32 || tp == 64)      maxT = 2;
   else if (p.dt == DType::F32) maxT = (tp == 8) ? 5 : (tp == 16) ? 4 : 0;
   else if (tp == 16)           maxT = 3;
   if (maxT == 0 && tp >= 9 && tp <= 15) maxT = 3;       // zero-padded form of the 16x16x3 wave-per-block kernel

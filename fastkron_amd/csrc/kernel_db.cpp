@@ -166,6 +166,18 @@ static bool row32CanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, 
 static hipError_t row32Launch(const KernelInfo&, const StepArgs& a, hipStream_t s) { return launchRow32x16x3(a, s); }
 static bool row32Check(const KernelInfo&, const StepArgs& a) { return row32x16x3Supported(a); }
 
+// ---- whole-row kernel for three fused 32x32 fp32 factors ----
+static bool row32x3CanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
+                          const DeviceInfo&) {
+  if (p.dt != DType::F32 || p.mm != MMType::MKM || hi - lo + 1 != 3 || p.forward) return false;
+  for (uint32_t i = lo; i <= hi; i++) if (p.P[i] != 32 || p.Q[i] != 32) return false;
+  if (p.colsBefore(hi) != 32768) return false;
+  if (first && p.opX == 2) return false;
+  return k.dt == p.dt;
+}
+static hipError_t row32x3Launch(const KernelInfo&, const StepArgs& a, hipStream_t s) { return launchRow32x3(a, s); }
+static bool row32x3Check(const KernelInfo&, const StepArgs& a) { return row32x3Supported(a); }
+
 // ---- single-factor MFMA step (fp64 and fp32) ----
 static bool stepF64CanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
                           const DeviceInfo& dev) {
@@ -275,6 +287,12 @@ void registerRowKernels(std::vector<KernelInfo>& out) {
   k32.dt = DType::F32; k32.P = 32; k32.Q = 16; k32.fused = 3; k32.tileM = 1; k32.tileK = 32768; k32.threads = 512;
   k32.variant = 0; k32.canRun = row32CanRun; k32.launch = row32Launch; k32.check = row32Check;
   out.push_back(k32);
+
+  KernelInfo k323{};
+  k323.name = "mkm_hip_gfx950_512_f_32x32_32x32_3_1x32768_mfma16x16x4_NN_strided_0_3";
+  k323.dt = DType::F32; k323.P = 32; k323.Q = 32; k323.fused = 3; k323.tileM = 1; k323.tileK = 32768; k323.threads = 512;
+  k323.variant = 0; k323.canRun = row32x3CanRun; k323.launch = row32x3Launch; k323.check = row32x3Check;
+  out.push_back(k323);
 
   for (DType dt : {DType::F32, DType::F64}) {
     KernelInfo k2{};

@@ -23,6 +23,8 @@ hipError_t launchRow8x5(const StepArgs& a, hipStream_t stream);
 // Three fused 32x16 fp32 factors on rows of exactly 32^3 columns, one workgroup per row, two per CU.
 bool row32x16x3Supported(const StepArgs& a);
 hipError_t launchRow32x16x3(const StepArgs& a, hipStream_t stream);
+bool row32x3Supported(const StepArgs& a);
+hipError_t launchRow32x3(const StepArgs& a, hipStream_t stream);
 
 // Two fused 32x32 or 64x64 factors (fp64 or fp32) on rows of exactly P*P columns (MKM layout), one wave per row.
 bool pairMfmaSupported(const StepArgs& a, DType dt);

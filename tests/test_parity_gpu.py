@@ -368,7 +368,9 @@ def test_chains_split_into_pair_kernel_plus_leading_kmm_step(fk, M, Ps, dt):
     matrix-core steps across the blocks."""
     check(fk, ko.MKM, M, Ps, Ps, dt, alpha=1.5, beta=0.5, seed=131)
     plan = fk.last_plan()
-    assert len(plan) == len(Ps) - 1 and plan[0][2].startswith("mkm_") and all("kmm_" in k for _, _, k in plan[1:]), plan
+    # (fp32 chains that end in three 32x32 factors fuse those three instead of two)
+    fused = 3 if dt == np.float32 and Ps[-3:] == [32] * 3 else 2
+    assert len(plan) == len(Ps) - fused + 1 and plan[0][2].startswith("mkm_") and all("kmm_" in k for _, _, k in plan[1:]), plan
     check(fk, ko.MKM, M, Ps, Ps, dt, alpha=1.0, beta=0.0, seed=132, opFs=ko.OP_T)
     check(fk, ko.MKM, M, Ps, Ps, dt, alpha=1.0, beta=1.0, seed=133, batch=2, share_f=True)
     check(fk, ko.MKM, M, Ps, Ps, dt, alpha=1.0, beta=1.0, seed=134, batch=2)
@@ -447,11 +449,12 @@ def test_eight_wave_build_of_the_16x16_block_kernel(tmp_path):
 
 @pytest.mark.parametrize("dt", [np.float32, np.float64])
 def test_two_part_plan_with_three_leading_launches(fk, dt):
-    """32x32^5: fused trailing pair, then three KMM-layout steps that ping-pong between the second temporary and Z
-    (not possible when Y is Z: then the chain runs as single steps)."""
+    """32x32^5: fused trailing pair (fp64; three factors in fp32), then three (two) KMM-layout steps that ping-pong
+    between the second temporary and Z (not possible when Y is Z: then the chain runs as single steps)."""
     check(fk, ko.MKM, 1, [32] * 5, [32] * 5, dt, alpha=1.5, beta=0.5, seed=181)
     plan = fk.last_plan()
-    assert len(plan) == 4 and plan[0][2].startswith("mkm_") and all(k.startswith("kmm_") for _, _, k in plan[1:]), plan
+    launches = 3 if dt == np.float32 else 4
+    assert len(plan) == launches and plan[0][2].startswith("mkm_") and all(k.startswith("kmm_") for _, _, k in plan[1:]), plan
 
 
 @pytest.mark.parametrize("M", [8, 72, 512])
@@ -599,6 +602,20 @@ def test_kmm_layout_pair_of_16x16_factors(fk, M, Ps, launches, dt):
     check(fk, ko.KMM, M, Ps, Ps, dt, alpha=1.0, beta=0.0, seed=702, opFs=ko.OP_T)
     check(fk, ko.KMM, M, Ps, Ps, dt, alpha=1.0, beta=1.0, seed=703, batch=3)
     check(fk, ko.KMM, M, Ps, Ps, dt, alpha=1.0, beta=0.0, seed=704, integer=True)
+
+
+@pytest.mark.parametrize("M,Ps,launches", [(1, [32] * 3, 1), (5, [32] * 3, 1), (64, [32] * 3, 1), (2, [32] * 4, 2),
+                                           (1, [4, 32, 32, 32], 2), (1, [32] * 5, 3)])
+def test_whole_row_kernel_for_three_32x32_factors(fk, M, Ps, launches):
+    """fp32 32x32^3 on rows (or contiguous blocks) of 32768 columns: one launch, one LDS exchange; longer chains
+    apply the three trailing factors block by block and the leading ones in the KMM layout."""
+    check(fk, ko.MKM, M, Ps, Ps, np.float32, alpha=1.5, beta=0.5, seed=1001)
+    plan = fk.last_plan()
+    assert any("_f_32x32_32x32_3_1x32768_" in k for _, _, k in plan) and len(plan) == launches, plan
+    check(fk, ko.MKM, M, Ps, Ps, np.float32, alpha=1.0, beta=0.0, seed=1002, opFs=ko.OP_T)
+    check(fk, ko.MKM, M, Ps, Ps, np.float32, alpha=1.0, beta=1.0, seed=1003, batch=3, share_f=True)
+    check(fk, ko.MKM, M, Ps, Ps, np.float32, alpha=2.0, beta=0.0, seed=1004, batch=2)
+    check(fk, ko.MKM, M, Ps, Ps, np.float32, alpha=1.0, beta=1.0, seed=1005, integer=True)
 
 
 @pytest.mark.parametrize("dt", [np.float32, np.float64])
