@@ -50,10 +50,18 @@ __global__ __launch_bounds__(512, 4) void kron_row32x3_kernel(const StepArgs a) 
 
   // factors to LDS ahead of the row loads (vector memory operations retire in order); a.f[0] is the factor of the
   // fastest digit (F3), element (p, q) at p*f_sp + q*f_sq
-  for (int e = tid; e < 3 * 1024; e += 512) {
-    const int j = e >> 10, p = (e >> 5) & 31, q = e & 31;
-    const float* F = (const float*)a.f[j] + (size_t)bt * a.f_batch[j];
-    fl[e] = F[(int64_t)p * a.f_sp[j] + (int64_t)q * a.f_sq[j]];
+  // (all six loads of a thread go out before the first LDS write waits for one: a loop of load, wait, write would
+  // put six memory round trips in front of the first barrier)
+  {
+    float v[6];
+#pragma unroll
+    for (int k = 0; k < 6; k++) {
+      const int j = k >> 1, e = tid + 512 * (k & 1), p = e >> 5, q = e & 31;
+      const float* F = (const float*)a.f[j] + (size_t)bt * a.f_batch[j];
+      v[k] = F[(int64_t)p * a.f_sp[j] + (int64_t)q * a.f_sq[j]];
+    }
+#pragma unroll
+    for (int k = 0; k < 6; k++) fl[tid + 512 * k] = v[k];
   }
 
   // x[s][h][c][r] = X[k1 = 4w+s][k2 = 16h + lo][k3 = 16c + 4hi + r]
