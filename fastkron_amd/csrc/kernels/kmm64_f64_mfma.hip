@@ -50,9 +50,18 @@ __global__ __launch_bounds__(256, 1) void kron_kmm64_f64_kernel(const StepArgs a
 
   {
     const double* F = (const double*)a.f[0] + (size_t)bt * a.f_batch[0];
-    for (int i = tid; i < P * P; i += 256) {
-      const int p = i / P, q = i % P;
-      fB[p * P + (q ^ (4 * (p & 3)))] = F[(int64_t)p * a.f_sp[0] + (int64_t)q * a.f_sq[0]];
+    // all loads of a thread go out before the first LDS write waits for one (a loop of load, wait, write puts one
+    // memory round trip per iteration in front of the first product)
+    double v[P * P / 256];
+#pragma unroll
+    for (int k = 0; k < P * P / 256; k++) {
+      const int i = tid + 256 * k, p = i / P, q = i % P;
+      v[k] = F[(int64_t)p * a.f_sp[0] + (int64_t)q * a.f_sq[0]];
+    }
+#pragma unroll
+    for (int k = 0; k < P * P / 256; k++) {
+      const int i = tid + 256 * k, p = i / P, q = i % P;
+      fB[p * P + (q ^ (4 * (p & 3)))] = v[k];
     }
   }
   __syncthreads();

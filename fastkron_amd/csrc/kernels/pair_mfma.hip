@@ -91,11 +91,17 @@ __global__ __launch_bounds__(256, 2) void kron_pair_kernel(const StepArgs a) {
   {
     const T* Fa = (const T*)a.f[0] + (size_t)bt * a.f_batch[0];
     const T* Fb = (const T*)a.f[1] + (size_t)bt * a.f_batch[1];
-    for (int i = tid; i < P * P; i += 256) {
-      const int p = i / P, q = i % P;
-      fA[i] = Fa[(int64_t)p * a.f_sp[0] + (int64_t)q * a.f_sq[0]];
-      fB[i] = Fb[(int64_t)p * a.f_sp[1] + (int64_t)q * a.f_sq[1]];
+    // all loads of a thread go out before the first LDS write waits for one (a loop of load, wait, write puts one
+    // memory round trip per iteration in front of the first product)
+    T va[P * P / 256], vb[P * P / 256];
+#pragma unroll
+    for (int k = 0; k < P * P / 256; k++) {
+      const int i = tid + 256 * k, p = i / P, q = i % P;
+      va[k] = Fa[(int64_t)p * a.f_sp[0] + (int64_t)q * a.f_sq[0]];
+      vb[k] = Fb[(int64_t)p * a.f_sp[1] + (int64_t)q * a.f_sq[1]];
     }
+#pragma unroll
+    for (int k = 0; k < P * P / 256; k++) { fA[tid + 256 * k] = va[k]; fB[tid + 256 * k] = vb[k]; }
   }
   __syncthreads();
 
@@ -215,10 +221,19 @@ __global__ __launch_bounds__(512, 2) void kron_pair64_f64_kernel(const StepArgs 
   {
     const double* Fa = (const double*)a.f[0] + (size_t)bt * a.f_batch[0];
     const double* Fb = (const double*)a.f[1] + (size_t)bt * a.f_batch[1];
-    for (int i = tid; i < P * P; i += 512) {
-      const int p = i / P, q = i % P;
-      fA[i] = Fa[(int64_t)p * a.f_sp[0] + (int64_t)q * a.f_sq[0]];
-      fB[p * P + (q ^ (4 * (p & 3)))] = Fb[(int64_t)p * a.f_sp[1] + (int64_t)q * a.f_sq[1]];
+    // (loads first, then the LDS writes: one memory round trip in front of the first product, not eight)
+    double va[P * P / 512], vb[P * P / 512];
+#pragma unroll
+    for (int k = 0; k < P * P / 512; k++) {
+      const int i = tid + 512 * k, p = i / P, q = i % P;
+      va[k] = Fa[(int64_t)p * a.f_sp[0] + (int64_t)q * a.f_sq[0]];
+      vb[k] = Fb[(int64_t)p * a.f_sp[1] + (int64_t)q * a.f_sq[1]];
+    }
+#pragma unroll
+    for (int k = 0; k < P * P / 512; k++) {
+      const int i = tid + 512 * k, p = i / P, q = i % P;
+      fA[i] = va[k];
+      fB[p * P + (q ^ (4 * (p & 3)))] = vb[k];
     }
   }
   __syncthreads();

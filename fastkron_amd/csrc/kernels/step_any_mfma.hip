@@ -87,12 +87,24 @@ __global__ __launch_bounds__(256, 2) void kron_step_any_kernel(const StepArgs a,
   {
     const T* F = (const T*)a.f[0] + (size_t)bt * a.f_batch[0];
     const uint32_t perK = g.pcPad * Qp;                // rows pc .. pcPad-1 of a lane group are zero
-    for (uint32_t idx = tid; idx < 4 * perK; idx += 256) {
-      const uint32_t k = idx / perK, rem = idx - k * perK, c = rem / Qp, q = rem - c * Qp;
-      const uint32_t p = k * pc + c, qq = 16 * ib0 + q;
-      T v = (T)0;
-      if (c < pc && p < g.P && qq < g.Q) v = F[(int64_t)p * a.f_sp[0] + (int64_t)qq * a.f_sq[0]];
-      fl[k * g.kStride + c * Qp + q] = v;
+    // eight loads of a thread go out before the first LDS write waits for one: a loop of load, wait, write would
+    // put one memory round trip per element of a thread in front of the first product
+    constexpr int kBatch = 8;
+    for (uint32_t base = tid; base < 4 * perK; base += kBatch * 256) {
+      T v[kBatch];
+      uint32_t dst[kBatch];
+#pragma unroll
+      for (int u = 0; u < kBatch; u++) {
+        const uint32_t idx = base + u * 256;
+        const uint32_t k = idx / perK, rem = idx - k * perK, c = rem / Qp, q = rem - c * Qp;
+        const uint32_t p = k * pc + c, qq = 16 * ib0 + q;
+        v[u] = (T)0;
+        if (idx < 4 * perK && c < pc && p < g.P && qq < g.Q) v[u] = F[(int64_t)p * a.f_sp[0] + (int64_t)qq * a.f_sq[0]];
+        dst[u] = k * g.kStride + c * Qp + q;
+      }
+#pragma unroll
+      for (int u = 0; u < kBatch; u++)
+        if (base + u * 256 < 4 * perK) fl[dst[u]] = v[u];
     }
   }
   __syncthreads();
