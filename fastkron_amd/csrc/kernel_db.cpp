@@ -1,7 +1,6 @@
 #include "kernel_db.h"
 
 #include <cstdio>
-#include <cstdlib>
 #include <fstream>
 #include <sstream>
 
@@ -102,6 +101,7 @@ void registerGenericKernels(std::vector<KernelInfo>& out) {
 }
 
 // ---- whole-row kernel for four fused 16x16 fp32 factors ----
+constexpr uint64_t kRow16MinBlocks = 96;
 static bool row16CanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
                         const DeviceInfo& dev) {
   const uint32_t nf = hi - lo + 1;
@@ -111,6 +111,11 @@ static bool row16CanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, 
   for (uint32_t i = nf; i < 4; i++) rows *= 16;
   if (p.colsBefore(hi) != kk || p.M % rows) return false;   // the group covers whole rows, M a whole number of blocks
   if (first && p.opX == 2) return false;
+  // A block is one workgroup's work for about 20 us (256 KB through one CU, 14 us of its matrix pipes): with few
+  // blocks the kernels that spread a block over many CUs finish sooner (measured crossover between 64 and 128 blocks).
+  // (Shorter chains have no such alternative when their factors differ per batch entry, and go to the wave-per-block
+  // kernel anyway when they do not.)
+  if (nf == 4 && (uint64_t)p.M * p.batch < kRow16MinBlocks) return false;
   return dev.ldsPerBlock >= 131072 && k.dt == p.dt;
 }
 static hipError_t row16Launch(const KernelInfo& k, const StepArgs& a, hipStream_t s) {

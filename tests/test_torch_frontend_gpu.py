@@ -125,7 +125,7 @@ def test_gradcheck(mm, m, n, p, q, trX, trF):
 def test_gradient_of_x_only_is_one_fused_call(mm):
     import torch
     import fastkron_amd as fk
-    x, fs, _ = make(mm, 16, 4, 16, 16, torch.float32, False, False, seed=3, high=3)
+    x, fs, _ = make(mm, 96, 4, 16, 16, torch.float32, False, False, seed=3, high=3)
     x = x.detach().requires_grad_(True)
     z = fk.gemkm(x, fs) if mm == "mkm" else fk.gekmm(fs, x)
     w = torch.randint(0, 3, z.shape, generator=torch.Generator().manual_seed(5)).float().cuda()
