@@ -267,6 +267,8 @@ fastKronError Handle::trySplitLeadingTrailing(const KronProblem& p, void* temp1,
   else if (tp == 32 || tp == 64)      maxT = 2;
   else if (p.dt == DType::F32) maxT = (tp == 8) ? 5 : (tp == 16) ? 4 : 0;
   else if (tp == 16)           maxT = 3;
+  // (few rows of 32^3, fp32: the pair kernel spreads them over more CUs than one workgroup per row does)
+  if (p.dt == DType::F32 && tp == 32 && (uint64_t)p.M * (p.K() / 32768) * p.batch < 96) maxT = 2;
   // (few blocks of 16^4: the wave-per-block kernel for three factors spreads them over more CUs)
   if (p.dt == DType::F32 && tp == 16 && p.N >= 4 && (uint64_t)p.M * (p.K() / 65536) * p.batch < 96) maxT = 3;
   if (maxT == 0 && tp >= 9 && tp <= 15) maxT = 3;       // zero-padded form of the 16x16x3 wave-per-block kernel

@@ -172,12 +172,16 @@ static hipError_t row32Launch(const KernelInfo&, const StepArgs& a, hipStream_t 
 static bool row32Check(const KernelInfo&, const StepArgs& a) { return row32x16x3Supported(a); }
 
 // ---- whole-row kernel for three fused 32x32 fp32 factors ----
+constexpr uint64_t kRow32MinRows = 96;
 static bool row32x3CanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
                           const DeviceInfo&) {
   if (p.dt != DType::F32 || p.mm != MMType::MKM || hi - lo + 1 != 3 || p.forward) return false;
   for (uint32_t i = lo; i <= hi; i++) if (p.P[i] != 32 || p.Q[i] != 32) return false;
   if (p.colsBefore(hi) != 32768) return false;
   if (first && p.opX == 2) return false;
+  // a row is one workgroup's work for about 17 us: with few rows the pair kernel (a wave per 1024-column block) plus
+  // one step across the blocks finishes sooner (measured crossover between 64 and 128 rows)
+  if ((uint64_t)p.M * p.batch < kRow32MinRows) return false;
   return k.dt == p.dt;
 }
 static hipError_t row32x3Launch(const KernelInfo&, const StepArgs& a, hipStream_t s) { return launchRow32x3(a, s); }

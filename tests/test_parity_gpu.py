@@ -379,8 +379,8 @@ def test_chains_split_into_pair_kernel_plus_leading_kmm_step(fk, M, Ps, dt):
     matrix-core steps across the blocks."""
     check(fk, ko.MKM, M, Ps, Ps, dt, alpha=1.5, beta=0.5, seed=131)
     plan = fk.last_plan()
-    # (fp32 chains that end in three 32x32 factors fuse those three instead of two)
-    fused = 3 if dt == np.float32 and Ps[-3:] == [32] * 3 else 2
+    # (fp32 chains that end in three 32x32 factors fuse those three instead of two, from 96 blocks of 32^3 on)
+    fused = 3 if dt == np.float32 and Ps[-3:] == [32] * 3 and M * int(np.prod(Ps[:-3])) >= 96 else 2
     assert len(plan) == len(Ps) - fused + 1 and plan[0][2].startswith("mkm_") and all("kmm_" in k for _, _, k in plan[1:]), plan
     check(fk, ko.MKM, M, Ps, Ps, dt, alpha=1.0, beta=0.0, seed=132, opFs=ko.OP_T)
     check(fk, ko.MKM, M, Ps, Ps, dt, alpha=1.0, beta=1.0, seed=133, batch=2, share_f=True)
@@ -616,11 +616,12 @@ def test_kmm_layout_pair_of_16x16_factors(fk, M, Ps, launches, dt):
     check(fk, ko.KMM, M, Ps, Ps, dt, alpha=1.0, beta=0.0, seed=704, integer=True)
 
 
-@pytest.mark.parametrize("M,Ps,launches", [(1, [32] * 3, 1), (5, [32] * 3, 1), (64, [32] * 3, 1), (2, [32] * 4, 2),
-                                           (1, [4, 32, 32, 32], 2), (1, [32] * 5, 3)])
+@pytest.mark.parametrize("M,Ps,launches", [(96, [32] * 3, 1), (101, [32] * 3, 1), (128, [32] * 3, 1), (3, [32] * 4, 2),
+                                           (24, [4, 32, 32, 32], 2), (1, [32] * 5, 3)])
 def test_whole_row_kernel_for_three_32x32_factors(fk, M, Ps, launches):
     """fp32 32x32^3 on rows (or contiguous blocks) of 32768 columns: one launch, one LDS exchange; longer chains
-    apply the three trailing factors block by block and the leading ones in the KMM layout."""
+    apply the three trailing factors block by block and the leading ones in the KMM layout.  (With fewer than 96
+    blocks the pair kernel plus one more step is faster and is chosen instead.)"""
     check(fk, ko.MKM, M, Ps, Ps, np.float32, alpha=1.5, beta=0.5, seed=1001)
     plan = fk.last_plan()
     assert any("_f_32x32_32x32_3_1x32768_" in k for _, _, k in plan) and len(plan) == launches, plan
