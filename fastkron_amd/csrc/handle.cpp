@@ -193,7 +193,14 @@ bool Handle::mergeSmallFactors(const KronProblem& p, KronProblem* out) {
   // fp32 GeKMM already fuses small factors in registers; everything else gains from merging
   if (p.mm == MMType::KMM && p.dt == DType::F32) return false;
   if (p.batch > 1) for (uint32_t i = 0; i < p.N; i++) if (p.strideF[i] != 0) return false;
-  const uint32_t target = (p.dt == DType::F32) ? 16 : 64;
+  // fp32: 16x16 products.  fp64: 64x64 products when the chain holds 8x8 (or 32x32) factors, which do not pack into
+  // 16x16 ones; chains of 2x2 and 4x4 factors alone run faster as 16x16 products (a quarter of the multiplications,
+  // and the wave-per-block kernel for three 16x16 factors: dgemkm 1024x4^8 0.57 -> 0.47 ms, 1024x4^6 60 -> 20 us).
+  uint32_t target = 16;
+  if (p.dt == DType::F64) {
+    for (uint32_t i = 0; i < p.N; i++)
+      if (p.P[i] == p.Q[i] && (p.P[i] == 8 || p.P[i] == 32)) target = 64;
+  }
   // groups of adjacent square power-of-two factors, formed from the last factor towards the first, each as
   // large as fits the target size
   struct Grp { uint32_t lo, hi, size; };

@@ -46,7 +46,7 @@ class Handle {
   // Returns fastKronKernelNotFound when the problem does not have that form.
   fastKronError trySplitLeadingTrailing(const KronProblem& p, void* temp1, void* temp2);
   // Chains of 2x2 / 4x4 (fp64: also 8x8) factors: adjacent factors are replaced by their Kronecker product
-  // (16x16 in fp32, 64x64 in fp64), computed into the handle's workspace by one small launch, so that the
+  // (16x16; 64x64 in fp64 when the chain holds 8x8 or 32x32 factors), computed into the handle's workspace by one small launch, so that the
   // kernels for those sizes apply.  Returns false when nothing is merged; on true `out` is the merged problem.
   bool mergeSmallFactors(const KronProblem& p, KronProblem* out);
 

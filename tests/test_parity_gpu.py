@@ -494,10 +494,12 @@ def test_kmm_six_4x4_factors_in_one_launch(fk, M):
     (ko.MKM, 4, [4] * 7, np.float32, 2),          # -> 4, 16x16^3: block kernel on 16 virtual rows + leading 4x4
     (ko.MKM, 3, [4] * 7, np.float32, None),       # same, but 12 virtual rows are no whole block: shorter launches
     (ko.MKM, 5, [2, 4, 2, 4, 8, 2], np.float32, None),
-    (ko.MKM, 8, [4] * 6, np.float64, 1),          # -> 64x64^2: the fp64 pair kernel
-    (ko.MKM, 2, [8] * 5, np.float64, 2),          # -> 8, 64x64^2: pair kernel + leading 8x8
-    (ko.MKM, 3, [2] * 9, np.float64, 2),          # -> 8, 64
-    (ko.KMM, 64, [4] * 6, np.float64, 2),         # -> 64x64^2 on the KMM layout
+    (ko.MKM, 8, [4] * 6, np.float64, 1),          # -> 16x16^3: chains of 2x2 / 4x4 alone become 16x16 in fp64 too
+    (ko.MKM, 2, [8] * 5, np.float64, 2),          # -> 8, 64x64^2 (8x8 factors: 64x64 products): pair kernel + leading 8x8
+    (ko.MKM, 3, [2] * 9, np.float64, None),       # -> 2, 16, 16
+    (ko.MKM, 16, [2] * 9, np.float64, 2),         # the same with whole blocks of rows: two 16x16 in one launch + the 2x2
+    (ko.MKM, 4, [2, 4, 8, 4, 2], np.float64, None),   # an 8x8 in the chain: 64x64 products
+    (ko.KMM, 64, [4] * 6, np.float64, 2),         # -> 16x16^3 on the KMM layout: a pair and a single step
     (ko.KMM, 20, [2] * 7, np.float64, None),
 ])
 def test_small_factors_are_merged_into_their_kronecker_products(fk, mm, M, Ps, dt, launches):
