@@ -27,7 +27,7 @@ EXPORTS = [
     "skmmForwardStridedBatched", "dkmmForwardStridedBatched",
 ]
 
-EXT_EXPORTS = ["fastKronGetLastPlan", "fastKronSetTunedDB"]     # include/fastkron_ext.h
+EXT_EXPORTS = ["fastKronGetLastPlan", "fastKronSetTunedDB", "fastKronSetPlanOnly", "fastKronGetLastLaunches"]     # include/fastkron_ext.h
 
 _lib = None
 
@@ -87,6 +87,9 @@ def load():
     lib.fastKronGetLastPlan.argtypes = [vp, ctypes.c_char_p, ctypes.c_size_t]
     lib.fastKronGetLastPlan.restype = ctypes.c_size_t
     lib.fastKronSetTunedDB.argtypes = [vp, ctypes.c_char_p]
+    lib.fastKronSetPlanOnly.argtypes = [vp, cint]
+    lib.fastKronGetLastLaunches.argtypes = [vp, ctypes.c_char_p, ctypes.c_size_t]
+    lib.fastKronGetLastLaunches.restype = ctypes.c_size_t
     for n in EXPORTS:
         f = getattr(lib, n)
         if f.restype is ctypes.c_int and n not in ("fastKronGetBackends",):

@@ -82,6 +82,23 @@ size_t fastKronGetLastPlan(fastKronHandle handle, char* buf, size_t bufLen) {
   return s.size();
 }
 
+fastKronError fastKronSetPlanOnly(fastKronHandle handle, int on) {
+  if (!handle) return fastKronInvalidArgument;
+  H(handle)->setPlanOnly(on != 0);
+  return fastKronSuccess;
+}
+
+size_t fastKronGetLastLaunches(fastKronHandle handle, char* buf, size_t bufLen) {
+  if (!handle) return 0;
+  const std::string& s = H(handle)->lastLaunches();
+  if (buf && bufLen) {
+    const size_t n = s.size() < bufLen - 1 ? s.size() : bufLen - 1;
+    memcpy(buf, s.data(), n);
+    buf[n] = 0;
+  }
+  return s.size();
+}
+
 fastKronError fastKronSetTunedDB(fastKronHandle handle, const char* path) {
   if (!handle) return fastKronInvalidArgument;
   H(handle)->setTunedDB(path);
@@ -138,6 +155,14 @@ fastKronError run(fastKronHandle handle, fastKronBackend backend, const Call& c,
       p.inter[i] = c.inter ? c.inter[i] : nullptr;
       if (c.strideInter) { p.strideInter[i] = c.strideInter[i]; p.haveStrideInter = true; }
     }
+  }
+  // A strided-batched call with a single batch entry never uses its strides: they are cleared here so that no
+  // plan that re-views the rows of one problem as batch entries of another (the two-part plan does) can carry a
+  // caller's stride into a batch index of its own.
+  if (p.batch == 1) {
+    p.strideX = p.strideZ = p.strideY = 0;
+    for (uint32_t i = 0; i < c.N; i++) { p.strideF[i] = 0; p.strideInter[i] = 0; }
+    p.haveStrideInter = false;
   }
   return H(handle)->xgemm(p, backend, t1, t2);
 }

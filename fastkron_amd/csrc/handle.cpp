@@ -25,7 +25,22 @@ Handle::Handle(uint32_t backends) : backends_(backends) {
 }
 
 Handle::~Handle() {
-  if (mergeWs_) (void)hipFree(mergeWs_);
+  if (mergeWs_ && mergeWsOwned_) (void)hipFree(mergeWs_);
+  if (mergeWsEvent_) (void)hipEventDestroy(mergeWsEvent_);
+}
+
+void Handle::setPlanOnly(bool on) {
+  planOnly_ = on;
+  if (on && !dev_.valid) {
+    // the device the library is written for: 256 compute units, 160 KB of LDS per workgroup
+    dev_.cus = 256; dev_.ldsPerBlock = 160 * 1024; dev_.waveSize = 64;
+  }
+  if (on && !mergeWs_) {
+    // never dereferenced: in this mode no launch is made
+    mergeWs_ = (void*)(uintptr_t)0x7f0000000000ull;
+    mergeWsBytes_ = (size_t)kMaxMergeGroups * 64 * 64 * sizeof(double);
+    mergeWsOwned_ = false;
+  }
 }
 
 void Handle::setTunedDB(const char* path) {
@@ -63,15 +78,34 @@ fastKronError Handle::initHIP(void* ptrToStream) {
   if (!mergeWs_) {
     mergeWsBytes_ = (size_t)kMaxMergeGroups * 64 * 64 * sizeof(double);
     if (hipMalloc(&mergeWs_, mergeWsBytes_) != hipSuccess) { mergeWs_ = nullptr; mergeWsBytes_ = 0; }
+    mergeWsOwned_ = mergeWs_ != nullptr;
+    if (mergeWs_ && hipEventCreateWithFlags(&mergeWsEvent_, hipEventDisableTiming) != hipSuccess) mergeWsEvent_ = nullptr;
   }
   return fastKronSuccess;
+}
+
+// The merged-factor workspace is the one piece of device state the handle owns.  A call on a new stream may
+// overwrite it while launches of an earlier call on another stream still read it; the new stream is therefore made
+// to wait for everything the old stream has been given so far.  (Nothing is recorded while either stream is being
+// captured into a graph: a handle that is used under capture stays on one stream.)
+void Handle::orderWorkspaceBehind(hipStream_t next) {
+  if (!mergeWsUsed_ || !mergeWsEvent_ || next == mergeWsStream_) return;
+  hipStreamCaptureStatus c0 = hipStreamCaptureStatusNone, c1 = hipStreamCaptureStatusNone;
+  (void)hipStreamIsCapturing(mergeWsStream_, &c0);
+  (void)hipStreamIsCapturing(next, &c1);
+  if (c0 == hipStreamCaptureStatusNone && c1 == hipStreamCaptureStatusNone &&
+      hipEventRecord(mergeWsEvent_, mergeWsStream_) == hipSuccess)
+    (void)hipStreamWaitEvent(next, mergeWsEvent_, 0);
+  mergeWsUsed_ = false;
 }
 
 fastKronError Handle::setStream(fastKronBackend backend, void* ptrToStream) {
   if (!ptrToStream) return fastKronInvalidArgument;                    // reference handle.cpp:94
   if (!hasBackend(backend)) return fastKronBackendNotAvailable;        // reference handle.cpp:95
   if (backend != fastKronBackend_HIP) return fastKronBackendNotAvailable;
-  stream_ = *(hipStream_t*)ptrToStream;
+  hipStream_t next = *(hipStream_t*)ptrToStream;
+  if (next != stream_ && !planOnly_) orderWorkspaceBehind(next);
+  stream_ = next;
   return fastKronSuccess;
 }
 
@@ -134,8 +168,9 @@ fastKronError Handle::xgemm(KronProblem p, fastKronBackend backend, void* temp1,
     p.opX = fastKronOp_N;
   }
 
-  fastKronError e = ensureDevice();
+  fastKronError e = planOnly_ ? fastKronSuccess : ensureDevice();
   if (e != fastKronSuccess) return e;
+  launchLog_.clear();
 
   {
     KronProblem merged;
@@ -145,14 +180,14 @@ fastKronError Handle::xgemm(KronProblem p, fastKronBackend backend, void* temp1,
   Plan plan;
   const std::string key = p.str();
   bool have = false;
-  if (!p.forward) have = db_.lookupTuned(key, &plan);
+  if (!p.forward) have = db_.lookupTuned(key, &plan) && db_.validPlan(p, plan, dev_);
   // chains longer than one whole-block kernel: the two-part plan, when the problem and the buffers allow it
   // (the tuner only searches single chains of launches, so it is asked after this)
   if (!have && useFusion()) {
     e = trySplitLeadingTrailing(p, temp1, temp2);
     if (e != fastKronKernelNotFound) return e;
   }
-  if (!have && canTune() && !p.forward) {
+  if (!have && canTune() && !p.forward && !planOnly_) {
     e = tune(p, &plan);
     if (e != fastKronSuccess) return e;
     have = true;
@@ -183,6 +218,7 @@ fastKronError Handle::xgemm(KronProblem p, fastKronBackend backend, void* temp1,
   lastPlan_ = key;
   for (auto& s : plan)
     lastPlan_ += ";" + std::to_string(s.lo) + "-" + std::to_string(s.hi) + ":" + db_.kernels()[s.kernel].name;
+  if (planOnly_) { launchLog_.clear(); return execute(p, plan, temp1, temp2, true); }
   return execute(p, plan, temp1, temp2);
 }
 
@@ -251,7 +287,11 @@ bool Handle::mergeSmallFactors(const KronProblem& p, KronProblem* out) {
     wsOff += (bytes + 255) & ~(size_t)255;
     q.P[g] = G.size; q.Q[g] = G.size; q.F[g] = mg.dst;
   }
-  if (launchMergeFactors(ma, p.dt, stream_) != hipSuccess) return false;
+  if (!planOnly_) {
+    if (mergeWsUsed_ && mergeWsStream_ != stream_) orderWorkspaceBehind(stream_);
+    if (launchMergeFactors(ma, p.dt, stream_) != hipSuccess) return false;
+    mergeWsStream_ = stream_; mergeWsUsed_ = true;
+  }
   *out = q;
   return true;
 }
@@ -292,8 +332,9 @@ fastKronError Handle::trySplitLeadingTrailing(const KronProblem& p, void* temp1,
   if (p.batch > 1) {
     if (p.strideX != (uint64_t)p.M * K || p.strideZ != (uint64_t)p.M * K) return fastKronKernelNotFound;
     if (p.Y && p.beta != 0.0 && p.strideY != (uint64_t)p.M * K) return fastKronKernelNotFound;
-    for (uint32_t i = 0; i < g; i++) if (p.strideF[i] != 0) return fastKronKernelNotFound;
   }
+  // the leading factors are read by a problem whose batch entries are the rows of this one: shared factors only
+  for (uint32_t i = 0; i < g; i++) if (p.strideF[i] != 0) return fastKronKernelNotFound;
   if ((uint64_t)p.M * p.batch > 65535 || (uint64_t)p.M * KA >= (1ull << 31)) return fastKronKernelNotFound;
 
   // part 1: trailing factors, X -> temp1, no epilogue
@@ -316,6 +357,7 @@ fastKronError Handle::trySplitLeadingTrailing(const KronProblem& p, void* temp1,
   q2.X = temp1; q2.strideX = K;
   q2.strideZ = K; q2.strideY = K;
   q2.batch = p.batch * p.M; q2.strided = true;
+  for (uint32_t i = 0; i < g; i++) q2.strideF[i] = 0;
   Plan plan2 = db_.selectOnline(q2, dev_, true);
   // more than two leading launches ping-pong between temp2 and Z, which must then not be Y
   if (plan2.size() > 2 && p.Y == p.Z && p.beta != 0.0) return fastKronKernelNotFound;
@@ -326,6 +368,11 @@ fastKronError Handle::trySplitLeadingTrailing(const KronProblem& p, void* temp1,
     lastPlan_ += ";" + std::to_string(g + s.lo) + "-" + std::to_string(g + s.hi) + ":" + db_.kernels()[s.kernel].name;
   for (auto& s : plan2)
     lastPlan_ += ";" + std::to_string(s.lo) + "-" + std::to_string(s.hi) + ":" + db_.kernels()[s.kernel].name;
+  if (planOnly_) {
+    launchLog_.clear();
+    (void)execute(q1, plan1, nullptr, nullptr, true);
+    return execute(q2, plan2, temp2, nullptr, true);
+  }
   fastKronError e = execute(q1, plan1, nullptr, nullptr);
   if (e != fastKronSuccess) return e;
   return execute(q2, plan2, temp2, nullptr);
@@ -422,8 +469,19 @@ fastKronError Handle::execute(const KronProblem& p, const Plan& plan, void* temp
       for (uint32_t j = 0; j < a.nf && j < kMaxFused; j++)
         c.f[j] = (const char*)a.f[j] + (size_t)b0 * a.f_batch[j] * es;
       if (dryRun) {
-        if (k.check && !k.check(k, c)) return fastKronKernelNotFound;
-        break;                                        // every chunk has the same strides and alignment class
+        if (k.check && !k.check(k, c)) return fastKronKernelNotFound;   // every chunk: its base pointers differ
+        if (planOnly_) {
+          char line[768];
+          int n = snprintf(line, sizeof(line), "kernel=%s lo=%u hi=%u M=%u batch=%u Kin=%llu Kout=%llu in=%p out=%p y=%p "
+                           "in_batch=%llu out_batch=%llu y_batch=%llu f_batch=", k.name.c_str(), s.lo, s.hi, c.M, c.batch,
+                           (unsigned long long)c.Kin, (unsigned long long)c.Kout, c.in, c.out, c.y,
+                           (unsigned long long)c.in_batch, (unsigned long long)c.out_batch, (unsigned long long)c.y_batch);
+          launchLog_.append(line, n > 0 ? (size_t)n : 0);
+          for (uint32_t j = 0; j < c.nf && j < kMaxFused; j++)
+            launchLog_ += (j ? "," : "") + std::to_string(c.f_batch[j]);
+          launchLog_ += "\n";
+        }
+        continue;
       }
       hipError_t he = k.launch(k, c, stream_);
       if (he != hipSuccess) {

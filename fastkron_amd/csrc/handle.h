@@ -53,12 +53,20 @@ class Handle {
   const std::string& lastPlan() const { return lastPlan_; }
   void setTunedDB(const char* path);
 
+  // Plan-only mode: calls go through every check, the planner and the kernels' argument checks, but nothing is
+  // launched and no device is needed (an MI355X is assumed); lastLaunches() then lists the launches the call
+  // would have made, one per line, with their buffers, strides and batch counts.
+  void setPlanOnly(bool on);
+  bool planOnly() const { return planOnly_; }
+  const std::string& lastLaunches() const { return launchLog_; }
+
   KernelDB& db() { return db_; }
   const DeviceInfo& device() const { return dev_; }
   hipStream_t stream() const { return stream_; }
 
  private:
   fastKronError ensureDevice();
+  void orderWorkspaceBehind(hipStream_t next);
 
   uint32_t backends_;
   uint32_t options_ = fastKronOptionsNone;
@@ -71,6 +79,12 @@ class Handle {
   std::string lastPlan_;
   void* mergeWs_ = nullptr;                           // device memory for merged factors, allocated by initHIP
   size_t mergeWsBytes_ = 0;
+  bool mergeWsOwned_ = false;
+  hipStream_t mergeWsStream_ = nullptr;               // stream of the last call that wrote the workspace
+  bool mergeWsUsed_ = false;
+  hipEvent_t mergeWsEvent_ = nullptr;                 // orders a new stream behind the last user of the workspace
+  bool planOnly_ = false;
+  std::string launchLog_;
 };
 
 }  // namespace fk

@@ -422,6 +422,20 @@ Plan KernelDB::selectOnline(const KronProblem& p, const DeviceInfo& dev, bool al
   return plan;
 }
 
+bool KernelDB::validPlan(const KronProblem& p, const Plan& plan, const DeviceInfo& dev) const {
+  if (plan.empty() || p.N == 0) return false;
+  int64_t expectHi = (int64_t)p.N - 1;
+  for (size_t l = 0; l < plan.size(); l++) {
+    const PlanStep& s = plan[l];
+    if (s.kernel < 0 || (size_t)s.kernel >= kernels_.size()) return false;
+    if ((int64_t)s.hi != expectHi || s.lo > s.hi || s.hi - s.lo + 1 > kMaxFused) return false;
+    const KernelInfo& k = kernels_[s.kernel];
+    if (!k.canRun(k, p, s.lo, s.hi, l == 0, s.lo == 0, dev)) return false;
+    expectHi = (int64_t)s.lo - 1;
+  }
+  return expectHi == -1;
+}
+
 bool KernelDB::lookupTuned(const std::string& key, Plan* plan) const {
   auto it = tuned_.find(key);
   if (it == tuned_.end()) return false;

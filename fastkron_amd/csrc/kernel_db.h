@@ -62,6 +62,10 @@ class KernelDB {
   std::vector<int> candidates(const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool last,
                               const DeviceInfo& dev) const;
 
+  // True when `plan` applies every factor of `p` exactly once, last factor first, and every step's kernel
+  // accepts its factor range (a plan read from a file is not trusted before it passes this).
+  bool validPlan(const KronProblem& p, const Plan& plan, const DeviceInfo& dev) const;
+
   // Tuned plans, keyed by the problem string.
   bool lookupTuned(const std::string& key, Plan* plan) const;
   void storeTuned(const std::string& key, const Plan& plan, float ms);

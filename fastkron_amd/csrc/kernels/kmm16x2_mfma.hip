@@ -180,13 +180,7 @@ bool kmm16x2Supported(const StepArgs& a, DType dt) {
 
 template <typename T, bool EXACT>
 static hipError_t launchKmm16x2T(const StepArgs& a, hipStream_t stream) {
-  static int cus = 0;
-  if (!cus) {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    cus = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
-              ? prop.multiProcessorCount : 256;
-  }
+  const int cus = deviceCUs();
   const uint32_t P = a.p[0];
   const uint32_t mTiles = (a.M + 15) / 16;
   const uint32_t totalTiles = (uint32_t)((a.Kin / (P * P)) * mTiles);

@@ -126,15 +126,16 @@ bool kmm4x6Supported(const StepArgs& a) {
 
 hipError_t launchKmm4x6(const StepArgs& a, hipStream_t stream) {
   if (!kmm4x6Supported(a)) return hipErrorInvalidValue;
-  static bool attrSet = false;
-  if (!attrSet) {
+  static PerDeviceOnce attrOnce;
+  const int devIdx = launchDeviceIndex();
+  if (!attrOnce.done(devIdx)) {
     hipError_t e = hipFuncSetAttribute((const void*)kron_kmm4x6_kernel<true>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)kK6LdsBytes);
     if (e != hipSuccess) return e;
     e = hipFuncSetAttribute((const void*)kron_kmm4x6_kernel<false>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)kK6LdsBytes);
     if (e != hipSuccess) return e;
-    attrSet = true;
+    attrOnce.mark(devIdx);
   }
   const uint32_t mTiles = a.M / 8;
   dim3 grid(mTiles, a.batch), block(512);

@@ -182,13 +182,7 @@ bool kmm64F64Supported(const StepArgs& a) {
 
 hipError_t launchKmm64F64(const StepArgs& a, hipStream_t stream) {
   if (!kmm64F64Supported(a)) return hipErrorInvalidValue;
-  static int cus = 0;
-  if (!cus) {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    cus = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
-              ? prop.multiProcessorCount : 256;
-  }
+  const int cus = deviceCUs();
   const uint64_t S = a.Kin / 64;
   const uint32_t mBlocks = (a.M + 63) / 64;
   const uint32_t totalTiles = (uint32_t)(S * mBlocks);

@@ -1,9 +1,35 @@
 // Launch entry points of the kernel translation units (one per .hip file).
 #pragma once
 #include <hip/hip_runtime.h>
+#include <atomic>
 #include "../problem.h"
 
 namespace fk {
+
+// Function attributes and the number of compute units belong to a device, not to the process: the launchers
+// keep both per device, so that handles on different GPUs of one process (and threads) do not share them.
+constexpr int kMaxDevices = 64;
+inline int launchDeviceIndex() {
+  int d = 0;
+  if (hipGetDevice(&d) != hipSuccess || d < 0 || d >= kMaxDevices) d = 0;
+  return d;
+}
+inline int deviceCUs() {
+  static std::atomic<int> cus[kMaxDevices];
+  const int d = launchDeviceIndex();
+  int c = cus[d].load(std::memory_order_relaxed);
+  if (c == 0) {
+    hipDeviceProp_t prop;
+    c = (hipGetDeviceProperties(&prop, d) == hipSuccess && prop.multiProcessorCount > 0) ? prop.multiProcessorCount : 256;
+    cus[d].store(c, std::memory_order_relaxed);
+  }
+  return c;
+}
+struct PerDeviceOnce {               // "done once on this device" for set-up such as hipFuncSetAttribute
+  std::atomic<uint64_t> mask{0};
+  bool done(int dev) const { return (mask.load(std::memory_order_acquire) >> dev) & 1; }
+  void mark(int dev) { mask.fetch_or(1ull << dev, std::memory_order_release); }
+};
 
 // Any shape, one factor per launch.
 hipError_t launchGenericStep(const StepArgs& a, DType dt, hipStream_t stream);

@@ -397,13 +397,7 @@ bool pairMfmaSupported(const StepArgs& a, DType dt) {
 
 template <typename T, int P>
 static hipError_t launchPairT(const StepArgs& a, hipStream_t stream) {
-  static int cus = 0;
-  if (!cus) {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    cus = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
-              ? prop.multiProcessorCount : 256;
-  }
+  const int cus = deviceCUs();
   const size_t ldsBytes = 2 * P * P * sizeof(T);
   uint32_t wgs = (uint32_t)cus * (P == 32 ? 4 : 2);   // persistent; the 32x32 kernels need few registers
   if (a.batch > 1) wgs = (wgs + a.batch - 1) / a.batch;
@@ -411,15 +405,16 @@ static hipError_t launchPairT(const StepArgs& a, hipStream_t stream) {
   if (wgs > need) wgs = need;
   if (wgs == 0) wgs = 1;
   dim3 grid(wgs, a.batch), block(256);
-  static bool attr[2] = {false, false};
+  static PerDeviceOnce attrOnce[2];
+  const int devIdx = launchDeviceIndex();
   const bool y = a.y && a.epilogue;
-  if (!attr[y]) {
+  if (!attrOnce[y].done(devIdx)) {
     hipError_t e = y ? hipFuncSetAttribute((const void*)kron_pair_kernel<T, P, true>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes)
                      : hipFuncSetAttribute((const void*)kron_pair_kernel<T, P, false>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes);
     if (e != hipSuccess) return e;
-    attr[y] = true;
+    attrOnce[y].mark(devIdx);
   }
   if (y) hipLaunchKernelGGL((kron_pair_kernel<T, P, true>), grid, block, ldsBytes, stream, a);
   else   hipLaunchKernelGGL((kron_pair_kernel<T, P, false>), grid, block, ldsBytes, stream, a);
@@ -427,28 +422,23 @@ static hipError_t launchPairT(const StepArgs& a, hipStream_t stream) {
 }
 
 static hipError_t launchPair64(const StepArgs& a, hipStream_t stream) {
-  static int cus = 0;
-  if (!cus) {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    cus = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
-              ? prop.multiProcessorCount : 256;
-  }
+  const int cus = deviceCUs();
   uint32_t wgs = (uint32_t)cus;                     // persistent, one workgroup per CU
   if (a.batch > 1) wgs = (wgs + a.batch - 1) / a.batch;
   const uint32_t need = (a.M + kPair64Waves - 1) / kPair64Waves;
   if (wgs > need) wgs = need;
   if (wgs == 0) wgs = 1;
   dim3 grid(wgs, a.batch), block(64 * kPair64Waves);
-  static bool attr[2] = {false, false};
+  static PerDeviceOnce attrOnce[2];
+  const int devIdx = launchDeviceIndex();
   const bool y = a.y && a.epilogue;
-  if (!attr[y]) {
+  if (!attrOnce[y].done(devIdx)) {
     hipError_t e = y ? hipFuncSetAttribute((const void*)kron_pair64_f64_kernel<true>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)kPair64LdsBytes)
                      : hipFuncSetAttribute((const void*)kron_pair64_f64_kernel<false>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)kPair64LdsBytes);
     if (e != hipSuccess) return e;
-    attr[y] = true;
+    attrOnce[y].mark(devIdx);
   }
   if (y) hipLaunchKernelGGL((kron_pair64_f64_kernel<true>), grid, block, kPair64LdsBytes, stream, a);
   else   hipLaunchKernelGGL((kron_pair64_f64_kernel<false>), grid, block, kPair64LdsBytes, stream, a);

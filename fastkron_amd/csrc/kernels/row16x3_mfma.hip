@@ -230,13 +230,7 @@ static void launchRow16x3T(const StepArgs& a, dim3 grid, uint32_t blocksPerBatch
 
 hipError_t launchRow16x3(const StepArgs& a, DType dt, hipStream_t stream) {
   if (!row16x3Supported(a, dt)) return hipErrorInvalidValue;
-  static int cus = 0;
-  if (!cus) {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    cus = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
-              ? prop.multiProcessorCount : 256;
-  }
+  const int cus = deviceCUs();
   const uint32_t P = a.p[0];
   const uint32_t blocksPerBatch = a.nf == 2 ? a.M / P : a.M;
   const uint64_t total = (uint64_t)blocksPerBatch * a.batch;

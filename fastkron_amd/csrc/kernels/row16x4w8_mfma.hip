@@ -291,7 +291,8 @@ bool row16x4W8Supported(const StepArgs& a) {
   // the rows of a block must be contiguous, and M must be a whole number of blocks
   if ((uint64_t)a.in_ldm != k || (uint64_t)a.out_ldm != k || (a.y && (uint64_t)a.y_ldm != k)) return false;
   if (a.M % w8Rows(a)) return false;
-  // 16-byte aligned blocks for the vector stores / Y loads
+  // 16-byte aligned blocks for the vector loads, stores and Y loads
+  if (((uintptr_t)a.in & 15) || (a.in_batch & 3)) return false;
   if (((uintptr_t)a.out & 15) || (a.out_batch & 3)) return false;
   if (a.y && (((uintptr_t)a.y & 15) || (a.y_batch & 3))) return false;
   return a.batch <= 65535;
@@ -299,24 +300,19 @@ bool row16x4W8Supported(const StepArgs& a) {
 
 hipError_t launchRow16x4W8(const StepArgs& a, hipStream_t stream) {
   if (!row16x4W8Supported(a)) return hipErrorInvalidValue;
-  static bool attrSet = false;
+  static PerDeviceOnce attrOnce;
+  const int devIdx = launchDeviceIndex();
   const size_t ldsBytes = (kW8LdsWords + 4 * 256) * sizeof(float);
-  if (!attrSet) {
+  if (!attrOnce.done(devIdx)) {
     hipError_t e = hipFuncSetAttribute((const void*)kron_row16x4w8_kernel<true>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes);
     if (e != hipSuccess) return e;
     e = hipFuncSetAttribute((const void*)kron_row16x4w8_kernel<false>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes);
     if (e != hipSuccess) return e;
-    attrSet = true;
+    attrOnce.mark(devIdx);
   }
-  static int cus = 0;
-  if (!cus) {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    cus = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
-              ? prop.multiProcessorCount : 256;
-  }
+  const int cus = deviceCUs();
   const uint32_t blocksPerBatch = a.M / w8Rows(a);
   const uint64_t total = (uint64_t)blocksPerBatch * a.batch;
   if (total >= (1ull << 32)) return hipErrorInvalidValue;

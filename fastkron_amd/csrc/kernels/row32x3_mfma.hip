@@ -196,16 +196,17 @@ bool row32x3Supported(const StepArgs& a) {
 
 hipError_t launchRow32x3(const StepArgs& a, hipStream_t stream) {
   if (!row32x3Supported(a)) return hipErrorInvalidValue;
-  static bool attrSet = false;
+  static PerDeviceOnce attrOnce;
+  const int devIdx = launchDeviceIndex();
   const size_t ldsBytes = kR32LdsWords * sizeof(float);
-  if (!attrSet) {
+  if (!attrOnce.done(devIdx)) {
     hipError_t e = hipFuncSetAttribute((const void*)kron_row32x3_kernel<true>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes);
     if (e != hipSuccess) return e;
     e = hipFuncSetAttribute((const void*)kron_row32x3_kernel<false>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes);
     if (e != hipSuccess) return e;
-    attrSet = true;
+    attrOnce.mark(devIdx);
   }
   dim3 grid(a.M, a.batch), block(512);
   if (a.y && a.epilogue)

@@ -230,16 +230,17 @@ bool row8x5Supported(const StepArgs& a) {
 
 hipError_t launchRow8x5(const StepArgs& a, hipStream_t stream) {
   if (!row8x5Supported(a)) return hipErrorInvalidValue;
-  static bool attrSet = false;
+  static PerDeviceOnce attrOnce;
+  const int devIdx = launchDeviceIndex();
   const size_t ldsBytes = kRow8LdsWords * sizeof(float);
-  if (!attrSet) {
+  if (!attrOnce.done(devIdx)) {
     hipError_t e = hipFuncSetAttribute((const void*)kron_row8x5_kernel<true>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes);
     if (e != hipSuccess) return e;
     e = hipFuncSetAttribute((const void*)kron_row8x5_kernel<false>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes);
     if (e != hipSuccess) return e;
-    attrSet = true;
+    attrOnce.mark(devIdx);
   }
   dim3 grid(a.M / row8Rows(a), a.batch), block(512);
   if (a.y && a.epilogue)

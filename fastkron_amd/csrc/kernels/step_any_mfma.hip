@@ -265,34 +265,31 @@ static hipError_t launchStepAnyT(const StepArgs& a, const StepAnyGeom& g, hipStr
   // the tile of the next iteration is held in registers too unless the two copies would not fit (fp64, P > 128)
   constexpr bool PF = PCMAX * sizeof(T) <= 256;
   const size_t ldsBytes = (size_t)4 * g.kStride * sizeof(T);
-  static bool attrSet = false;
-  if (!attrSet) {
+  static PerDeviceOnce attrOnce;
+  const int devIdx = launchDeviceIndex();
+  if (!attrOnce.done(devIdx)) {
     hipError_t e = hipFuncSetAttribute((const void*)kron_step_any_kernel<T, PCMAX, true, PF>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, 140 * 1024);
     if (e != hipSuccess) return e;
     e = hipFuncSetAttribute((const void*)kron_step_any_kernel<T, PCMAX, false, PF>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, 140 * 1024);
     if (e != hipSuccess) return e;
-    attrSet = true;
+    attrOnce.mark(devIdx);
   }
-  static int cus = 0;
-  if (!cus) {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    cus = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
-              ? prop.multiProcessorCount : 256;
-  }
+  const int cus = deviceCUs();
   // persistent workgroups, as many per CU as registers and the factor's LDS copy allow: a wave has one tile in
   // flight, so the bytes in flight per CU (what hides the HBM latency) grow with the number of resident waves
-  static size_t occLds = ~(size_t)0;
-  static int occ = 1;
-  if (occLds != ldsBytes) {
+  // (the last answer is kept per device, the LDS size and the count packed into one word)
+  static std::atomic<uint64_t> occCache[kMaxDevices];
+  const uint64_t cached = occCache[devIdx].load(std::memory_order_relaxed);
+  int occ = (int)(cached & 15);
+  if (occ == 0 || (cached >> 4) != ldsBytes) {
     int n = 0;
     const void* fn = (a.y && a.epilogue) ? (const void*)kron_step_any_kernel<T, PCMAX, true, PF>
                                          : (const void*)kron_step_any_kernel<T, PCMAX, false, PF>;
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, fn, 256, ldsBytes) != hipSuccess || n < 1) n = 1;
     occ = n > 8 ? 8 : n;
-    occLds = ldsBytes;
+    occCache[devIdx].store(((uint64_t)ldsBytes << 4) | (uint64_t)occ, std::memory_order_relaxed);
   }
   uint32_t wgs = (uint32_t)cus * (uint32_t)occ;
   const uint32_t share = a.batch * g.nSlabs;                  // the other two grid dimensions

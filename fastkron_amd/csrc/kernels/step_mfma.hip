@@ -202,13 +202,7 @@ static hipError_t launchStepMfmaT(const StepArgs& a, hipStream_t stream) {
   const bool kmm = stepMfmaIsKmm(a);
   const uint32_t tilesPerRow = kmm ? (a.M + 15) / 16 : (uint32_t)((S + 15) / 16);
   const uint32_t totalTiles = kmm ? (uint32_t)(tilesPerRow * S) : tilesPerRow * a.M;
-  static int cus = 0;
-  if (!cus) {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    cus = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
-              ? prop.multiProcessorCount : 256;
-  }
+  const int cus = deviceCUs();
   // persistent workgroups: 2 per CU (8 waves, 2 per SIMD at up to 256 VGPRs), fewer when there is not enough work
   uint32_t wgs = (uint32_t)cus * 2;
   if (a.batch > 1) wgs = (wgs + a.batch - 1) / a.batch;         // the batch index is the second grid dimension

@@ -26,6 +26,20 @@ size_t fastKronGetLastPlan(fastKronHandle handle, char* buf, size_t bufLen);
  */
 fastKronError fastKronSetTunedDB(fastKronHandle handle, const char* path);
 
+/*
+ * Plan-only mode (on != 0): GeMKM/GeKMM calls on `handle` run every argument check, the launch planner and each
+ * chosen kernel's check of the concrete buffers (alignment, strides), but launch nothing and touch no device;
+ * an MI355X is assumed when none has been initialised.  fastKronGetLastPlan then names the kernels and
+ * fastKronGetLastLaunches lists the launches the call would have made, one text line per launch:
+ *   "kernel=<name> lo=<lo> hi=<hi> M=<rows> batch=<n> Kin=<cols> Kout=<cols> in=<ptr> out=<ptr> y=<ptr>
+ *    in_batch=<elems> out_batch=<elems> y_batch=<elems> f_batch=<elems>,<elems>,..."
+ * Meant for host-side tests of the planner and for inspecting what a call will do.  The reference has no such
+ * mode; its nearest counterpart is the kernel series printed under FASTKRON_LOG=INFO
+ * (reference src/kernel_db/kernel_db.cpp:282-285).
+ */
+fastKronError fastKronSetPlanOnly(fastKronHandle handle, int on);
+size_t fastKronGetLastLaunches(fastKronHandle handle, char* buf, size_t bufLen);
+
 #ifdef __cplusplus
 }
 #endif

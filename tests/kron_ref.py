@@ -41,6 +41,18 @@ def mkm_intermediate_dense(X, Fs, j):
     return R.reshape(M, kpre, lsuf).swapaxes(1, 2).reshape(M, kpre * lsuf)
 
 
+def kmm_intermediate_dense(X, Fs, j):
+    """KMM counterpart: X (K, M), Fs[i] (Q_i, P_i); rows of the result ordered (q_j .. q_{N-1}, k_0 .. k_{j-1}).
+    Identities stand in for the factors not yet applied; the row blocks are then swapped explicitly."""
+    X = np.asarray(X, np.float64)
+    M = X.shape[1]
+    mats = [np.eye(f.shape[1]) for f in Fs[:j]] + [np.asarray(f, np.float64) for f in Fs[j:]]
+    R = kron_chain(mats) @ X
+    kpre = int(np.prod([f.shape[1] for f in Fs[:j]])) if j > 0 else 1
+    lsuf = int(np.prod([f.shape[0] for f in Fs[j:]]))
+    return R.reshape(kpre, lsuf, M).swapaxes(0, 1).reshape(kpre * lsuf, M)
+
+
 def normwise(a, b):
     a = np.asarray(a, np.float64).reshape(-1)
     b = np.asarray(b, np.float64).reshape(-1)

@@ -4,7 +4,7 @@ import numpy as np
 import pytest
 
 from oracle import kron_oracle as ko
-from tests.kron_ref import (kmm_dense, mkm_dense, mkm_intermediate_dense, normwise)
+from tests.kron_ref import (kmm_dense, kmm_intermediate_dense, mkm_dense, mkm_intermediate_dense, normwise)
 
 SHAPES = [
     # (M, Ps, Qs)
@@ -148,6 +148,53 @@ def test_strided_batches_and_broadcast():
                             batch=B, strideF=[0, 0], strideY=0).reshape(B, M, L)
     for b in range(B):
         assert normwise(Zs[b], mkm_dense(X[b], [f[0] for f in Fs], 1.0, 2.0, Y[0])) < 1e-14
+
+
+def test_kmm_strided_batches_and_broadcast():
+    """GeKMM batches: X is K x M per entry, factors Q x P, every entry against numpy.kron of its own factors."""
+    rng = np.random.default_rng(17)
+    M, Ps, Qs, B = 5, [4, 2, 3], [2, 3, 2], 3
+    K, L = 24, 12
+    X = rand(rng, (B, K, M), np.float64)
+    Fs = [rand(rng, (B, q, p), np.float64) for p, q in zip(Ps, Qs)]
+    Y = rand(rng, (B, L, M), np.float64)
+    Z = ko.sliced_multiply(ko.KMM, M, Ps, Qs, X, Fs, alpha=1.5, beta=0.5, Y=Y, batch=B).reshape(B, L, M)
+    for b in range(B):
+        assert normwise(Z[b], kmm_dense(X[b], [f[b] for f in Fs], 1.5, 0.5, Y[b])) < 1e-14
+    # shared factors, shared Y, and X shared against per-entry factors
+    Zs = ko.sliced_multiply(ko.KMM, M, Ps, Qs, X, [f[0] for f in Fs], alpha=1.0, beta=2.0, Y=Y[0], batch=B,
+                            strideF=[0, 0, 0], strideY=0).reshape(B, L, M)
+    for b in range(B):
+        assert normwise(Zs[b], kmm_dense(X[b], [f[0] for f in Fs], 1.0, 2.0, Y[0])) < 1e-14
+    Zx = ko.sliced_multiply(ko.KMM, M, Ps, Qs, X[0], Fs, batch=B, strideX=0).reshape(B, L, M)
+    for b in range(B):
+        assert normwise(Zx[b], kmm_dense(X[0], [f[b] for f in Fs])) < 1e-14
+    # opX = T: the buffer of an entry is M x K
+    Xt = np.ascontiguousarray(X.transpose(0, 2, 1))
+    Zt = ko.sliced_multiply(ko.KMM, M, Ps, Qs, Xt, Fs, batch=B, opX=ko.OP_T).reshape(B, L, M)
+    for b in range(B):
+        assert normwise(Zt[b], kmm_dense(X[b], [f[b] for f in Fs])) < 1e-14
+
+
+def test_kmm_forward_intermediates_layout():
+    rng = np.random.default_rng(18)
+    M, Ps, Qs = 3, [3, 4, 2], [2, 3, 5]
+    X = rand(rng, (24, M), np.float64)
+    Fs = [rand(rng, (q, p), np.float64) for p, q in zip(Ps, Qs)]
+    Z, inter = ko.sliced_multiply(ko.KMM, M, Ps, Qs, X, Fs, keep_intermediates=True)
+    assert normwise(Z.reshape(-1, M), kmm_dense(X, Fs)) < 1e-14
+    for j in (1, 2):   # Intermediates[j-1] is the output of the step multiplying factor j
+        assert normwise(inter[j - 1].reshape(-1, M), kmm_intermediate_dense(X, Fs, j)) < 1e-14
+    # batched: every entry keeps its own intermediates, entry after entry
+    B = 2
+    Xb = rand(rng, (B, 24, M), np.float64)
+    Fb = [rand(rng, (B, q, p), np.float64) for p, q in zip(Ps, Qs)]
+    Zb, interb = ko.sliced_multiply(ko.KMM, M, Ps, Qs, Xb, Fb, batch=B, keep_intermediates=True)
+    for b in range(B):
+        fsb = [f[b] for f in Fb]
+        assert normwise(Zb.reshape(B, -1, M)[b], kmm_dense(Xb[b], fsb)) < 1e-14
+        for j in (1, 2):
+            assert normwise(interb[j - 1].reshape(B, -1, M)[b], kmm_intermediate_dense(Xb[b], fsb, j)) < 1e-14
 
 
 def test_forward_intermediates_layout():

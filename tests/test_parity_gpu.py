@@ -256,6 +256,49 @@ def test_misaligned_buffers_fall_back_to_the_generic_plan(fk):
     assert normwise(Z.cpu().numpy(), want) <= 1e-5
 
 
+@pytest.mark.parametrize("which", ["x", "y", "z"])
+@pytest.mark.parametrize("M,Ps,dt", [(96, [16] * 4, np.float32), (16, [16] * 3, np.float32), (100, [32] * 3, np.float32),
+                                     (8, [64, 64], np.float64), (8, [32, 32], np.float32), (64, [64], np.float64)])
+def test_one_misaligned_operand_at_a_time(fk, which, M, Ps, dt):
+    """X, Y or Z alone starts one element past a 256-byte boundary: kernels with 16-byte accesses to that operand
+    must not be chosen, and the answer must still be right."""
+    import torch
+    K = int(np.prod(Ps))
+    X, Fs, Y = make_case(ko.MKM, M, Ps, Ps, dt, seed=62, with_y=True)
+    want = oracle_answer(ko.MKM, M, Ps, Ps, X, Fs, Y, 1.5, 0.5)
+    dev = "cuda:0"
+    tdt = torch.float32 if dt == np.float32 else torch.float64
+
+    def place(host, shifted):
+        buf = torch.full((host.size + 64,), float("nan"), dtype=tdt, device=dev)
+        v = buf[1:1 + host.size] if shifted else buf[:host.size]
+        v.copy_(torch.from_numpy(host.reshape(-1)))
+        return v
+
+    tX, tY = place(X, which == "x"), place(Y, which == "y")
+    Z = place(np.full(M * K, np.nan, dt), which == "z")
+    tFs = [torch.from_numpy(f).to(dev) for f in Fs]
+    t1 = torch.empty(M * K, dtype=tdt, device=dev)
+    t2 = torch.empty(M * K, dtype=tdt, device=dev)
+    e = fk.xgemkm(M, Ps, Ps, tX, tFs, Z, 1.5, 0.5, tY, t1, t2)
+    torch.cuda.synchronize()
+    assert e == 0
+    assert normwise(Z.cpu().numpy(), want) <= TOL[dt], (which, fk.last_plan())
+
+
+@pytest.mark.parametrize("M,Ps,dt", [(8, [16] * 5, np.float32), (4, [8] * 6, np.float32), (2, [32] * 4, np.float32),
+                                     (8, [16] * 4, np.float64), (2, [64] * 3, np.float64), (16, [4] * 8, np.float32),
+                                     (4, [8] * 5, np.float64), (3, [4, 4] + [8] * 5, np.float32)])
+def test_strided_entry_point_with_a_single_batch_entry(fk, M, Ps, dt):
+    """batchCount = 1 with the natural strides (strideF = P*Q): the two-part plan turns rows into batch entries of
+    its second part, which must not inherit the caller's factor strides."""
+    check(fk, ko.MKM, M, Ps, Ps, dt, alpha=1.5, beta=0.5, seed=105, batch=1, strided=True)
+    strided_plan = fk.last_plan()
+    check(fk, ko.MKM, M, Ps, Ps, dt, alpha=1.5, beta=0.5, seed=105)
+    assert [k for _, _, k in fk.last_plan()] == [k for _, _, k in strided_plan]
+    check(fk, ko.KMM, M, Ps, Ps, dt, alpha=1.5, beta=0.5, seed=106, batch=1, strided=True)
+
+
 @pytest.mark.parametrize("mm,name", [(ko.MKM, "mkm"), (ko.KMM, "kmm")])
 def test_forward_strided_batched(fk, mm, name):
     import ctypes

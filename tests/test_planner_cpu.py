@@ -1,0 +1,207 @@
+"""Host-side tests of the launch planner through the C ABI in plan-only mode (include/fastkron_ext.h): every
+argument check, the planner and each kernel's check of the concrete buffers run, nothing is launched, no GPU is
+needed.  Covered here: which kernels a problem gets, what the launches are handed (strides, batch counts), and the
+fallback to plainer kernels when a buffer does not have the alignment a kernel's vector accesses need
+(the reference's counterpart is the optimisation level of a kernel, reference src/kernels/kernel_opt.h:42-84,
+checked per problem in KMMKernel::canCompute, src/kernels/kmmkernel.cpp:85-126)."""
+import ctypes
+
+import pytest
+
+from fastkron_amd import capi
+
+BASE = 0x7000_0000_0000          # fake device addresses, 4 GiB apart; never dereferenced in plan-only mode
+GAP = 1 << 32
+
+
+@pytest.fixture
+def planner():
+    lib = capi.load()
+    h = ctypes.c_void_p()
+    assert lib.fastKronInit(ctypes.byref(h), capi.BACKEND_HIP) == capi.SUCCESS
+    assert lib.fastKronSetPlanOnly(h, 1) == capi.SUCCESS
+    yield lib, h
+    lib.fastKronDestroy(h)
+
+
+def plan(planner, mm, dt, M, Ps, Qs, batch=None, alpha=1.0, beta=0.0, with_y=False, offs=None, strides=None,
+         strideF=None, opX=capi.OP_N, opF=capi.OP_N, temp2=True, y_is_z=False):
+    """Runs one call in plan-only mode.  `offs` shifts the fake base pointers of x / z / y / t1 / t2 by bytes,
+    `strides` overrides the element strides of x / z / y.  Returns (error, kernel names, launch records)."""
+    lib, h = planner
+    offs = offs or {}
+    K, L = 1, 1
+    for p, q in zip(Ps, Qs):
+        K, L = K * p, L * q
+    ptr = {n: BASE + i * GAP + offs.get(n, 0) for i, n in enumerate(["x", "z", "y", "t1", "t2"])}
+    if y_is_z:
+        ptr["y"] = ptr["z"]
+    fs = capi.arr_ptr([BASE + (8 + i) * GAP + offs.get("f", 0) for i in range(len(Ps))])
+    sc = ctypes.c_float if dt == "s" else ctypes.c_double
+    X, Z = ctypes.c_void_p(ptr["x"]), ctypes.c_void_p(ptr["z"])
+    Y = ctypes.c_void_p(ptr["y"]) if (with_y or y_is_z) else None
+    t1, t2 = ctypes.c_void_p(ptr["t1"]), (ctypes.c_void_p(ptr["t2"]) if temp2 else None)
+    PsA, QsA = capi.arr_u32(Ps), capi.arr_u32(Qs)
+    if batch is None:
+        if mm == "mkm":
+            e = getattr(lib, dt + "gemkm")(h, capi.BACKEND_HIP, M, len(Ps), PsA, QsA, X, opX, fs, opF, Z, sc(alpha), sc(beta),
+                                           Y, t1, t2)
+        else:
+            e = getattr(lib, dt + "gekmm")(h, capi.BACKEND_HIP, len(Ps), QsA, PsA, M, fs, opF, X, opX, Z, sc(alpha), sc(beta),
+                                           Y, t1, t2)
+    else:
+        st = {"x": M * K, "z": M * L, "y": M * L}
+        st.update(strides or {})
+        sF = capi.arr_u64(strideF if strideF is not None else [p * q for p, q in zip(Ps, Qs)])
+        if mm == "mkm":
+            e = getattr(lib, dt + "gemkmStridedBatched")(h, capi.BACKEND_HIP, M, len(Ps), PsA, QsA, X, opX, st["x"], fs, opF,
+                                                         sF, Z, st["z"], sc(alpha), sc(beta), batch, Y, st["y"], t1, t2)
+        else:
+            e = getattr(lib, dt + "gekmmStridedBatched")(h, capi.BACKEND_HIP, len(Ps), QsA, PsA, M, fs, opF, sF, X, opX,
+                                                         st["x"], Z, st["z"], sc(alpha), sc(beta), batch, Y, st["y"], t1, t2)
+    buf = ctypes.create_string_buffer(1 << 16)
+    lib.fastKronGetLastPlan(h, buf, len(buf))
+    names = [s.split(":")[1] for s in buf.value.decode().split(";")[1:]]
+    lib.fastKronGetLastLaunches(h, buf, len(buf))
+    launches = []
+    for line in buf.value.decode().splitlines():
+        rec = dict(kv.split("=", 1) for kv in line.split())
+        rec["f_batch"] = [int(v) for v in rec["f_batch"].split(",")]
+        launches.append(rec)
+    return e, names, launches
+
+
+# ---- a strided-batched call with one batch entry must not carry its strides into any launch ----
+@pytest.mark.parametrize("dt,M,P,N", [("s", 8, 16, 5), ("s", 4, 8, 6), ("s", 2, 32, 4), ("d", 8, 16, 4), ("d", 2, 64, 3),
+                                      ("s", 16, 4, 8), ("d", 4, 8, 5), ("s", 4, 12, 4)])
+def test_single_entry_batches_carry_no_strides(planner, dt, M, P, N):
+    e, names, launches = plan(planner, "mkm", dt, M, [P] * N, [P] * N, batch=1)
+    assert e == capi.SUCCESS
+    assert len(launches) >= 1
+    for rec in launches:
+        assert rec["f_batch"] == [0] * len(rec["f_batch"]), (names, rec)
+    # ... and it gets the plan of the plain entry point
+    e2, names2, launches2 = plan(planner, "mkm", dt, M, [P] * N, [P] * N)
+    assert e2 == capi.SUCCESS and names2 == names
+    assert [r["batch"] for r in launches2] == [r["batch"] for r in launches]
+
+
+def test_two_part_plan_reads_leading_factors_with_stride_zero(planner):
+    """M rows become batch entries of the leading part: per-entry factor strides there would walk off F."""
+    e, names, launches = plan(planner, "mkm", "s", 8, [16] * 5, [16] * 5, batch=1)
+    assert e == capi.SUCCESS and len(launches) == 2
+    assert "_16x16_16x16_4_1x65536" in launches[0]["kernel"] and int(launches[0]["M"]) == 8 * 16
+    assert int(launches[1]["batch"]) == 8 and launches[1]["f_batch"] == [0]
+    # per-batch leading factors rule the two-part plan out altogether
+    e, names, launches = plan(planner, "mkm", "s", 8, [16] * 5, [16] * 5, batch=2)
+    assert e == capi.SUCCESS
+    assert all(int(r["batch"]) == 2 for r in launches), launches
+    # shared factors (stride 0) with several batch entries keep it
+    e, names, launches = plan(planner, "mkm", "s", 8, [16] * 5, [16] * 5, batch=2, strideF=[0] * 5)
+    assert e == capi.SUCCESS and int(launches[-1]["batch"]) == 16 and launches[-1]["f_batch"] == [0]
+
+
+# ---- kernels with 16-byte global accesses are only chosen for buffers that allow them ----
+VECTOR_CASES = [
+    # (label, mm, dt, M, Ps, Qs, batch, beta, substring of the kernel expected on aligned buffers)
+    ("row16x4", "mkm", "s", 128, [16] * 4, [16] * 4, None, 0.5, "_16x16_16x16_4_1x65536"),
+    ("row16x3", "mkm", "s", 64, [16] * 3, [16] * 3, None, 0.5, "_16x16_16x16_3_1x4096"),
+    ("row16x3d", "mkm", "d", 64, [16] * 3, [16] * 3, None, 0.5, "_d_16x16_16x16_3_1x4096"),
+    ("row32x3", "mkm", "s", 128, [32] * 3, [32] * 3, None, 0.5, "_32x32_32x32_3_1x32768"),
+    ("pair32", "mkm", "s", 64, [32] * 2, [32] * 2, None, 0.5, "_32x32_32x32_2_1x1024"),
+    ("pair64d", "mkm", "d", 64, [64] * 2, [64] * 2, None, 0.5, "_d_64x64_64x64_2_1x4096"),
+    ("step64", "mkm", "s", 64, [64], [64], None, 0.5, "_64x64_64x64_1_"),
+    ("kmm64d", "kmm", "d", 64, [64], [64], None, 0.5, "kmm_hip_gfx950_256_d_64x64_64x64_1_64x64"),
+    ("row8x5", "mkm", "s", 64, [8] * 5, [8] * 5, None, 0.5, "_8x8_8x8_5_1x32768"),
+    ("row32x16", "mkm", "s", 64, [32] * 3, [16] * 3, None, 0.5, "_32x16_32x16_3_1x32768"),
+    ("kmm4x6", "kmm", "s", 64, [4] * 6, [4] * 6, None, 0.5, "_4x4_4x4_6_8x4096"),
+]
+
+
+@pytest.mark.parametrize("case", VECTOR_CASES, ids=[c[0] for c in VECTOR_CASES])
+def test_aligned_buffers_get_the_specialised_kernel(planner, case):
+    _, mm, dt, M, Ps, Qs, batch, beta, want = case
+    e, names, _ = plan(planner, mm, dt, M, Ps, Qs, batch=batch, beta=beta, with_y=True)
+    assert e == capi.SUCCESS
+    assert any(want in n for n in names), names
+
+
+@pytest.mark.parametrize("which", ["x", "z", "y"])
+@pytest.mark.parametrize("case", VECTOR_CASES, ids=[c[0] for c in VECTOR_CASES])
+def test_a_buffer_off_by_one_element_still_gets_a_plan_that_accepts_it(planner, case, which):
+    """The base pointer of X, Z or Y is moved by one element: whatever plan comes back passed every kernel's own
+    check of these buffers (plan-only mode runs them), and the call does not fail."""
+    _, mm, dt, M, Ps, Qs, batch, beta, want = case
+    esize = 4 if dt == "s" else 8
+    e, names, launches = plan(planner, mm, dt, M, Ps, Qs, batch=batch, beta=beta, with_y=True, offs={which: esize})
+    assert e == capi.SUCCESS and len(launches) >= 1, names
+
+
+VECTOR_KERNELS_NEEDING = {
+    # kernels whose 16-byte accesses make them refuse a misaligned operand: label -> operands they vector-access
+    "row16x4": "xzy", "row16x3": "x", "row16x3d": "x", "row32x3": "xzy", "pair32": "x", "pair64d": "xzy", "step64": "x",
+    "kmm64d": "xzy",
+}
+
+
+@pytest.mark.parametrize("label,which", [(k, w) for k, ws in VECTOR_KERNELS_NEEDING.items() for w in ws])
+def test_misaligned_operand_rules_the_vector_kernel_out(planner, label, which):
+    case = [c for c in VECTOR_CASES if c[0] == label][0]
+    _, mm, dt, M, Ps, Qs, batch, beta, want = case
+    esize = 4 if dt == "s" else 8
+    e, names, _ = plan(planner, mm, dt, M, Ps, Qs, batch=batch, beta=beta, with_y=True, offs={which: esize})
+    assert e == capi.SUCCESS
+    assert not any(want in n for n in names), (which, names)
+
+
+@pytest.mark.parametrize("label", ["row16x4", "row32x3", "pair64d", "row16x3"])
+@pytest.mark.parametrize("which", ["x", "z", "y"])
+def test_odd_batch_strides_rule_the_vector_kernel_out(planner, label, which):
+    """Batch entries one element further apart than the operand is long: entry 1 is misaligned although entry 0 is not."""
+    case = [c for c in VECTOR_CASES if c[0] == label][0]
+    _, mm, dt, M, Ps, Qs, _, beta, want = case
+    K, L = 1, 1
+    for p, q in zip(Ps, Qs):
+        K, L = K * p, L * q
+    odd = {"x": M * K + 1, "z": M * L + 1, "y": M * L + 1}[which]
+    e, names, launches = plan(planner, mm, dt, M, Ps, Qs, batch=3, beta=beta, with_y=True, strides={which: odd},
+                              strideF=[0] * len(Ps))
+    assert e == capi.SUCCESS
+    needs = VECTOR_KERNELS_NEEDING[label]
+    if which in needs:
+        assert not any(want in n for n in names), (which, names)
+
+
+def test_batches_beyond_one_grid_dimension_are_checked_chunk_by_chunk(planner):
+    e, names, launches = plan(planner, "mkm", "s", 1, [16, 16], [16, 16], batch=70000, strideF=[0, 0])
+    assert e == capi.SUCCESS
+    assert [int(r["batch"]) for r in launches] == [65535, 70000 - 65535] * (len(launches) // 2)
+    first, second = launches[0], launches[1]
+    assert int(second["in"], 16) - int(first["in"], 16) == 65535 * 256 * 4
+
+
+# ---- tuned-plan files are not trusted ----
+def test_tuned_plans_that_do_not_fit_the_problem_are_ignored(planner, tmp_path):
+    lib, h = planner
+    e, online, _ = plan(planner, "mkm", "s", 8, [8, 8, 8], [8, 8, 8])
+    generic = "gekmm_hip_gfx950_256_f_generic_1"
+    key = "8x512*(8x8^3)_NN_f"
+    bad = [
+        f"{key} 0.01 1 0 5 {generic}",                       # factor index beyond the chain
+        f"{key} 0.01 2 2 2 {generic} 0 0 {generic}",         # factor 1 never applied
+        f"{key} 0.01 3 0 0 {generic} 1 1 {generic} 2 2 {generic}",   # first factor first
+        f"{key} 0.01 1 0 2 {generic}",                       # a one-factor kernel given three factors
+        f"{key} 0.01 1 0 2 mkm_hip_gfx950_1024_f_16x16_16x16_4_1x65536_mfma16x16x4_NN_strided_0_3",   # wrong factor size
+    ]
+    for line in bad:
+        f = tmp_path / "tuned.db"
+        f.write_text(line + "\n")
+        assert lib.fastKronSetTunedDB(h, str(f).encode()) == capi.SUCCESS
+        e, names, _ = plan(planner, "mkm", "s", 8, [8, 8, 8], [8, 8, 8])
+        assert e == capi.SUCCESS and names == online, line
+    good = f"{key} 0.01 3 2 2 {generic} 1 1 {generic} 0 0 {generic}"
+    f = tmp_path / "tuned.db"
+    f.write_text(good + "\n")
+    lib.fastKronSetTunedDB(h, str(f).encode())
+    e, names, _ = plan(planner, "mkm", "s", 8, [8, 8, 8], [8, 8, 8])
+    assert e == capi.SUCCESS and names == [generic] * 3
