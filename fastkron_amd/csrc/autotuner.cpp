@@ -49,7 +49,9 @@ fastKronError Handle::tune(const KronProblem& p, Plan* best) {
     for (int lo = hi; lo >= 0 && hi - lo < (int)kMaxFused; lo--) {
       if (!useFusion() && lo != hi) break;
       const bool first = (hi == (int)N - 1), last = (lo == 0);
-      auto cands = db_.candidates(p, lo, hi, first, last, dev_);
+      DeviceInfo able = dev_;
+      able.rulesOfThumb = false;      // every kernel able to run the group is timed
+      auto cands = db_.candidates(p, lo, hi, first, last, able);
       for (int ki : cands) {
         const KernelInfo& k = db_.kernels()[ki];
         StepArgs a = makeStepArgs(p, lo, hi, first, last);

@@ -31,7 +31,7 @@ static hipError_t genericLaunch(const KernelInfo& k, const StepArgs& a, hipStrea
 
 // ---- several small factors of any shape fused through LDS ----
 static bool fusedSmallCanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
-                             const DeviceInfo&) {
+                             const DeviceInfo& dev) {
   const uint32_t nf = hi - lo + 1;
   if (k.dt != p.dt || nf < 2 || nf > kMaxFused || p.forward) return false;
   if (first && p.opX == 2) return false;                   // input and output in the same layout only
@@ -42,13 +42,13 @@ static bool fusedSmallCanRun(const KernelInfo& k, const KronProblem& p, uint32_t
     const bool mfma = sq && (p.P[i] == 16 || (p.dt == DType::F32 && p.mm == MMType::KMM && (p.P[i] == 4 || p.P[i] == 8)));
     if (!mfma) dedicated = false;
   }
-  if (dedicated) return false;
+  if (dedicated && dev.rulesOfThumb) return false;
   uint32_t ps[kMaxFused], qs[kMaxFused];
   for (uint32_t j = 0; j < nf; j++) { ps[j] = p.P[hi - j]; qs[j] = p.Q[hi - j]; }
   const bool kmm = p.mm == MMType::KMM && p.M > 1;
   // In the KMM layout the plain kernel already runs every factor at about 5 TB/s: fusing pays off only for
   // groups of three or more factors of at most 6 rows (measured against tuned plans).
-  if (kmm) {
+  if (kmm && dev.rulesOfThumb) {
     if (nf < 3) return false;
     for (uint32_t j = 0; j < nf; j++) if (ps[j] > 6) return false;
   }
@@ -61,7 +61,7 @@ static bool fusedSmallCheck(const KernelInfo& k, const StepArgs& a) { return fus
 
 // ---- one factor of any shape up to 256x512 on the matrix cores (zero padded) ----
 static bool stepAnyCanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, uint32_t hi, bool, bool,
-                          const DeviceInfo&) {
+                          const DeviceInfo& dev) {
   if (k.dt != p.dt || lo != hi) return false;
   const uint32_t P = p.P[lo], Q = p.Q[lo];
   if (P > 256 || Q > 512) return false;
@@ -69,7 +69,7 @@ static bool stepAnyCanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo
   // (measured per layout and type: e.g. fp32 MKM 18x18, fp64 MKM 12x12, fp32 KMM 31x31, fp64 KMM 20x20).
   const bool kmm = p.mm == MMType::KMM && p.M > 1;
   const uint64_t minPQ = kmm ? (p.dt == DType::F32 ? 900 : 400) : (p.dt == DType::F32 ? 256 : 144);
-  return (uint64_t)P * Q >= minPQ && P >= 4;
+  return ((uint64_t)P * Q >= minPQ || !dev.rulesOfThumb) && P >= 4;
 }
 static hipError_t stepAnyLaunch(const KernelInfo& k, const StepArgs& a, hipStream_t s) {
   return launchStepAnyMfma(a, k.dt, s);
@@ -115,7 +115,7 @@ static bool row16CanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, 
   // blocks the kernels that spread a block over many CUs finish sooner (measured crossover between 64 and 128 blocks).
   // (Shorter chains have no such alternative when their factors differ per batch entry, and go to the wave-per-block
   // kernel anyway when they do not.)
-  if (nf == 4 && (uint64_t)p.M * p.batch < kRow16MinBlocks) return false;
+  if (dev.rulesOfThumb && nf == 4 && (uint64_t)p.M * p.batch < kRow16MinBlocks) return false;
   return dev.ldsPerBlock >= 131072 && k.dt == p.dt;
 }
 static hipError_t row16Launch(const KernelInfo& k, const StepArgs& a, hipStream_t s) {
@@ -174,14 +174,14 @@ static bool row32Check(const KernelInfo&, const StepArgs& a) { return row32x16x3
 // ---- whole-row kernel for three fused 32x32 fp32 factors ----
 constexpr uint64_t kRow32MinRows = 96;
 static bool row32x3CanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
-                          const DeviceInfo&) {
+                          const DeviceInfo& dev) {
   if (p.dt != DType::F32 || p.mm != MMType::MKM || hi - lo + 1 != 3 || p.forward) return false;
   for (uint32_t i = lo; i <= hi; i++) if (p.P[i] != 32 || p.Q[i] != 32) return false;
   if (p.colsBefore(hi) != 32768) return false;
   if (first && p.opX == 2) return false;
   // a row is one workgroup's work for about 17 us: with few rows the pair kernel (a wave per 1024-column block) plus
   // one step across the blocks finishes sooner (measured crossover between 64 and 128 rows)
-  if ((uint64_t)p.M * p.batch < kRow32MinRows) return false;
+  if (dev.rulesOfThumb && (uint64_t)p.M * p.batch < kRow32MinRows) return false;
   return k.dt == p.dt;
 }
 static hipError_t row32x3Launch(const KernelInfo&, const StepArgs& a, hipStream_t s) { return launchRow32x3(a, s); }
@@ -245,7 +245,7 @@ static bool kmm4x6CanRun(const KernelInfo&, const KronProblem& p, uint32_t lo, u
   // Only while all column tiles are resident at once (one per CU): the tiles of an XCD then walk the rows of X
   // together and their 32-byte pieces meet in its L2.  With more tiles than CUs that order is lost and the
   // two-launch plan, which reads 256 bytes per row and wave, is faster (measured from M = 4096 on).
-  if ((uint64_t)(p.M / 8) * p.batch > (uint64_t)dev.cus) return false;
+  if (dev.rulesOfThumb && (uint64_t)(p.M / 8) * p.batch > (uint64_t)dev.cus) return false;
   return dev.ldsPerBlock >= 8 * (64 * 65 + 4) * 4;
 }
 static hipError_t kmm4x6Launch(const KernelInfo&, const StepArgs& a, hipStream_t s) { return launchKmm4x6(a, s); }
@@ -430,7 +430,9 @@ bool KernelDB::validPlan(const KronProblem& p, const Plan& plan, const DeviceInf
     if (s.kernel < 0 || (size_t)s.kernel >= kernels_.size()) return false;
     if ((int64_t)s.hi != expectHi || s.lo > s.hi || s.hi - s.lo + 1 > kMaxFused) return false;
     const KernelInfo& k = kernels_[s.kernel];
-    if (!k.canRun(k, p, s.lo, s.hi, l == 0, s.lo == 0, dev)) return false;
+    DeviceInfo able = dev;
+    able.rulesOfThumb = false;
+    if (!k.canRun(k, p, s.lo, s.hi, l == 0, s.lo == 0, able)) return false;
     expectHi = (int64_t)s.lo - 1;
   }
   return expectHi == -1;

@@ -21,6 +21,10 @@ struct DeviceInfo {
   int  clockKHz = 2400000;
   char arch[64] = "gfx950";
   bool valid = false;
+  // Selection without timing: a kernel's canRun then also refuses where a measured rule of thumb says another plan
+  // is faster (few rows, small factors ...).  The tuner and the check of a tuned plan switch this off and ask only
+  // what a kernel is able to run.
+  bool rulesOfThumb = true;
 };
 
 struct KernelInfo;
