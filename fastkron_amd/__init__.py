@@ -113,6 +113,13 @@ class FastKron:
                   capi.arr_ptr([f.data_ptr() for f in Fs]), opFs, _ptr(Z), sc(alpha), sc(beta),
                   _ptr(Y), _ptr(temp1), _ptr(temp2))
 
+    def xgemkm_static_scratch(self, M, Ps, Qs, X, Fs, Z, alpha=1.0, beta=0.0, Y=None, opX=OP_N, opFs=OP_N,
+                              backend=BACKEND_HIP):
+        """sgemkm without temporaries: they come from the library's static device array; allocates nothing."""
+        return self.lib.sgemkmStaticScratch(self.h, backend, M, len(Ps), capi.arr_u32(Ps), capi.arr_u32(Qs), _ptr(X), opX,
+                                            capi.arr_ptr([f.data_ptr() for f in Fs]), opFs, _ptr(Z),
+                                            ctypes.c_float(alpha), ctypes.c_float(beta), _ptr(Y))
+
     def xgekmm(self, M, Ps, Qs, X, Fs, Z, alpha=1.0, beta=0.0, Y=None, temp1=None, temp2=None,
                opX=OP_N, opFs=OP_N, backend=BACKEND_HIP):
         pre, sc = self._prefix(X.dtype)

@@ -15,6 +15,7 @@ BACKEND_NONE, BACKEND_X86, BACKEND_ARM, BACKEND_CUDA, BACKEND_HIP = 1, 2, 4, 8, 
 OPT_NONE, OPT_USE_FUSION, OPT_TUNE = 1, 2, 4
 SUCCESS, BACKEND_NOT_AVAILABLE, INVALID_MEMORY_ACCESS, KERNEL_NOT_FOUND, INVALID_ARGUMENT, \
     INVALID_KMM_PROBLEM, OTHER_ERROR = range(7)
+STATIC_SCRATCH_TEMP_BYTES = 16 << 20        # FASTKRON_STATIC_SCRATCH_TEMP_BYTES of include/fastkron_ext.h
 
 EXPORTS = [
     "fastKronVersion", "fastKronCUDAArchs", "fastKronGetErrorString", "fastKronGetBackends",
@@ -27,7 +28,8 @@ EXPORTS = [
     "skmmForwardStridedBatched", "dkmmForwardStridedBatched",
 ]
 
-EXT_EXPORTS = ["fastKronGetLastPlan", "fastKronSetTunedDB", "fastKronSetPlanOnly", "fastKronGetLastLaunches"]     # include/fastkron_ext.h
+EXT_EXPORTS = ["fastKronGetLastPlan", "fastKronSetTunedDB", "fastKronSetPlanOnly", "fastKronGetLastLaunches",
+               "sgemkmStaticScratch"]     # include/fastkron_ext.h
 
 _lib = None
 
@@ -87,6 +89,9 @@ def load():
     lib.fastKronGetLastPlan.argtypes = [vp, ctypes.c_char_p, ctypes.c_size_t]
     lib.fastKronGetLastPlan.restype = ctypes.c_size_t
     lib.fastKronSetTunedDB.argtypes = [vp, ctypes.c_char_p]
+    lib.sgemkmStaticScratch.argtypes = [vp, cint, u32, u32, u32p, u32p, vp, cint, vpp, cint, vp, ctypes.c_float,
+                                        ctypes.c_float, vp]
+    lib.sgemkmStaticScratch.restype = cint
     lib.fastKronSetPlanOnly.argtypes = [vp, cint]
     lib.fastKronGetLastLaunches.argtypes = [vp, ctypes.c_char_p, ctypes.c_size_t]
     lib.fastKronGetLastLaunches.restype = ctypes.c_size_t

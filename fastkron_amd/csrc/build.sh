@@ -10,7 +10,7 @@ HIPCC="${HIPCC:-/opt/rocm/bin/hipcc}"
 # -packed-fp32-ops is switched off: hipcc must not form v_pk_*_f32 from scalar float code.
 FLAGS=(-O3 -std=c++17 -fPIC --offload-arch=gfx950 -Xclang -target-feature -Xclang -packed-fp32-ops
        -Wall -Wno-unused-function -Wno-unused-value -Wno-unused-result -Wno-unused-command-line-argument -I"$HERE/../../include" "$@")
-SRCS=("$HERE"/api.cpp "$HERE"/handle.cpp "$HERE"/kernel_db.cpp "$HERE"/autotuner.cpp "$HERE"/kernels/*.hip)
+SRCS=("$HERE"/api.cpp "$HERE"/handle.cpp "$HERE"/kernel_db.cpp "$HERE"/autotuner.cpp "$HERE"/static_scratch.hip "$HERE"/kernels/*.hip)
 pids=()
 objs=()
 for s in "${SRCS[@]}"; do

@@ -73,6 +73,8 @@ fastKronError Handle::initHIP(void* ptrToStream) {
   hipInit_ = true;
   fastKronError e = ensureDevice();
   if (e != fastKronSuccess) return e;
+  // the static scratch array of the calls that must not allocate: its address on this GPU is looked up here, once
+  { void* p = nullptr; (void)staticScratchForCurrentDevice(&p); }
   // workspace for merged factors (kMaxMergeGroups products of at most 64x64 doubles); allocated here so that
   // the gemkm / gekmm calls themselves never allocate
   if (!mergeWs_) {
@@ -144,7 +146,7 @@ fastKronError Handle::sizesForward(uint32_t M, uint32_t N, const uint32_t* Ps, c
   return fastKronSuccess;
 }
 
-fastKronError Handle::xgemm(KronProblem p, fastKronBackend backend, void* temp1, void* temp2) {
+fastKronError Handle::xgemm(KronProblem p, fastKronBackend backend, void* temp1, void* temp2, const CallWorkspace* ws) {
   // argument checks in the order of reference src/handle/handle.cpp:116-122
   if (!p.forward) {
     if (p.Z == nullptr || temp1 == nullptr || !hasBackend(backend)) return fastKronInvalidArgument;
@@ -174,7 +176,7 @@ fastKronError Handle::xgemm(KronProblem p, fastKronBackend backend, void* temp1,
 
   {
     KronProblem merged;
-    if (useFusion() && mergeSmallFactors(p, &merged)) p = merged;
+    if (useFusion() && mergeSmallFactors(p, &merged, ws)) p = merged;
   }
 
   Plan plan;
@@ -187,7 +189,7 @@ fastKronError Handle::xgemm(KronProblem p, fastKronBackend backend, void* temp1,
     e = trySplitLeadingTrailing(p, temp1, temp2);
     if (e != fastKronKernelNotFound) return e;
   }
-  if (!have && canTune() && !p.forward && !planOnly_) {
+  if (!have && canTune() && !p.forward && !planOnly_ && !ws) {
     e = tune(p, &plan);
     if (e != fastKronSuccess) return e;
     have = true;
@@ -224,8 +226,10 @@ fastKronError Handle::xgemm(KronProblem p, fastKronBackend backend, void* temp1,
 
 static bool isPow2(uint32_t v) { return v && !(v & (v - 1)); }
 
-bool Handle::mergeSmallFactors(const KronProblem& p, KronProblem* out) {
-  if (!mergeWs_ || p.forward || p.N < 2) return false;
+bool Handle::mergeSmallFactors(const KronProblem& p, KronProblem* out, const CallWorkspace* ws) {
+  void* const wsBase = ws ? ws->merge : mergeWs_;
+  const size_t wsBytes = ws ? ws->mergeBytes : mergeWsBytes_;
+  if (!wsBase || p.forward || p.N < 2) return false;
   // fp32 GeKMM already fuses small factors in registers; everything else gains from merging
   if (p.mm == MMType::KMM && p.dt == DType::F32) return false;
   if (p.batch > 1) for (uint32_t i = 0; i < p.N; i++) if (p.strideF[i] != 0) return false;
@@ -280,17 +284,17 @@ bool Handle::mergeSmallFactors(const KronProblem& p, KronProblem* out) {
       mg.sq[j] = pMajor ? 1 : (int64_t)p.P[fi];
     }
     const size_t bytes = (size_t)G.size * G.size * dtypeSize(p.dt);
-    if (wsOff + bytes > mergeWsBytes_) return false;
-    mg.dst = (char*)mergeWs_ + wsOff;
+    if (wsOff + bytes > wsBytes) return false;
+    mg.dst = (char*)wsBase + wsOff;
     mg.dsp = pMajor ? (int64_t)G.size : 1;
     mg.dsq = pMajor ? 1 : (int64_t)G.size;
     wsOff += (bytes + 255) & ~(size_t)255;
     q.P[g] = G.size; q.Q[g] = G.size; q.F[g] = mg.dst;
   }
   if (!planOnly_) {
-    if (mergeWsUsed_ && mergeWsStream_ != stream_) orderWorkspaceBehind(stream_);
+    if (!ws && mergeWsUsed_ && mergeWsStream_ != stream_) orderWorkspaceBehind(stream_);
     if (launchMergeFactors(ma, p.dt, stream_) != hipSuccess) return false;
-    mergeWsStream_ = stream_; mergeWsUsed_ = true;
+    if (!ws) { mergeWsStream_ = stream_; mergeWsUsed_ = true; }
   }
   *out = q;
   return true;

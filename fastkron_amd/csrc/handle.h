@@ -15,6 +15,9 @@ struct BufferPlan {          // where each launch reads and writes
   uint64_t in_batch, out_batch;
 };
 
+// Address of the library's static scratch array on the current GPU (static_scratch.hip).
+hipError_t staticScratchForCurrentDevice(void** out);
+
 StepArgs makeStepArgs(const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool last);
 
 class Handle {
@@ -36,7 +39,10 @@ class Handle {
                                     size_t* yElems, size_t* interElems);
 
   // Entry point of every gemkm/gekmm/forward call (reference src/handle/handle.cpp:114-286).
-  fastKronError xgemm(KronProblem p, fastKronBackend backend, void* temp1, void* temp2);
+  // With `ws` the call takes its merged-factor workspace from the caller instead of the handle's own, and neither
+  // tunes nor allocates anything on the device.
+  struct CallWorkspace { void* merge; size_t mergeBytes; };
+  fastKronError xgemm(KronProblem p, fastKronBackend backend, void* temp1, void* temp2, const CallWorkspace* ws = nullptr);
 
   // Runs `plan` on the stream; temps may be null when the plan has a single launch.
   fastKronError execute(const KronProblem& p, const Plan& plan, void* temp1, void* temp2, bool dryRun = false);
@@ -48,7 +54,7 @@ class Handle {
   // Chains of 2x2 / 4x4 (fp64: also 8x8) factors: adjacent factors are replaced by their Kronecker product
   // (16x16; 64x64 in fp64 when the chain holds 8x8 or 32x32 factors), computed into the handle's workspace by one small launch, so that the
   // kernels for those sizes apply.  Returns false when nothing is merged; on true `out` is the merged problem.
-  bool mergeSmallFactors(const KronProblem& p, KronProblem* out);
+  bool mergeSmallFactors(const KronProblem& p, KronProblem* out, const CallWorkspace* ws = nullptr);
 
   const std::string& lastPlan() const { return lastPlan_; }
   void setTunedDB(const char* path);

@@ -40,6 +40,22 @@ fastKronError fastKronSetTunedDB(fastKronHandle handle, const char* path);
 fastKronError fastKronSetPlanOnly(fastKronHandle handle, int on);
 size_t fastKronGetLastLaunches(fastKronHandle handle, char* buf, size_t bufLen);
 
+/*
+ * sgemkm for callers that cannot allocate device memory: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Same arguments and result as sgemkm
+ * (include/fastkron.h) without temp1 / temp2: the two temporaries and the workspace for merged factors are parts of
+ * one array that the library keeps in device memory on every GPU it is loaded on, for the life of the process
+ * (2 * FASTKRON_STATIC_SCRATCH_TEMP_BYTES + 512 KiB).  The call itself allocates and frees nothing and never tunes.
+ * A problem whose temporaries (gekmmSizes' tmpElems * 4 bytes) exceed FASTKRON_STATIC_SCRATCH_TEMP_BYTES is refused
+ * with fastKronInvalidArgument and a message on stderr.  All calls on one GPU share the array: calls that overlap
+ * on one GPU race, whatever their handles and streams.  fastKronInitHIP resolves the array's address on its GPU.
+ */
+#define FASTKRON_STATIC_SCRATCH_TEMP_BYTES (16u << 20)
+fastKronError sgemkmStaticScratch(fastKronHandle handle, fastKronBackend backend, uint32_t M, uint32_t N,
+                                  uint32_t Ps[], uint32_t Qs[], const float* X, fastKronOp opX,
+                                  const float* const Fs[], fastKronOp opFs, float* Z, float alpha, float beta,
+                                  const float* Y);
+
 #ifdef __cplusplus
 }
 #endif
