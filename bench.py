@@ -1,14 +1,15 @@
 #!/usr/bin/env python3
 """Benchmark of the Kronecker-matrix multiplication hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c1|c2|c3|c4|c5] [--tune] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c1|c2|c3|c4|c5] [--only] [--tune] [--no-cpu]
 
 One "step" is one call of the C-ABI entry point (sgemkm / dgemkm / sgekmm / sgemkmStridedBatched) on a
 synthetic problem whose operands are already resident in HBM.  The default workload is c2, the
 configuration the headline metric is quoted on: sgemkm, X 1024 x 65536, four 16x16 factors.
 Prints ONE JSON line: GFLOP/s with FastKron's FLOP count (2*M*sum_i Kin_i*Q_i), the roofline of the
-dominant kernel measured with HIP events on the library's stream, and a CPU baseline (the oracle's
-vectorised OpenMP port) timed on the host cores in the same run.
+dominant kernel measured with HIP events on the library's stream, a CPU baseline (the oracle's
+vectorised OpenMP port) timed on the host cores in the same run, and under "configs" the same GPU figures
+(ms, GFLOP/s, roofline fraction, launches, kernels) for the other four configurations, timed the same way.
 """
 import argparse
 import ctypes
@@ -102,39 +103,17 @@ def cpu_baseline(M, Ps, Qs, dt, alpha, beta, batch, budget_s):
                       f"({spent:.1f} s of CPU work)"}
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=50)
-    ap.add_argument("--ramp-seconds", type=float, default=0.25,
-                    help="untimed steps run for this long before the warm-up steps (the GPU raises its clocks over "
-                         "the first tens of milliseconds of load; steady-state throughput is what is reported)")
-    ap.add_argument("--config", default="c2", choices=sorted(CONFIGS))
-    ap.add_argument("--tune", action="store_true", help="time candidate launch plans first (excluded from timing)")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--cpu-seconds", type=float, default=10.0)
-    ap.add_argument("--sets", type=int, default=3, help="operand sets rotated between steps (keeps the 256 MB Infinity Cache cold)")
-    ap.add_argument("--calibrate-copy", action="store_true",
-                    help="also run 4 plain device copies of 256 MiB (a known-size kernel for scaling rocprof counters)")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print("bench.py: this build runs on ONE GPU only (no multi-GPU path exists); use --gpus 1", file=sys.stderr)
-        sys.exit(2)
-
+def measure(fk, name, steps, warmup, ramp_seconds, nsets, ev, stream, calibrate_copy=False):
+    """Times `steps` calls of configuration `name` (operands resident in HBM, `nsets` operand sets rotated) and
+    returns its figures: wall-clock and hipEvent time per step, GFLOP/s, and the roofline of its launches."""
     import torch
-    import fastkron_amd
     from fastkron_amd import capi
 
-    call, M, Ps, Qs, dts, alpha, beta, batch, bound = CONFIGS[args.config]
-    dt = np.float32 if dts == "f32" else np.float64
+    call, M, Ps, Qs, dts, alpha, beta, batch, bound = CONFIGS[name]
     tdt = torch.float32 if dts == "f32" else torch.float64
     esize = 4 if dts == "f32" else 8
     K, L = int(np.prod(Ps)), int(np.prod(Qs))
     dev = torch.device("cuda:0")
-    torch.cuda.set_device(dev)
-    stream = torch.cuda.current_stream()
-    fk = fastkron_amd.FastKron(stream=stream, tune=args.tune)
     ye, te = fk.sizes(M, Ps, Qs)
 
     gen = torch.Generator(device=dev)
@@ -144,7 +123,7 @@ def main():
         return torch.rand(n, generator=gen, device=dev, dtype=tdt) * 2 - 1
 
     sets = []
-    for _ in range(args.sets):
+    for _ in range(nsets):
         X = uniform(batch * M * K)
         Fs = [uniform(batch * p * q) for p, q in zip(Ps, Qs)]
         Y = uniform(batch * M * L) if beta != 0 else None
@@ -169,7 +148,7 @@ def main():
         if e != capi.SUCCESS:
             raise RuntimeError(f"{call} failed with fastKronError {e}")
 
-    if args.calibrate_copy:
+    if calibrate_copy:
         src = torch.empty(64 * 1024 * 1024, device=dev, dtype=torch.float32).normal_()
         dst = torch.empty_like(src)
         for _ in range(4):
@@ -177,73 +156,122 @@ def main():
         torch.cuda.synchronize()
 
     t_ramp = time.perf_counter()
-    while time.perf_counter() - t_ramp < args.ramp_seconds:
+    while time.perf_counter() - t_ramp < ramp_seconds:
         for i in range(20):
             step(i)
         torch.cuda.synchronize()
-    for i in range(max(args.warmup, 1)):
+    for i in range(max(warmup, 1)):
         step(i)
     torch.cuda.synchronize()
 
-    ev = HipEvents()
-    sp = ctypes.c_void_p(stream.cuda_stream)
     e0, e1 = ev.create(), ev.create()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    ev.record(e0, sp)
-    for i in range(args.steps):
+    ev.record(e0, stream)
+    for i in range(steps):
         step(i)
-    ev.record(e1, sp)
+    ev.record(e1, stream)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     gpu_ms = ev.elapsed_ms(e0, e1)
 
-    ms_per_step = wall * 1e3 / args.steps
     flop = flop_count(M, Ps, Qs, batch)
-    value = flop / (wall / args.steps) / 1e9
-
     # Roofline of the dominant kernel.  The unit of work is "one factor applied to one row"; the
     # algorithmic bytes of a unit are the call's compulsory bytes / (rows * factors), so the launches
-    # of one call add up to exactly the compulsory bytes.  Every launch of a call runs the same
-    # kernel family, hence: average launch duration = event time / launches, bytes per launch =
-    # compulsory bytes / launches.
+    # of one call add up to exactly the compulsory bytes.  Average launch duration = event time / launches,
+    # bytes (or FLOPs) per launch = the call's / launches.
     plan = fk.last_plan()
     launches = len(plan)
-    kernel_ms = gpu_ms / args.steps / launches
+    kernel_ms = gpu_ms / steps / launches
     cbytes = compulsory_bytes(M, Ps, Qs, batch, esize, beta)
-    traffic = None
-    tpath = os.path.join(ROOT, "profiles", "traffic.json")
-    if os.path.exists(tpath):
-        traffic = json.load(open(tpath)).get(args.config, {}).get("traffic_bytes_per_launch")
     if bound == "hbm":
         achieved = cbytes / launches / (kernel_ms * 1e-3) / 1e9
         roof = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic}
+                "frac": round(achieved / HBM_PEAK_GBS, 4)}
     else:
         achieved = flop / launches / (kernel_ms * 1e-3) / 1e12
         roof = {"bound": "mfma", "achieved": round(achieved, 2), "peak": FP64_PEAK_TFLOPS, "unit": "TFLOP/s",
-                "frac": round(achieved / FP64_PEAK_TFLOPS, 4), "traffic": traffic}
+                "frac": round(achieved / FP64_PEAK_TFLOPS, 4)}
+    # HBM bytes per launch as rocprofv3 --pmc measured them in separate runs of this command (FETCH_SIZE, then
+    # WRITE_SIZE, scaled by a device copy of known size): read from the committed summary, not measured in this run
+    tpath = os.path.join(ROOT, "profiles", "traffic.json")
+    traffic = None
+    if os.path.exists(tpath):
+        traffic = json.load(open(tpath)).get(name, {}).get("traffic_bytes_per_launch")
+    roof["traffic"] = traffic
+    roof["traffic_source"] = "profiles/traffic.json (rocprofv3 --pmc runs of this command, not this run)" if traffic else None
     # the other roof of the same run, for reference: the fraction of the matrix peak of the element type
     # and the fraction of the HBM peak that the compulsory bytes of the whole call correspond to
-    step_s = gpu_ms / args.steps * 1e-3
+    step_s = gpu_ms / steps * 1e-3
     roof["matrix_frac"] = round(flop / step_s / 1e12 / (FP32_PEAK_TFLOPS if dts == "f32" else FP64_PEAK_TFLOPS), 4)
     roof["compulsory_hbm_frac"] = round(cbytes / step_s / 1e9 / HBM_PEAK_GBS, 4)
     roof["kernel"] = sorted(set(k for _, _, k in plan))
     roof["launches_per_step"] = launches
     roof["kernel_ms"] = round(kernel_ms, 5)
+    workload = (f"{name}: {call} M={M} factors={len(Ps)}x({Ps[0]}x{Qs[0]}) K={K} L={L} alpha={alpha} beta={beta} "
+                f"batch={batch}, uniform[-1,1], seed 0xFA57C0DE")
+    del sets, calls, t1, t2
+    torch.cuda.empty_cache()
+    return {"workload": workload, "dtype": dts, "ms_per_step": wall * 1e3 / steps, "gpu_ms_per_step": gpu_ms / steps,
+            "gflops": flop / (wall / steps) / 1e9, "roofline": roof, "dims": (M, Ps, Qs, alpha, beta, batch)}
 
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=50)
+    ap.add_argument("--ramp-seconds", type=float, default=0.25,
+                    help="untimed steps run for this long before the warm-up steps (the GPU raises its clocks over "
+                         "the first tens of milliseconds of load; steady-state throughput is what is reported)")
+    ap.add_argument("--config", default="c2", choices=sorted(CONFIGS), help="the workload of the headline figures")
+    ap.add_argument("--only", action="store_true", help="time the --config workload alone (profiling runs)")
+    ap.add_argument("--tune", action="store_true", help="time candidate launch plans first (excluded from timing)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-seconds", type=float, default=10.0)
+    ap.add_argument("--sets", type=int, default=3, help="operand sets rotated between steps (keeps the 256 MB Infinity Cache cold)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run 4 plain device copies of 256 MiB (a known-size kernel for scaling rocprof counters)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU only (no multi-GPU path exists); use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import fastkron_amd
+
+    torch.cuda.set_device(torch.device("cuda:0"))
+    stream = torch.cuda.current_stream()
+    fk = fastkron_amd.FastKron(stream=stream, tune=args.tune)
+    ev = HipEvents()
+    sp = ctypes.c_void_p(stream.cuda_stream)
+
+    head = measure(fk, args.config, args.steps, args.warmup, args.ramp_seconds, args.sets, ev, sp, args.calibrate_copy)
     out = {
         "metric": "GeMKM/GeKMM GFLOP/s on 1 MI355X (FastKron FLOP count 2*M*sum Kin_i*Q_i)",
-        "value": round(value, 1), "unit": "GFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": dts, "data": "synthetic",
-        "config": {"workload": f"{args.config}: {call} M={M} factors={len(Ps)}x({Ps[0]}x{Qs[0]}) K={K} L={L} "
-                               f"alpha={alpha} beta={beta} batch={batch}, uniform[-1,1], seed 0xFA57C0DE",
-                   "operand_sets_rotated": args.sets, "tuned": bool(args.tune)},
-        "roofline": roof,
-        "gpu_ms_per_step_events": round(gpu_ms / args.steps, 5),
+        "value": round(head["gflops"], 1), "unit": "GFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(head["ms_per_step"], 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": head["dtype"], "data": "synthetic",
+        "config": {"workload": head["workload"], "operand_sets_rotated": args.sets, "tuned": bool(args.tune)},
+        "roofline": head["roofline"],
+        "gpu_ms_per_step_events": round(head["gpu_ms_per_step"], 5),
     }
+    # the other configurations, timed the same way in the same process (the CPU leg stays with the headline workload)
+    if not args.only:
+        others = {}
+        for name in sorted(CONFIGS):
+            if name == args.config:
+                continue
+            r = measure(fk, name, args.steps, args.warmup, args.ramp_seconds, args.sets, ev, sp)
+            rf = r["roofline"]
+            others[name] = {"workload": r["workload"], "dtype": r["dtype"], "ms": round(r["gpu_ms_per_step"], 5),
+                            "ms_wall": round(r["ms_per_step"], 5), "gflops": round(r["gflops"], 1),
+                            "roofline": {k: rf[k] for k in ("bound", "achieved", "peak", "unit", "frac")},
+                            "launches": rf["launches_per_step"], "kernel": rf["kernel"]}
+        out["configs"] = others
     if not args.no_cpu:
+        M, Ps, Qs, alpha, beta, batch = head["dims"]
+        dt = np.float32 if head["dtype"] == "f32" else np.float64
         out["cpu_baseline"] = cpu_baseline(M, Ps, Qs, dt, alpha, beta, batch, args.cpu_seconds)
     print(json.dumps(out))
 
