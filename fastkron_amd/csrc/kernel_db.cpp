@@ -246,7 +246,7 @@ static bool kmm4x6CanRun(const KernelInfo&, const KronProblem& p, uint32_t lo, u
   // together and their 32-byte pieces meet in its L2.  With more tiles than CUs that order is lost and the
   // two-launch plan, which reads 256 bytes per row and wave, is faster (measured from M = 4096 on).
   if (dev.rulesOfThumb && (uint64_t)(p.M / 8) * p.batch > (uint64_t)dev.cus) return false;
-  return dev.ldsPerBlock >= 8 * (64 * 65 + 4) * 4;
+  return dev.ldsPerBlock >= (8 * 64 * 65 + 32) * 4;
 }
 static hipError_t kmm4x6Launch(const KernelInfo&, const StepArgs& a, hipStream_t s) { return launchKmm4x6(a, s); }
 static bool kmm4x6Check(const KernelInfo&, const StepArgs& a) { return kmm4x6Supported(a); }
