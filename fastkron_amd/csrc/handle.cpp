@@ -20,6 +20,9 @@ static int logLevel() {
 }
 
 Handle::Handle(uint32_t backends) : backends_(backends) {
+  // the plans that ship with the library first, then the user's own file on top of them
+  const std::string shipped = KernelDB::shippedPath();
+  if (!shipped.empty()) db_.loadFile(shipped);
   dbPath_ = KernelDB::defaultPath();
   if (!dbPath_.empty()) db_.loadFile(dbPath_);
 }
@@ -174,6 +177,25 @@ fastKronError Handle::xgemm(KronProblem p, fastKronBackend backend, void* temp1,
   if (e != fastKronSuccess) return e;
   launchLog_.clear();
 
+  // 1. A tuned record under the call's own problem string says everything: whether small factors are merged,
+  //    whether the chain runs as a two-part plan, and which kernel runs which factors.  With tuning switched on a
+  //    problem without a record is tuned here, once.  A record that does not fit the call's buffers falls through
+  //    to the online selection.
+  if (!p.forward) {
+    Choice c;
+    bool have = lookupChoice(p, &c);
+    if (!have && canTune() && !planOnly_ && !ws) {
+      e = tune(p, temp2 != nullptr, &c);
+      if (e != fastKronSuccess && e != fastKronKernelNotFound) return e;
+      have = (e == fastKronSuccess);
+    }
+    if (have) {
+      e = runChoice(p, c, temp1, temp2, ws);
+      if (e != fastKronKernelNotFound) return e;
+    }
+  }
+
+  // 2. Online selection.
   {
     KronProblem merged;
     if (useFusion() && mergeSmallFactors(p, &merged, ws)) p = merged;
@@ -182,17 +204,15 @@ fastKronError Handle::xgemm(KronProblem p, fastKronBackend backend, void* temp1,
   Plan plan;
   const std::string key = p.str();
   bool have = false;
-  if (!p.forward) have = db_.lookupTuned(key, &plan) && db_.validPlan(p, plan, dev_);
+  // (records without the merge / split fields are keyed by the chain as the online rules rewrite it)
+  if (!p.forward) {
+    int merge = -1;
+    have = db_.lookupTuned(key, &plan, &merge) && merge < 0 && db_.validPlan(p, plan, dev_);
+  }
   // chains longer than one whole-block kernel: the two-part plan, when the problem and the buffers allow it
-  // (the tuner only searches single chains of launches, so it is asked after this)
   if (!have && useFusion()) {
     e = trySplitLeadingTrailing(p, temp1, temp2);
     if (e != fastKronKernelNotFound) return e;
-  }
-  if (!have && canTune() && !p.forward && !planOnly_ && !ws) {
-    e = tune(p, &plan);
-    if (e != fastKronSuccess) return e;
-    have = true;
   }
   if (!have) {
     const std::string ck = key + (p.forward ? "_fwd" : "") + (useFusion() ? "" : "_nofuse");
@@ -305,6 +325,74 @@ bool Handle::mergeSmallFactors(const KronProblem& p, KronProblem* out, const Cal
 // apply the leading factors A = F_0 x ... x F_{g-1} across the blocks: for every row that is a KMM problem
 // on a K_A x T matrix whose T columns are contiguous.  Two or three launches instead of N.  The layout
 // between the two parts is [row][k_A][q_B] (digits in place), which only these two sub-problems see.
+//
+// buildSplit sets up the two sub-problems for g leading factors (q1: trailing factors, X -> temp1; q2: leading
+// factors, temp1 -> Z with the call's epilogue) and returns false when the problem does not have that form.
+bool Handle::buildSplit(const KronProblem& p, uint32_t g, void* temp1, void* temp2, KronProblem* q1out,
+                        KronProblem* q2out) const {
+  if (p.mm != MMType::MKM || p.forward || p.opX != fastKronOp_N) return false;
+  if (!temp1 || !temp2 || p.N < 3 || g == 0 || g >= p.N) return false;
+  const uint32_t nT = p.N - g;
+  for (uint32_t i = 0; i < p.N; i++) if (p.P[i] != p.Q[i]) return false;            // square: K and L agree throughout
+  uint64_t KA = 1, T = 1;
+  for (uint32_t i = 0; i < g; i++) KA *= p.P[i];
+  for (uint32_t i = g; i < p.N; i++) T *= p.P[i];
+  const uint64_t K = KA * T;
+  if (T >= (1ull << 32)) return false;
+  if (p.batch > 1) {
+    if (p.strideX != (uint64_t)p.M * K || p.strideZ != (uint64_t)p.M * K) return false;
+    if (p.Y && p.beta != 0.0 && p.strideY != (uint64_t)p.M * K) return false;
+  }
+  // the leading factors are read by a problem whose batch entries are the rows of this one: shared factors only
+  for (uint32_t i = 0; i < g; i++) if (p.strideF[i] != 0) return false;
+  if ((uint64_t)p.M * p.batch > 65535 || (uint64_t)p.M * KA >= (1ull << 31)) return false;
+
+  // part 1: trailing factors, X -> temp1, no epilogue
+  KronProblem q1 = p;
+  q1.M = (uint32_t)(p.M * KA); q1.N = nT;
+  for (uint32_t i = 0; i < nT; i++) {
+    q1.P[i] = p.P[g + i]; q1.Q[i] = p.Q[g + i]; q1.F[i] = p.F[g + i]; q1.strideF[i] = p.strideF[g + i];
+  }
+  q1.Z = temp1; q1.strideZ = (uint64_t)p.M * K;
+  q1.Y = nullptr; q1.strideY = 0; q1.alpha = 1.0; q1.beta = 0.0;
+
+  // part 2: leading factors as a KMM over every row block; P x Q storage is the transpose of KMM's Q x P
+  KronProblem q2 = p;
+  q2.mm = MMType::KMM; q2.M = (uint32_t)T; q2.N = g;
+  q2.opF = (p.opF == fastKronOp_N) ? fastKronOp_T : fastKronOp_N;
+  q2.opX = fastKronOp_N;
+  q2.X = temp1; q2.strideX = K;
+  q2.strideZ = K; q2.strideY = K;
+  q2.batch = p.batch * p.M; q2.strided = true;
+  for (uint32_t i = 0; i < g; i++) q2.strideF[i] = 0;
+  *q1out = q1; *q2out = q2;
+  return true;
+}
+
+// Validates (on the concrete buffers) and runs a two-part plan: plan1 on q1, plan2 on q2 with temp2 as its scratch.
+fastKronError Handle::runSplit(const KronProblem& p, uint32_t g, const KronProblem& q1, const Plan& plan1,
+                               const KronProblem& q2, const Plan& plan2, void* temp2) {
+  if (plan1.size() != 1) return fastKronKernelNotFound;                    // q1 has no scratch of its own
+  // more than two leading launches ping-pong between temp2 and Z, which must then not be Y
+  if (plan2.size() > 2 && p.Y == p.Z && p.beta != 0.0) return fastKronKernelNotFound;
+  if (execute(q1, plan1, nullptr, nullptr, true) != fastKronSuccess) return fastKronKernelNotFound;
+  if (execute(q2, plan2, temp2, nullptr, true) != fastKronSuccess) return fastKronKernelNotFound;
+  lastPlan_ = p.str();
+  for (auto& s : plan1)
+    lastPlan_ += ";" + std::to_string(g + s.lo) + "-" + std::to_string(g + s.hi) + ":" + db_.kernels()[s.kernel].name;
+  for (auto& s : plan2)
+    lastPlan_ += ";" + std::to_string(s.lo) + "-" + std::to_string(s.hi) + ":" + db_.kernels()[s.kernel].name;
+  if (planOnly_) {
+    launchLog_.clear();
+    (void)execute(q1, plan1, nullptr, nullptr, true);
+    return execute(q2, plan2, temp2, nullptr, true);
+  }
+  fastKronError e = execute(q1, plan1, nullptr, nullptr);
+  if (e != fastKronSuccess) return e;
+  return execute(q2, plan2, temp2, nullptr);
+}
+
+// The online rule for the two-part plan: how many trailing factors one whole-block kernel takes.
 fastKronError Handle::trySplitLeadingTrailing(const KronProblem& p, void* temp1, void* temp2) {
   if (p.mm != MMType::MKM || p.forward || p.opX != fastKronOp_N) return fastKronKernelNotFound;
   if (!temp1 || !temp2 || p.N < 3) return fastKronKernelNotFound;
@@ -328,58 +416,52 @@ fastKronError Handle::trySplitLeadingTrailing(const KronProblem& p, void* temp1,
   while (nT < maxT && nT < p.N && p.P[p.N - 1 - nT] == tp && p.Q[p.N - 1 - nT] == tp) nT++;
   if (nT < 2 || nT == p.N) return fastKronKernelNotFound;         // a chain of nT factors alone is a whole-row problem
   const uint32_t g = p.N - nT;
-  for (uint32_t i = 0; i < g; i++) if (p.P[i] != p.Q[i]) return fastKronKernelNotFound;   // square: K and L agree
-  uint64_t KA = 1, T = 1;
-  for (uint32_t i = 0; i < g; i++) KA *= p.P[i];
-  for (uint32_t i = 0; i < nT; i++) T *= tp;
-  const uint64_t K = KA * T;
-  if (p.batch > 1) {
-    if (p.strideX != (uint64_t)p.M * K || p.strideZ != (uint64_t)p.M * K) return fastKronKernelNotFound;
-    if (p.Y && p.beta != 0.0 && p.strideY != (uint64_t)p.M * K) return fastKronKernelNotFound;
-  }
-  // the leading factors are read by a problem whose batch entries are the rows of this one: shared factors only
-  for (uint32_t i = 0; i < g; i++) if (p.strideF[i] != 0) return fastKronKernelNotFound;
-  if ((uint64_t)p.M * p.batch > 65535 || (uint64_t)p.M * KA >= (1ull << 31)) return fastKronKernelNotFound;
-
-  // part 1: trailing factors, X -> temp1, no epilogue
-  KronProblem q1 = p;
-  q1.M = (uint32_t)(p.M * KA); q1.N = nT;
-  for (uint32_t i = 0; i < nT; i++) {
-    q1.P[i] = p.P[g + i]; q1.Q[i] = p.Q[g + i]; q1.F[i] = p.F[g + i]; q1.strideF[i] = p.strideF[g + i];
-  }
-  q1.Z = temp1; q1.strideZ = (uint64_t)p.M * K;
-  q1.Y = nullptr; q1.strideY = 0; q1.alpha = 1.0; q1.beta = 0.0;
+  KronProblem q1, q2;
+  if (!buildSplit(p, g, temp1, temp2, &q1, &q2)) return fastKronKernelNotFound;
   Plan plan1 = db_.selectOnline(q1, dev_, true);
   if (plan1.size() != 1 || db_.kernels()[plan1[0].kernel].P == 0) return fastKronKernelNotFound;
-  if (execute(q1, plan1, nullptr, nullptr, true) != fastKronSuccess) return fastKronKernelNotFound;
-
-  // part 2: leading factors as a KMM over every row block; P x Q storage is the transpose of KMM's Q x P
-  KronProblem q2 = p;
-  q2.mm = MMType::KMM; q2.M = (uint32_t)T; q2.N = g;
-  q2.opF = (p.opF == fastKronOp_N) ? fastKronOp_T : fastKronOp_N;
-  q2.opX = fastKronOp_N;
-  q2.X = temp1; q2.strideX = K;
-  q2.strideZ = K; q2.strideY = K;
-  q2.batch = p.batch * p.M; q2.strided = true;
-  for (uint32_t i = 0; i < g; i++) q2.strideF[i] = 0;
   Plan plan2 = db_.selectOnline(q2, dev_, true);
-  // more than two leading launches ping-pong between temp2 and Z, which must then not be Y
-  if (plan2.size() > 2 && p.Y == p.Z && p.beta != 0.0) return fastKronKernelNotFound;
-  if (execute(q2, plan2, temp2, nullptr, true) != fastKronSuccess) return fastKronKernelNotFound;
+  return runSplit(p, g, q1, plan1, q2, plan2, temp2);
+}
 
-  lastPlan_ = p.str();
-  for (auto& s : plan1)
-    lastPlan_ += ";" + std::to_string(g + s.lo) + "-" + std::to_string(g + s.hi) + ":" + db_.kernels()[s.kernel].name;
-  for (auto& s : plan2)
-    lastPlan_ += ";" + std::to_string(s.lo) + "-" + std::to_string(s.hi) + ":" + db_.kernels()[s.kernel].name;
-  if (planOnly_) {
-    launchLog_.clear();
-    (void)execute(q1, plan1, nullptr, nullptr, true);
-    return execute(q2, plan2, temp2, nullptr, true);
+// A tuned record with explicit merge / split fields for this problem, if the file has one.
+bool Handle::lookupChoice(const KronProblem& p, Choice* c) const {
+  int merge = -1;
+  uint32_t split = 0;
+  Plan plan;
+  if (!db_.lookupTuned(p.str(), &plan, &merge, &split) || merge < 0) return false;
+  c->merge = merge != 0; c->split = split; c->plan = plan;
+  return true;
+}
+
+// Runs a tuned choice; fastKronKernelNotFound when it does not fit this call (the caller then selects online).
+fastKronError Handle::runChoice(const KronProblem& p0, const Choice& c, void* temp1, void* temp2, const CallWorkspace* ws) {
+  KronProblem p = p0;
+  if (c.merge) {
+    KronProblem merged;
+    if (!mergeSmallFactors(p0, &merged, ws)) return fastKronKernelNotFound;
+    p = merged;
   }
-  fastKronError e = execute(q1, plan1, nullptr, nullptr);
+  if (c.split) {
+    KronProblem q1, q2;
+    if (!buildSplit(p, c.split, temp1, temp2, &q1, &q2)) return fastKronKernelNotFound;
+    Plan plan1, plan2;
+    for (auto& s : c.plan) {
+      if (s.lo >= c.split) plan1.push_back(PlanStep{s.lo - c.split, s.hi - c.split, s.kernel});
+      else if (s.hi < c.split) plan2.push_back(s);
+      else return fastKronKernelNotFound;
+    }
+    if (!db_.validPlan(q1, plan1, dev_) || !db_.validPlan(q2, plan2, dev_)) return fastKronKernelNotFound;
+    return runSplit(p, c.split, q1, plan1, q2, plan2, temp2);
+  }
+  if (!db_.validPlan(p, c.plan, dev_)) return fastKronKernelNotFound;
+  fastKronError e = execute(p, c.plan, temp1, temp2, true);
   if (e != fastKronSuccess) return e;
-  return execute(q2, plan2, temp2, nullptr);
+  lastPlan_ = p.str();
+  for (auto& s : c.plan)
+    lastPlan_ += ";" + std::to_string(s.lo) + "-" + std::to_string(s.hi) + ":" + db_.kernels()[s.kernel].name;
+  if (planOnly_) { launchLog_.clear(); return execute(p, c.plan, temp1, temp2, true); }
+  return execute(p, c.plan, temp1, temp2);
 }
 
 // Everything of a launch's arguments that follows from the problem and the factor range; the caller

@@ -46,7 +46,18 @@ class Handle {
 
   // Runs `plan` on the stream; temps may be null when the plan has a single launch.
   fastKronError execute(const KronProblem& p, const Plan& plan, void* temp1, void* temp2, bool dryRun = false);
-  fastKronError tune(const KronProblem& p, Plan* best);
+  // What a tuned record prescribes for a problem: merge small factors or not, two-part plan with `split` leading
+  // factors or one chain (0), and the launches (numbered in the chain after merging; for a two-part plan the
+  // trailing part's steps, on factors >= split, come first).
+  struct Choice { bool merge = false; uint32_t split = 0; Plan plan; };
+  // Times the alternatives for `p` (merged or not, every two-part split, every kernel on every sub-chain), stores the
+  // fastest under the problem's own string and returns it.
+  fastKronError tune(const KronProblem& p, bool haveTemp2, Choice* best);
+  bool lookupChoice(const KronProblem& p, Choice* c) const;
+  fastKronError runChoice(const KronProblem& p, const Choice& c, void* temp1, void* temp2, const CallWorkspace* ws);
+  bool buildSplit(const KronProblem& p, uint32_t g, void* temp1, void* temp2, KronProblem* q1, KronProblem* q2) const;
+  fastKronError runSplit(const KronProblem& p, uint32_t g, const KronProblem& q1, const Plan& plan1,
+                         const KronProblem& q2, const Plan& plan2, void* temp2);
   // MKM chains longer than a whole-row kernel can take: trailing factors by the row kernel on
   // M * prod(leading P) virtual rows, leading factors as a batched KMM over the row blocks.
   // Returns fastKronKernelNotFound when the problem does not have that form.

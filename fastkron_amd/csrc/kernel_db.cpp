@@ -1,6 +1,10 @@
 #include "kernel_db.h"
 
+#include <dlfcn.h>
+
 #include <cstdio>
+#include <cstdlib>
+#include <cstring>
 #include <fstream>
 #include <sstream>
 
@@ -438,9 +442,11 @@ bool KernelDB::validPlan(const KronProblem& p, const Plan& plan, const DeviceInf
   return expectHi == -1;
 }
 
-bool KernelDB::lookupTuned(const std::string& key, Plan* plan) const {
+bool KernelDB::lookupTuned(const std::string& key, Plan* plan, int* merge, uint32_t* split) const {
   auto it = tuned_.find(key);
   if (it == tuned_.end()) return false;
+  if (merge) *merge = it->second.merge;
+  if (split) *split = it->second.split;
   Plan pl;
   for (auto& s : it->second.steps) {
     int k = findByName(s.second);
@@ -451,15 +457,16 @@ bool KernelDB::lookupTuned(const std::string& key, Plan* plan) const {
   return true;
 }
 
-void KernelDB::storeTuned(const std::string& key, const Plan& plan, float ms) {
+void KernelDB::storeTuned(const std::string& key, const Plan& plan, float ms, int merge, uint32_t split) {
   Tuned t;
-  t.ms = ms;
+  t.ms = ms; t.merge = merge; t.split = split;
   for (auto& s : plan) t.steps.push_back({{s.lo, s.hi}, kernels_[s.kernel].name});
   tuned_[key] = t;
 }
 
 // File format, one problem per line:
-//   <problem string> <ms> <nsteps> {<lo> <hi> <kernel name>}...
+//   <problem string> <ms> [M<merge> S<split>] <nsteps> {<lo> <hi> <kernel name>}...
+// (lines without the M / S fields leave both to the online selection)
 bool KernelDB::loadFile(const std::string& path) {
   std::ifstream f(path);
   if (!f) return false;
@@ -467,9 +474,20 @@ bool KernelDB::loadFile(const std::string& path) {
   while (std::getline(f, line)) {
     if (line.empty() || line[0] == '#') continue;
     std::istringstream is(line);
-    std::string key; float ms; size_t n;
-    if (!(is >> key >> ms >> n)) continue;
+    std::string key, tok; float ms; size_t n = 0;
+    if (!(is >> key >> ms >> tok)) continue;
     Tuned t; t.ms = ms;
+    if (!tok.empty() && tok[0] == 'M') {
+      std::string stok;
+      if (!(is >> stok >> n) || stok.empty() || stok[0] != 'S') continue;
+      t.merge = atoi(tok.c_str() + 1) ? 1 : 0;
+      t.split = (uint32_t)strtoul(stok.c_str() + 1, nullptr, 10);
+    } else {
+      char* end = nullptr;
+      n = strtoul(tok.c_str(), &end, 10);
+      if (end == tok.c_str() || *end) continue;
+    }
+    if (n == 0 || n > kMaxFactors) continue;
     bool ok = true;
     for (size_t i = 0; i < n; i++) {
       uint32_t lo, hi; std::string name;
@@ -486,7 +504,9 @@ bool KernelDB::saveFile(const std::string& path) const {
   if (!f) return false;
   f << "# fastkron gfx950 tuned launch plans: problem ms nsteps {lo hi kernel}\n";
   for (auto& kv : tuned_) {
-    f << kv.first << " " << kv.second.ms << " " << kv.second.steps.size();
+    f << kv.first << " " << kv.second.ms;
+    if (kv.second.merge >= 0) f << " M" << kv.second.merge << " S" << kv.second.split;
+    f << " " << kv.second.steps.size();
     for (auto& s : kv.second.steps) f << " " << s.first.first << " " << s.first.second << " " << s.second;
     f << "\n";
   }
@@ -496,6 +516,19 @@ bool KernelDB::saveFile(const std::string& path) const {
 std::string KernelDB::defaultPath() {
   if (const char* e = getenv("FASTKRON_TUNED_DB")) return e;
   return "";
+}
+
+// The plans tuned on an MI355X that ship with the library: gfx950_plans.txt in the directory above the one that
+// holds libFastKron.so (found through the address of this function).  FASTKRON_SHIPPED_PLANS=0 switches them off.
+std::string KernelDB::shippedPath() {
+  const char* e = getenv("FASTKRON_SHIPPED_PLANS");
+  if (e && !strcmp(e, "0")) return "";
+  Dl_info info;
+  if (!dladdr((const void*)&KernelDB::shippedPath, &info) || !info.dli_fname) return "";
+  std::string lib = info.dli_fname;
+  const size_t slash = lib.rfind('/');
+  if (slash == std::string::npos) return "";
+  return lib.substr(0, slash) + "/../gfx950_plans.txt";
 }
 
 }  // namespace fk

@@ -70,16 +70,25 @@ class KernelDB {
   // accepts its factor range (a plan read from a file is not trusted before it passes this).
   bool validPlan(const KronProblem& p, const Plan& plan, const DeviceInfo& dev) const;
 
-  // Tuned plans, keyed by the problem string.
-  bool lookupTuned(const std::string& key, Plan* plan) const;
-  void storeTuned(const std::string& key, const Plan& plan, float ms);
+  // Tuned plans, keyed by the problem string.  A record may also say how the chain is to be rewritten before the plan
+  // applies: `merge` (1: adjacent small factors replaced by their Kronecker products, 0: not, -1: unspecified, as the
+  // online selection decides) and `split` (g > 0: the plan's steps on factors >= g are the trailing part of a two-part
+  // plan, run on the contiguous blocks of the rows, the steps on factors < g the leading part, run across the blocks).
+  bool lookupTuned(const std::string& key, Plan* plan, int* merge = nullptr, uint32_t* split = nullptr) const;
+  void storeTuned(const std::string& key, const Plan& plan, float ms, int merge = -1, uint32_t split = 0);
   bool loadFile(const std::string& path);
   bool saveFile(const std::string& path) const;
   static std::string defaultPath();
+  static std::string shippedPath();
 
  private:
   std::vector<KernelInfo> kernels_;
-  struct Tuned { std::vector<std::pair<std::pair<uint32_t, uint32_t>, std::string>> steps; float ms; };
+  struct Tuned {
+    std::vector<std::pair<std::pair<uint32_t, uint32_t>, std::string>> steps;
+    float ms;
+    int merge = -1;
+    uint32_t split = 0;
+  };
   std::map<std::string, Tuned> tuned_;
 };
 

@@ -93,5 +93,7 @@ hipError_t launchFusedSmall(const StepArgs& a, DType dt, hipStream_t stream);
 
 // Kronecker products of adjacent small factors into the handle's workspace, one workgroup per product.
 hipError_t launchMergeFactors(const MergeArgs& a, DType dt, hipStream_t stream);
+// Fills `elems` elements with values spread over [-1, 1] (data for the tuner's timing runs).
+hipError_t launchFill(void* dst, size_t elems, DType dt, hipStream_t stream);
 
 }  // namespace fk

@@ -34,6 +34,26 @@ __global__ __launch_bounds__(256) void kron_merge_kernel(const MergeArgs a) {
   }
 }
 
+// Fills a buffer with values spread over [-1, 1] (a hash of the index): what the tuner times kernels on.  Zeros or a
+// constant would let the device clock higher than real data does.
+template <typename T>
+__global__ __launch_bounds__(256) void kron_fill_kernel(T* dst, size_t n) {
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
+    uint32_t h = (uint32_t)i * 2654435761u + (uint32_t)(i >> 32) * 40503u;
+    h ^= h >> 15; h *= 2246822519u; h ^= h >> 13;
+    dst[i] = (T)((double)(h & 0xffffff) / 8388608.0 - 1.0);
+  }
+}
+
+hipError_t launchFill(void* dst, size_t elems, DType dt, hipStream_t stream) {
+  if (elems == 0) return hipSuccess;
+  const size_t want = (elems + 255) / 256;
+  const uint32_t grid = want < 4096 ? (uint32_t)want : 4096;
+  if (dt == DType::F32) hipLaunchKernelGGL(kron_fill_kernel<float>, dim3(grid), dim3(256), 0, stream, (float*)dst, elems);
+  else                  hipLaunchKernelGGL(kron_fill_kernel<double>, dim3(grid), dim3(256), 0, stream, (double*)dst, elems);
+  return hipGetLastError();
+}
+
 hipError_t launchMergeFactors(const MergeArgs& a, DType dt, hipStream_t stream) {
   if (a.groups == 0 || a.groups > kMaxMergeGroups) return hipErrorInvalidValue;
   if (dt == DType::F32) hipLaunchKernelGGL(kron_merge_kernel<float>, dim3(a.groups), dim3(256), 0, stream, a);

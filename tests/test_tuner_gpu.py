@@ -1,0 +1,101 @@
+"""The tuner (fastKronOptionsTune): what it searches, what it stores, and that a stored plan is what a later handle
+runs.  Counterpart of the reference's fast tuning (reference src/autotuner/autotuner.cpp:24-150,158-328), which times
+every kernel on every sub-chain and keeps the result in memory; here the search also covers merged / unmerged chains
+and two-part plans, and the result is kept in a file."""
+import re
+import time
+
+import numpy as np
+import pytest
+
+from oracle import kron_oracle as ko
+from tests.gpu_util import TOL, make_case, normwise, oracle_answer, run_gpu
+
+pytestmark = pytest.mark.gpu
+
+
+def run_and_check(h, mm, M, Ps, dt, alpha, beta, seed, **run_kw):
+    X, Fs, Y = make_case(mm, M, Ps, Ps, dt, seed=seed, with_y=(beta != 0))
+    want = oracle_answer(mm, M, Ps, Ps, X, Fs, Y, alpha, beta)
+    got, e = run_gpu(h, mm, M, Ps, Ps, X, Fs, Y, alpha, beta, **run_kw)
+    assert e == 0
+    assert normwise(got, want) <= TOL[dt]
+
+
+def record_of(text, key):
+    for line in text.splitlines():
+        if line.startswith(key + " "):
+            return line
+    return None
+
+
+@pytest.mark.parametrize("M,Ps,dt", [(8, [16] * 5, np.float32), (4, [4] * 8, np.float32), (2, [64] * 3, np.float64),
+                                     (16, [2, 3, 4, 5, 6, 7, 8], np.float32), (4, [8] * 5, np.float64)])
+def test_tuned_record_names_merging_and_split_and_is_reused(tmp_path, M, Ps, dt):
+    import fastkron_amd
+    db = str(tmp_path / "plans.txt")
+    h = fastkron_amd.FastKron(tune=True)
+    h.set_tuned_db(db)
+    try:
+        run_and_check(h, ko.MKM, M, Ps, dt, 1.5, 0.5, seed=301)
+        tuned_plan = h.last_plan()
+    finally:
+        h.close()
+    K = int(np.prod(Ps))
+    facs = f"{Ps[0]}x{Ps[0]}^{len(Ps)}" if len(set(Ps)) == 1 else "(x)".join(f"{p}x{p}" for p in Ps)
+    key = f"{M}x{K}*({facs})_NN_{'f' if dt == np.float32 else 'd'}"
+    rec = record_of(open(db).read(), key)
+    assert rec is not None, open(db).read()
+    assert re.match(re.escape(key) + r" [0-9.e+-]+ M[01] S\d+ \d+ ", rec), rec
+    # a handle that does not tune runs the stored plan, on other data
+    h2 = fastkron_amd.FastKron(tune=False)
+    h2.set_tuned_db(db)
+    try:
+        run_and_check(h2, ko.MKM, M, Ps, dt, 1.0, 0.0, seed=302)
+        assert h2.last_plan() == tuned_plan
+        # ... and falls back to the online selection when the call's buffers do not allow the stored plan
+        run_and_check(h2, ko.MKM, M, Ps, dt, 1.0, 0.0, seed=303, use_temp2=False)
+    finally:
+        h2.close()
+
+
+def _time_calls(h, M, Ps, X, Fs, Z, t1, t2, reps=30):
+    import torch
+    for _ in range(5):
+        assert h.xgemkm(M, Ps, Ps, X, Fs, Z, 1.0, 0.0, None, t1, t2) == 0
+    torch.cuda.synchronize()
+    best = float("inf")
+    for _ in range(5):
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            h.xgemkm(M, Ps, Ps, X, Fs, Z, 1.0, 0.0, None, t1, t2)
+        torch.cuda.synchronize()
+        best = min(best, (time.perf_counter() - t0) / reps)
+    return best
+
+
+def test_tuned_plan_of_a_mixed_chain_is_not_slower_than_the_online_one(tmp_path):
+    """2x2 (x) 3x3 (x) ... (x) 8x8: the online rules group the factors greedily from the last one; the tuner times the
+    groupings and must come out at least as fast (5 % allowed for timing noise)."""
+    import torch
+    import fastkron_amd
+    M, Ps = 1024, [2, 3, 4, 5, 6, 7, 8]
+    K = int(np.prod(Ps))
+    dev = "cuda:0"
+    X = torch.rand(M * K, device=dev) * 2 - 1
+    Fs = [torch.rand(p * p, device=dev) * 2 - 1 for p in Ps]
+    Z = torch.empty(M * K, device=dev)
+    t1, t2 = torch.empty(M * K, device=dev), torch.empty(M * K, device=dev)
+    online = fastkron_amd.FastKron(tune=False)
+    tuned = fastkron_amd.FastKron(tune=True)
+    tuned.set_tuned_db(str(tmp_path / "plans.txt"))
+    try:
+        t_online = _time_calls(online, M, Ps, X, Fs, Z, t1, t2)
+        z_online = Z.clone()
+        t_tuned = _time_calls(tuned, M, Ps, X, Fs, Z, t1, t2)
+        assert normwise(Z.cpu().numpy(), z_online.cpu().numpy()) <= 1e-5
+        print(f"online {t_online * 1e3:.4f} ms {online.last_plan()}\ntuned  {t_tuned * 1e3:.4f} ms {tuned.last_plan()}")
+        assert t_tuned <= 1.05 * t_online, (t_tuned, t_online, tuned.last_plan(), online.last_plan())
+    finally:
+        online.close()
+        tuned.close()
