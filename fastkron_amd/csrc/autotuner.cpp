@@ -183,19 +183,46 @@ fastKronError Handle::tune(const KronProblem& p0, bool haveTemp2, Choice* best) 
 
   struct Variant { Choice c; float estimate; float measured; };
   std::vector<Variant> variants;
+  // op(X) = T: also everything the untransposed problem offers, behind a transposed copy of X (timed by itself here)
+  float transposeMs = 0.f;
+  KronProblem pT = p0;
+  bool canTranspose = false;
+  if (p0.opX == fastKronOp_T && useFusion()) {
+    void* xt = nullptr;
+    KronProblem src = onBuffers(p0);
+    canTranspose = transposedProblem(src, B.t1, haveTemp2 ? B.t2 : nullptr, &pT, &xt);
+    if (canTranspose) {
+      for (int i = 0; i < kWarm; i++) (void)launchTransposeX(src, xt, pT.strideX);
+      (void)hipStreamSynchronize(stream_);
+      (void)hipEventRecord(B.e0, stream_);
+      for (int i = 0; i < kRuns; i++) {
+        src.X = B.in[i % B.in.size()];
+        (void)launchTransposeX(src, xt, pT.strideX);
+      }
+      (void)hipEventRecord(B.e1, stream_);
+      (void)hipEventSynchronize(B.e1);
+      (void)hipEventElapsedTime(&transposeMs, B.e0, B.e1);
+      transposeMs /= kRuns;
+    }
+  }
+  for (int tx = 0; tx < (canTranspose ? 2 : 1); tx++)
   for (int merge = 0; merge < 2; merge++) {
-    KronProblem q = p0;
+    KronProblem base = p0;
+    if (tx) { base.opX = fastKronOp_N; }
+    KronProblem q = base;
     if (merge) {
       KronProblem m;
-      if (!useFusion() || !mergeSmallFactors(p0, &m)) continue;
+      if (!useFusion() || !mergeSmallFactors(base, &m)) continue;
       q = m;
     }
     q = onBuffers(q);
+    const float extra = tx ? transposeMs : 0.f;
     Plan plan;
     float ms = 0;
     if (tuneChain(*this, q, B, useFusion(), verbose, &plan, &ms)) {
-      Variant v; v.c.merge = merge != 0; v.c.split = 0; v.c.plan = plan; v.estimate = ms; v.measured = FLT_MAX;
-      variants.push_back(v);
+      Variant v; v.c.merge = merge != 0; v.c.split = 0; v.c.plan = plan; v.estimate = ms + extra; v.measured = FLT_MAX;
+      v.c.transposeX = tx != 0;
+      if (!(tx && !haveTemp2 && plan.size() != 1)) variants.push_back(v);
     }
     if (!useFusion() || !haveTemp2) continue;
     for (uint32_t g = 1; g < q.N; g++) {
@@ -206,7 +233,8 @@ fastKronError Handle::tune(const KronProblem& p0, bool haveTemp2, Choice* best) 
       if (!tuneSingle(*this, q1, B, verbose, &plan1, &ms1)) continue;
       if (!tuneChain(*this, q2, B, true, verbose, &plan2, &ms2)) continue;
       if (plan2.size() > 2 && p0.Y == p0.Z && p0.beta != 0.0) continue;
-      Variant v; v.c.merge = merge != 0; v.c.split = g; v.estimate = ms1 + ms2; v.measured = FLT_MAX;
+      Variant v; v.c.merge = merge != 0; v.c.split = g; v.estimate = ms1 + ms2 + extra; v.measured = FLT_MAX;
+      v.c.transposeX = tx != 0;
       for (auto& s : plan1) v.c.plan.push_back(PlanStep{s.lo + g, s.hi + g, s.kernel});
       for (auto& s : plan2) v.c.plan.push_back(s);
       variants.push_back(v);
@@ -240,8 +268,8 @@ fastKronError Handle::tune(const KronProblem& p0, bool haveTemp2, Choice* best) 
     (void)hipEventElapsedTime(&ms, B.e0, B.e1);
     v.measured = ms / kRuns;
     if (verbose) {
-      printf("[fastkron] tune %s: merge=%d split=%u estimate %.4f ms, end to end %.4f ms:", p0.str().c_str(), (int)v.c.merge,
-             v.c.split, v.estimate, v.measured);
+      printf("[fastkron] tune %s: transposeX=%d merge=%d split=%u estimate %.4f ms, end to end %.4f ms:", p0.str().c_str(),
+             (int)v.c.transposeX, (int)v.c.merge, v.c.split, v.estimate, v.measured);
       for (auto& s : v.c.plan) printf(" [%u,%u] %s", s.lo, s.hi, db_.kernels()[s.kernel].name.c_str());
       printf("\n");
     }
@@ -252,7 +280,7 @@ fastKronError Handle::tune(const KronProblem& p0, bool haveTemp2, Choice* best) 
     if (variants[vi].measured != FLT_MAX && (!win || variants[vi].measured < win->measured)) win = &variants[vi];
   if (!win) return fastKronKernelNotFound;
   *best = win->c;
-  db_.storeTuned(p0.str(), win->c.plan, win->measured, win->c.merge ? 1 : 0, win->c.split);
+  db_.storeTuned(p0.str(), win->c.plan, win->measured, win->c.merge ? 1 : 0, win->c.split, win->c.transposeX ? 1 : 0);
   if (!dbPath_.empty()) db_.saveFile(dbPath_);
   return fastKronSuccess;
 }

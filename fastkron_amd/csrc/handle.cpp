@@ -195,7 +195,98 @@ fastKronError Handle::xgemm(KronProblem p, fastKronBackend backend, void* temp1,
     }
   }
 
-  // 2. Online selection.
+  // 2. Online selection.  With op(X) = T first the question whether to transpose X ahead of the launches.
+  if (p.opX == fastKronOp_T && !p.forward && useFusion()) {
+    KronProblem pn;
+    void* xt = nullptr;
+    if (transposedProblem(p, temp1, temp2, &pn, &xt) && transposeFirstOnline(p, pn, temp1, temp2, ws)) {
+      if (!planOnly_) {
+        hipError_t he = launchTransposeX(p, xt, pn.strideX);
+        if (he != hipSuccess) return fastKronInvalidArgument;
+      }
+      e = runOnline(pn, temp1, temp2, ws);
+      if (e == fastKronSuccess) noteTranspose(p);
+      return e;
+    }
+  }
+  return runOnline(p, temp1, temp2, ws);
+}
+
+// How many launches the last planned call makes (entries of lastPlan_).
+static size_t countLaunches(const std::string& plan) {
+  size_t n = 0;
+  for (char ch : plan) if (ch == ';') n++;
+  return n;
+}
+
+// The problem with X already transposed into `xt` (temp2, or temp1 when there is no temp2): false when X does not
+// fit there.  The transposed copy has the compact layout, batch entries one after the other.
+bool Handle::transposedProblem(const KronProblem& p, void* temp1, void* temp2, KronProblem* pn, void** xt) const {
+  if (p.opX != fastKronOp_T) return false;
+  size_t yElems = 0, tmpElems = 0;
+  if (sizes(p.M, p.N, p.P, p.Q, &yElems, &tmpElems) != fastKronSuccess) return false;
+  if ((size_t)p.M * p.K() > tmpElems) return false;                  // shrinking chains: X is larger than a temporary
+  *xt = temp2 ? temp2 : temp1;
+  if (!*xt) return false;
+  *pn = p;
+  pn->opX = fastKronOp_N;
+  pn->X = *xt;
+  pn->strideX = (p.batch > 1 && p.strideX != 0) ? (uint64_t)p.M * p.K() : 0;
+  return true;
+}
+
+hipError_t Handle::launchTransposeX(const KronProblem& p, void* xt, uint64_t xtStride) {
+  // MKM: op(X) = T means the buffer holds K x M; KMM: it holds M x K (reference tests/testBase.h:272-273,303-304)
+  const uint32_t R = p.mm == MMType::MKM ? (uint32_t)p.K() : p.M;
+  const uint32_t C = p.mm == MMType::MKM ? p.M : (uint32_t)p.K();
+  const uint32_t nb = (p.batch > 1 && p.strideX != 0) ? p.batch : 1;       // a shared X is transposed once
+  constexpr uint32_t kMaxGridBatch = 65535;
+  for (uint32_t b0 = 0; b0 < nb; b0 += kMaxGridBatch) {
+    const uint32_t n = nb - b0 < kMaxGridBatch ? nb - b0 : kMaxGridBatch;
+    const size_t es = dtypeSize(p.dt);
+    hipError_t he = launchTranspose((const char*)p.X + (size_t)b0 * p.strideX * es, (char*)xt + (size_t)b0 * xtStride * es, R, C, n,
+                                    p.strideX, xtStride, p.dt, stream_);
+    if (he != hipSuccess) return he;
+  }
+  return hipSuccess;
+}
+
+// lastPlan_ of a call that transposed X first: the call's own problem string, the transposition as a launch ahead
+// of the last factor, then the launches of the untransposed problem.
+void Handle::noteTranspose(const KronProblem& p) {
+  const size_t semi = lastPlan_.find(';');
+  const std::string rest = semi == std::string::npos ? "" : lastPlan_.substr(semi);
+  lastPlan_ = p.str() + ";" + std::to_string(p.N - 1) + "-" + std::to_string(p.N - 1) + ":transpose_hip_gfx950_256_" +
+              (p.dt == DType::F32 ? "f" : "d") + "_x" + rest;
+}
+
+// Online rule for op(X) = T: transpose first when that plus the launches of the untransposed problem are no more
+// launches (passes over the data) than the kernels that read a transposed X need.  Both plans are laid out in
+// plan-only mode on the call's own buffers; the answer is kept per problem.
+bool Handle::transposeFirstOnline(const KronProblem& p, const KronProblem& pn, void* temp1, void* temp2,
+                                  const CallWorkspace* ws) {
+  const std::string ck = p.str() + (temp2 ? "_t2" : "_t1");
+  auto it = transposeCache_.find(ck);
+  if (it != transposeCache_.end()) return it->second;
+  const bool wasPlanOnly = planOnly_;
+  const std::string savedPlan = lastPlan_, savedLog = launchLog_;
+  planOnly_ = true;
+  size_t nT = 0, nN = 0;
+  const bool okT = runOnline(p, temp1, temp2, ws) == fastKronSuccess;
+  nT = countLaunches(lastPlan_);
+  const bool okN = runOnline(pn, temp1, temp2, ws) == fastKronSuccess;
+  nN = countLaunches(lastPlan_);
+  planOnly_ = wasPlanOnly;
+  lastPlan_ = savedPlan; launchLog_ = savedLog;
+  // without a second temporary the transposed copy sits in temp1, which a plan of several launches writes
+  bool yes = okN && (!okT || 1 + nN <= nT);
+  if (yes && !temp2 && nN != 1) yes = false;
+  transposeCache_[ck] = yes;
+  return yes;
+}
+
+fastKronError Handle::runOnline(KronProblem p, void* temp1, void* temp2, const CallWorkspace* ws) {
+  fastKronError e;
   {
     KronProblem merged;
     if (useFusion() && mergeSmallFactors(p, &merged, ws)) p = merged;
@@ -426,16 +517,28 @@ fastKronError Handle::trySplitLeadingTrailing(const KronProblem& p, void* temp1,
 
 // A tuned record with explicit merge / split fields for this problem, if the file has one.
 bool Handle::lookupChoice(const KronProblem& p, Choice* c) const {
-  int merge = -1;
+  int merge = -1, transposeX = 0;
   uint32_t split = 0;
   Plan plan;
-  if (!db_.lookupTuned(p.str(), &plan, &merge, &split) || merge < 0) return false;
-  c->merge = merge != 0; c->split = split; c->plan = plan;
+  if (!db_.lookupTuned(p.str(), &plan, &merge, &split, &transposeX) || merge < 0) return false;
+  c->merge = merge != 0; c->split = split; c->plan = plan; c->transposeX = transposeX != 0;
   return true;
 }
 
 // Runs a tuned choice; fastKronKernelNotFound when it does not fit this call (the caller then selects online).
 fastKronError Handle::runChoice(const KronProblem& p0, const Choice& c, void* temp1, void* temp2, const CallWorkspace* ws) {
+  if (c.transposeX) {
+    KronProblem pn;
+    void* xt = nullptr;
+    if (!transposedProblem(p0, temp1, temp2, &pn, &xt)) return fastKronKernelNotFound;
+    if (!temp2 && (c.split || c.plan.size() != 1)) return fastKronKernelNotFound;      // the copy sits in temp1 then
+    Choice rest = c;
+    rest.transposeX = false;
+    if (!planOnly_ && launchTransposeX(p0, xt, pn.strideX) != hipSuccess) return fastKronInvalidArgument;
+    fastKronError e = runChoice(pn, rest, temp1, temp2, ws);
+    if (e == fastKronSuccess) noteTranspose(p0);
+    return e;
+  }
   KronProblem p = p0;
   if (c.merge) {
     KronProblem merged;

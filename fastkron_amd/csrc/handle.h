@@ -49,10 +49,17 @@ class Handle {
   // What a tuned record prescribes for a problem: merge small factors or not, two-part plan with `split` leading
   // factors or one chain (0), and the launches (numbered in the chain after merging; for a two-part plan the
   // trailing part's steps, on factors >= split, come first).
-  struct Choice { bool merge = false; uint32_t split = 0; Plan plan; };
+  struct Choice { bool transposeX = false; bool merge = false; uint32_t split = 0; Plan plan; };
   // Times the alternatives for `p` (merged or not, every two-part split, every kernel on every sub-chain), stores the
   // fastest under the problem's own string and returns it.
   fastKronError tune(const KronProblem& p, bool haveTemp2, Choice* best);
+  // The online selection: merge by rule, tuned records of the older kind, the two-part plan by rule, greedy choice.
+  fastKronError runOnline(KronProblem p, void* temp1, void* temp2, const CallWorkspace* ws);
+  // op(X) = T handled by a transposed copy of X ahead of the launches (into temp2, or temp1 for a single launch)
+  bool transposedProblem(const KronProblem& p, void* temp1, void* temp2, KronProblem* pn, void** xt) const;
+  bool transposeFirstOnline(const KronProblem& p, const KronProblem& pn, void* temp1, void* temp2, const CallWorkspace* ws);
+  hipError_t launchTransposeX(const KronProblem& p, void* xt, uint64_t xtStride);
+  void noteTranspose(const KronProblem& p);
   bool lookupChoice(const KronProblem& p, Choice* c) const;
   fastKronError runChoice(const KronProblem& p, const Choice& c, void* temp1, void* temp2, const CallWorkspace* ws);
   bool buildSplit(const KronProblem& p, uint32_t g, void* temp1, void* temp2, KronProblem* q1, KronProblem* q2) const;
@@ -92,6 +99,7 @@ class Handle {
   DeviceInfo dev_;
   KernelDB db_;
   std::unordered_map<std::string, Plan> planCache_;   // online selections, per problem string
+  std::unordered_map<std::string, bool> transposeCache_;   // op(X) = T: transpose first or not, per problem string
   std::string dbPath_;
   std::string lastPlan_;
   void* mergeWs_ = nullptr;                           // device memory for merged factors, allocated by initHIP

@@ -442,11 +442,12 @@ bool KernelDB::validPlan(const KronProblem& p, const Plan& plan, const DeviceInf
   return expectHi == -1;
 }
 
-bool KernelDB::lookupTuned(const std::string& key, Plan* plan, int* merge, uint32_t* split) const {
+bool KernelDB::lookupTuned(const std::string& key, Plan* plan, int* merge, uint32_t* split, int* transposeX) const {
   auto it = tuned_.find(key);
   if (it == tuned_.end()) return false;
   if (merge) *merge = it->second.merge;
   if (split) *split = it->second.split;
+  if (transposeX) *transposeX = it->second.transposeX;
   Plan pl;
   for (auto& s : it->second.steps) {
     int k = findByName(s.second);
@@ -457,15 +458,15 @@ bool KernelDB::lookupTuned(const std::string& key, Plan* plan, int* merge, uint3
   return true;
 }
 
-void KernelDB::storeTuned(const std::string& key, const Plan& plan, float ms, int merge, uint32_t split) {
+void KernelDB::storeTuned(const std::string& key, const Plan& plan, float ms, int merge, uint32_t split, int transposeX) {
   Tuned t;
-  t.ms = ms; t.merge = merge; t.split = split;
+  t.ms = ms; t.merge = merge; t.split = split; t.transposeX = transposeX;
   for (auto& s : plan) t.steps.push_back({{s.lo, s.hi}, kernels_[s.kernel].name});
   tuned_[key] = t;
 }
 
 // File format, one problem per line:
-//   <problem string> <ms> [M<merge> S<split>] <nsteps> {<lo> <hi> <kernel name>}...
+//   <problem string> <ms> [M<merge> S<split> [X<transposeX>]] <nsteps> {<lo> <hi> <kernel name>}...
 // (lines without the M / S fields leave both to the online selection)
 bool KernelDB::loadFile(const std::string& path) {
   std::ifstream f(path);
@@ -478,10 +479,17 @@ bool KernelDB::loadFile(const std::string& path) {
     if (!(is >> key >> ms >> tok)) continue;
     Tuned t; t.ms = ms;
     if (!tok.empty() && tok[0] == 'M') {
-      std::string stok;
-      if (!(is >> stok >> n) || stok.empty() || stok[0] != 'S') continue;
+      std::string stok, ntok;
+      if (!(is >> stok >> ntok) || stok.empty() || stok[0] != 'S') continue;
       t.merge = atoi(tok.c_str() + 1) ? 1 : 0;
       t.split = (uint32_t)strtoul(stok.c_str() + 1, nullptr, 10);
+      if (!ntok.empty() && ntok[0] == 'X') {
+        t.transposeX = atoi(ntok.c_str() + 1) ? 1 : 0;
+        if (!(is >> ntok)) continue;
+      }
+      char* end = nullptr;
+      n = strtoul(ntok.c_str(), &end, 10);
+      if (end == ntok.c_str() || *end) continue;
     } else {
       char* end = nullptr;
       n = strtoul(tok.c_str(), &end, 10);
@@ -505,7 +513,10 @@ bool KernelDB::saveFile(const std::string& path) const {
   f << "# fastkron gfx950 tuned launch plans: problem ms nsteps {lo hi kernel}\n";
   for (auto& kv : tuned_) {
     f << kv.first << " " << kv.second.ms;
-    if (kv.second.merge >= 0) f << " M" << kv.second.merge << " S" << kv.second.split;
+    if (kv.second.merge >= 0) {
+      f << " M" << kv.second.merge << " S" << kv.second.split;
+      if (kv.second.transposeX) f << " X1";
+    }
     f << " " << kv.second.steps.size();
     for (auto& s : kv.second.steps) f << " " << s.first.first << " " << s.first.second << " " << s.second;
     f << "\n";

@@ -74,8 +74,11 @@ class KernelDB {
   // applies: `merge` (1: adjacent small factors replaced by their Kronecker products, 0: not, -1: unspecified, as the
   // online selection decides) and `split` (g > 0: the plan's steps on factors >= g are the trailing part of a two-part
   // plan, run on the contiguous blocks of the rows, the steps on factors < g the leading part, run across the blocks).
-  bool lookupTuned(const std::string& key, Plan* plan, int* merge = nullptr, uint32_t* split = nullptr) const;
-  void storeTuned(const std::string& key, const Plan& plan, float ms, int merge = -1, uint32_t split = 0);
+  // `transposeX` (1: op(X) = T is handled by a transposed copy of X ahead of the launches, which then see op(X) = N).
+  bool lookupTuned(const std::string& key, Plan* plan, int* merge = nullptr, uint32_t* split = nullptr,
+                   int* transposeX = nullptr) const;
+  void storeTuned(const std::string& key, const Plan& plan, float ms, int merge = -1, uint32_t split = 0,
+                  int transposeX = 0);
   bool loadFile(const std::string& path);
   bool saveFile(const std::string& path) const;
   static std::string defaultPath();
@@ -88,6 +91,7 @@ class KernelDB {
     float ms;
     int merge = -1;
     uint32_t split = 0;
+    int transposeX = 0;
   };
   std::map<std::string, Tuned> tuned_;
 };

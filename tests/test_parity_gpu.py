@@ -74,6 +74,21 @@ def test_transposed_operands(fk, mm, opX, opFs, M, Ps, Qs):
     check(fk, mm, M, Ps, Qs, np.float64, alpha=2.0, beta=1.0, opX=opX, opFs=opFs)
 
 
+@pytest.mark.parametrize("mm,M,Ps,dt", [(ko.MKM, 16, [8] * 5, np.float32), (ko.MKM, 4, [16] * 4, np.float32),
+                                        (ko.MKM, 100, [32] * 3, np.float32), (ko.MKM, 3, [64] * 2, np.float64),
+                                        (ko.MKM, 2, [16] * 5, np.float32), (ko.MKM, 5, [16] * 3, np.float64),
+                                        (ko.KMM, 64, [4] * 6, np.float32), (ko.KMM, 40, [16] * 2, np.float64),
+                                        (ko.MKM, 13, [12] * 3, np.float32), (ko.MKM, 7, [4] * 8, np.float32)])
+def test_transposed_x_ahead_of_the_whole_row_kernels(fk, mm, M, Ps, dt):
+    """op(X) = T on shapes whose fast kernels need contiguous rows: X is transposed into a temporary first
+    (reference general-tests-TT.cpp:36-83 runs its whole shape list with transposed operands)."""
+    check(fk, mm, M, Ps, Ps, dt, alpha=1.5, beta=0.5, seed=71, opX=ko.OP_T, opFs=ko.OP_T)
+    plan = fk.last_plan()
+    assert plan[0][2].startswith("transpose_"), plan
+    check(fk, mm, M, Ps, Ps, dt, alpha=1.0, beta=0.0, seed=72, opX=ko.OP_T, opFs=ko.OP_N, batch=3, share_f=True)
+    check(fk, mm, M, Ps, Ps, dt, alpha=1.0, beta=1.0, seed=73, opX=ko.OP_T, opFs=ko.OP_N, batch=2)
+
+
 @pytest.mark.parametrize("mm", [ko.MKM, ko.KMM])
 @pytest.mark.parametrize("share_f,share_y", [(False, False), (True, False), (True, True)])
 @pytest.mark.parametrize("M,Ps,Qs", [(16, [32] * 3, [16] * 3), (8, [32, 32], [64, 64]), (5, [3, 4], [2, 5])])

@@ -205,3 +205,33 @@ def test_tuned_plans_that_do_not_fit_the_problem_are_ignored(planner, tmp_path):
     lib.fastKronSetTunedDB(h, str(f).encode())
     e, names, _ = plan(planner, "mkm", "s", 8, [8, 8, 8], [8, 8, 8])
     assert e == capi.SUCCESS and names == [generic] * 3
+
+
+# ---- op(X) = T: a transposed copy of X ahead of the launches when that saves passes over the data ----
+def test_transposed_x_is_copied_first_when_the_whole_row_kernels_then_apply(planner):
+    e, names, launches = plan(planner, "mkm", "s", 64, [8] * 5, [8] * 5, opX=capi.OP_T)
+    assert e == capi.SUCCESS
+    assert names[0].startswith("transpose_") and "_8x8_8x8_5_1x32768" in names[1] and len(names) == 2, names
+    # the launches read the copy (temp2), not X
+    assert int(launches[0]["in"], 16) == BASE + 4 * GAP
+    # the same for the two-part plan of a longer chain and for GeKMM
+    e, names, _ = plan(planner, "mkm", "s", 8, [16] * 5, [16] * 5, opX=capi.OP_T)
+    assert e == capi.SUCCESS and names[0].startswith("transpose_") and len(names) == 3, names
+    e, names, _ = plan(planner, "kmm", "s", 64, [4] * 6, [4] * 6, opX=capi.OP_T)
+    assert e == capi.SUCCESS and names[0].startswith("transpose_") and "_4x4_4x4_6_8x4096" in names[1], names
+
+
+def test_transposed_x_is_read_in_place_when_a_copy_does_not_pay_or_does_not_fit(planner):
+    # one factor: the stride-general kernels read the transposed X directly, a copy would add a pass
+    e, names, _ = plan(planner, "mkm", "s", 64, [64], [64], opX=capi.OP_T)
+    assert e == capi.SUCCESS and not any(n.startswith("transpose_") for n in names), names
+    # shrinking chain: X (M x 32768) is larger than a temporary (M x 16384)
+    e, names, _ = plan(planner, "mkm", "s", 64, [32] * 3, [16] * 3, opX=capi.OP_T)
+    assert e == capi.SUCCESS and not any(n.startswith("transpose_") for n in names), names
+    # no second temporary and a plan of several launches: temp1 cannot hold the copy
+    e, names, _ = plan(planner, "mkm", "s", 8, [16] * 5, [16] * 5, opX=capi.OP_T, temp2=False)
+    assert e == capi.SUCCESS and not any(n.startswith("transpose_") for n in names), names
+    # no second temporary but a single launch: the copy goes to temp1
+    e, names, launches = plan(planner, "mkm", "s", 64, [8] * 5, [8] * 5, opX=capi.OP_T, temp2=False)
+    assert e == capi.SUCCESS and names[0].startswith("transpose_") and len(names) == 2, names
+    assert int(launches[0]["in"], 16) == BASE + 3 * GAP
