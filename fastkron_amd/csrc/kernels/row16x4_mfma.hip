@@ -60,7 +60,9 @@ constexpr int kCarry = ROW16_CARRY;        // slices of the next row in flight d
 constexpr uint32_t kStaggerGroups = 5;     // measured: 5 groups 2.5 us apart or 3 groups 4 us apart; 2 or 4 groups lose to no stagger
 constexpr uint32_t kStaggerTicks = 250;    // of the 100 MHz wall clock
 constexpr int kQuarterWords = 16384;       // 64 KB: 16 rows k1 of 1024 columns (four values of q2)
-constexpr int kLdsWords = 2 * kQuarterWords + 5 * 256;   // two quarters + the four factors + F2 transposed
+constexpr int kFacWords = 320;            // a staged factor: element (p, q) at 16*(p + p/4) + q (rows padded so that lanes
+                                          // reading rows 4k + c, k = lane/16, cover all 64 banks)
+constexpr int kLdsWords = 2 * kQuarterWords + 4 * kFacWords + 256;   // two quarters + the four factors + F2 transposed
 
 template <bool HAS_Y>
 __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a, const uint32_t blocksPerBatch,
@@ -76,12 +78,12 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a,
   // Factors: a.f[0] is the last factor (F4) ... a.f[3] the first (F1); with fewer than four factors the
   // leading digits are row indices (16^(4-nf) consecutive rows form the same contiguous 65536-element
   // block) and their factor slots hold the identity.  The four 16x16 matrices are staged in LDS behind
-  // the exchange buffers, fl[j*256 + p*16 + q], F2 a second time as f2t[k2*16 + (q2%4)*4 + q2/4] (the 4x4x1 operand of a lane, the four
+  // the exchange buffers, fl[j*320 + 16*(p + p/4) + q], F2 a second time as f2t[k2*16 + (q2%4)*4 + q2/4] (the 4x4x1 operand of a lane, the four
   // values F2[k2][4*qq + lane%4], is one 16-byte read), and operands
   // are read from there right before use: LDS reads do not queue behind the row loads the way small global
   // loads would (vector memory operations retire in order).
   float* fl = lds + 2 * kQuarterWords;
-  float* f2t = fl + 4 * 256;
+  float* f2t = fl + 4 * kFacWords;
   auto stageFactors = [&](uint32_t b) {
     const int j = tid >> 8, p = (tid >> 4) & 15, q = tid & 15;
     float v = (p == q) ? 1.f : 0.f;
@@ -89,7 +91,7 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a,
       const float* f = (const float*)a.f[j] + (size_t)b * a.f_batch[j];
       v = f[(int64_t)p * a.f_sp[j] + (int64_t)q * a.f_sq[j]];
     }
-    fl[tid] = v;
+    fl[j * kFacWords + 16 * (p + (p >> 2)) + q] = v;
     if (j == 2) f2t[p * 16 + (q & 3) * 4 + (q >> 2)] = v;      // [k2][q2 % 4][q2 / 4]
   };
   bool perBatchFactors = false;
@@ -162,8 +164,8 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a,
       float FA[4], FB[4];
 #pragma unroll
       for (int c = 0; c < 4; c++) {
-        FA[c] = fl[1 * 256 + (4 * kb + c) * 16 + i];      // F3
-        FB[c] = fl[0 * 256 + (4 * kb + c) * 16 + i];      // F4
+        FA[c] = fl[1 * kFacWords + (5 * kb + c) * 16 + i];      // F3
+        FB[c] = fl[0 * kFacWords + (5 * kb + c) * 16 + i];      // F4
       }
       const float* const xcur = slicePtr(item);
 #pragma unroll
@@ -201,17 +203,20 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a,
 
     // Exchange geometry.  A quarter buffer holds T2[k1][q2l][piece][4]: row k1 (1024 words), q2l = q2 % 4, and the
     // 256 columns (q3,q4) of one q2 as 64 pieces of four.  Column piece o = 4*q3 + q4/4 sits at position
-    // (o & 48) | ((o & 15) ^ (o >> 4)): the writers of a quarter wave (one kb, 16 values of i: pieces 4 apart) and
-    // the readers of a quarter wave (16 consecutive pieces) both cover all 64 banks.
+    // (o & 48) | (swap(o & 15) ^ 4*((o >> 4) & 1)), swap exchanging the two bit pairs of its argument.  The LDS takes a
+    // 16-byte write eight consecutive lanes at a time and a 16-byte read sixteen at a time (measured: patterns that
+    // repeat a bank within such a group count as conflicts, others do not): the eight writers (one kb, i = 8h .. 8h+7:
+    // pieces 4 apart) land on positions that differ modulo 8, the sixteen readers (consecutive pieces) on positions
+    // that differ modulo 16.
     const int wo = i * 4 + kb;
-    float* const wbase = lds + w * 1024 + (((wo & 48) | ((wo & 15) ^ (wo >> 4))) << 2);
+    float* const wbase = lds + w * 1024 + (((wo & 48) | ((((wo & 15) >> 2) | ((wo & 3) << 2)) ^ (((wo >> 4) & 1) << 2))) << 2);
     // reader: wave w takes q2l = w/4 and the 64 columns g = w%4 of it; lane (kb, i) reads row k1 = 4c + kb,
     // piece 16*g + i, and ends up with Z[q1 = 4kb + r][q2][64*g + 4*i + e] in register r of accumulator e
     const int g = w & 3, q2l = w >> 2;
-    const float* const rbase = lds + kb * 1024 + q2l * 256 + g * 64 + ((i ^ g) << 2);
+    const float* const rbase = lds + kb * 1024 + q2l * 256 + g * 64 + ((((i >> 2) | ((i & 3) << 2)) ^ ((g & 1) << 2)) << 2);
     float f1[4];
 #pragma unroll
-    for (int c = 0; c < 4; c++) f1[c] = fl[3 * 256 + (4 * c + kb) * 16 + i];      // A operand: F1[k1 = 4c+kb][q1 = i]
+    for (int c = 0; c < 4; c++) f1[c] = fl[3 * kFacWords + (5 * c + kb) * 16 + i];      // A operand: F1[k1 = 4c+kb][q1 = i]
 
     // quarter qq of the k2 result, written to buffer qq % 2
     auto produce = [&](const int qq) {
