@@ -502,6 +502,7 @@ fastKronError Handle::trySplitLeadingTrailing(const KronProblem& p, void* temp1,
   // (few blocks of 16^4: the wave-per-block kernel for three factors spreads them over more CUs)
   if (p.dt == DType::F32 && tp == 16 && p.N >= 4 && (uint64_t)p.M * (p.K() / 65536) * p.batch < 96) maxT = 3;
   if (maxT == 0 && tp >= 9 && tp <= 15) maxT = 3;       // zero-padded form of the 16x16x3 wave-per-block kernel
+  if (maxT == 0 && tp >= 17 && tp <= 31) maxT = 2;      // zero-padded form of the 32x32 pair kernel
   if (maxT == 0) return fastKronKernelNotFound;
   uint32_t nT = 0;
   while (nT < maxT && nT < p.N && p.P[p.N - 1 - nT] == tp && p.Q[p.N - 1 - nT] == tp) nT++;

@@ -209,8 +209,11 @@ static bool stepF64Check(const KernelInfo& k, const StepArgs& a) { return stepMf
 static bool pairCanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
                        const DeviceInfo& dev) {
   if (p.dt != k.dt || p.mm != MMType::MKM || hi - lo + 1 != 2 || p.forward) return false;
-  for (uint32_t i = lo; i <= hi; i++) if (p.P[i] != k.P || p.Q[i] != k.Q) return false;
-  if (p.colsBefore(hi) != (uint64_t)k.P * k.P) return false;
+  // the 32x32 kernel also takes factors of 17x17 ... 31x31, zero-padded to its tile
+  const uint32_t P = p.P[hi];
+  if (!(P == k.P || (k.P == 32 && P >= 17 && P < 32))) return false;
+  for (uint32_t i = lo; i <= hi; i++) if (p.P[i] != P || p.Q[i] != P) return false;
+  if (p.colsBefore(hi) != (uint64_t)P * P) return false;
   if (first && p.opX == 2) return false;
   return dev.ldsPerBlock >= (int)(2 * k.P * k.P * 8 + 8 * 8192);
 }

@@ -66,7 +66,10 @@ template <> struct PairMfma<float> {
   static __device__ __forceinline__ int row(int r, int hi) { return 4 * hi + r; }
 };
 
-template <typename T, int P, bool HAS_Y>
+// EXACT = false: factors of R x R with 16 < R < P, operands zero-padded to the P x P tile: a row is R*R contiguous
+// elements, loaded and stored element by element with indices >= R masked (what the padded lanes and registers
+// compute is exact zeros and is never stored).
+template <typename T, int P, bool HAS_Y, bool EXACT = true>
 __global__ __launch_bounds__(256, 2) void kron_pair_kernel(const StepArgs a) {
   using MF = PairMfma<T>;
   using Acc = typename MF::Acc;
@@ -87,6 +90,7 @@ __global__ __launch_bounds__(256, 2) void kron_pair_kernel(const StepArgs a) {
   const T* YB = HAS_Y ? (const T*)a.y + (size_t)bt * a.y_batch : nullptr;
   // multiplying by 1 is exact: launches that do not write Z need no branch around the scaling
   const T alpha = a.epilogue ? (T)a.alpha : (T)1, beta = (T)a.beta;
+  const int R = EXACT ? P : (int)a.p[0];            // the factors' real size; the row is R * R elements
 
   {
     const T* Fa = (const T*)a.f[0] + (size_t)bt * a.f_batch[0];
@@ -97,8 +101,9 @@ __global__ __launch_bounds__(256, 2) void kron_pair_kernel(const StepArgs a) {
 #pragma unroll
     for (int k = 0; k < P * P / 256; k++) {
       const int i = tid + 256 * k, p = i / P, q = i % P;
-      va[k] = Fa[(int64_t)p * a.f_sp[0] + (int64_t)q * a.f_sq[0]];
-      vb[k] = Fb[(int64_t)p * a.f_sp[1] + (int64_t)q * a.f_sq[1]];
+      const bool in = EXACT || (p < R && q < R);
+      va[k] = in ? Fa[(int64_t)p * a.f_sp[0] + (int64_t)q * a.f_sq[0]] : (T)0;
+      vb[k] = in ? Fb[(int64_t)p * a.f_sp[1] + (int64_t)q * a.f_sq[1]] : (T)0;
     }
 #pragma unroll
     for (int k = 0; k < P * P / 256; k++) { fA[tid + 256 * k] = va[k]; fB[tid + 256 * k] = vb[k]; }
@@ -108,7 +113,15 @@ __global__ __launch_bounds__(256, 2) void kron_pair_kernel(const StepArgs a) {
   const uint32_t stride = gridDim.x * kPairWaves;
   auto loadRow = [&](uint32_t row, T (&x)[PB][PC]) {
     const int lo = l0 & 15, hi = l0 >> 4;
-    const T* xp = inB + (size_t)row * a.in_ldm + lo * P + PC * hi;
+    const T* xp = inB + (size_t)row * a.in_ldm + lo * R + PC * hi;
+    if (!EXACT) {
+#pragma unroll
+      for (int g = 0; g < PB; g++)
+#pragma unroll
+        for (int c = 0; c < PC; c++)
+          x[g][c] = (16 * g + lo < R && PC * hi + c < R) ? xp[g * 16 * R + c] : (T)0;
+      return;
+    }
 #pragma unroll
     for (int g = 0; g < PB; g++)
 #pragma unroll
@@ -160,7 +173,9 @@ __global__ __launch_bounds__(256, 2) void kron_pair_kernel(const StepArgs a) {
 #pragma unroll
           for (int u = 0; u < 2; u++)
 #pragma unroll
-            for (int r = 0; r < 4; r++) yv[u][r] = Y[(16 * (jb2 + u) + MF::row(r, hi)) * P + ofs];
+            for (int r = 0; r < 4; r++)
+              yv[u][r] = (EXACT || (16 * (jb2 + u) + MF::row(r, hi) < R && ofs < R))
+                             ? Y[(16 * (jb2 + u) + MF::row(r, hi)) * R + ofs] : (T)0;
         }
 #pragma unroll
         for (int u = 0; u < 2; u++)
@@ -168,7 +183,8 @@ __global__ __launch_bounds__(256, 2) void kron_pair_kernel(const StepArgs a) {
           for (int r = 0; r < 4; r++) {               // q_b = 16*(jb2+u) + row(r, hi), q_a = 16*jb + lo
             T v = acc[u][r] * alpha;
             if (HAS_Y) v += beta * yv[u][r];
-            out[(16 * (jb2 + u) + MF::row(r, hi)) * P + ofs] = v;
+            if (EXACT || (16 * (jb2 + u) + MF::row(r, hi) < R && ofs < R))
+              out[(16 * (jb2 + u) + MF::row(r, hi)) * R + ofs] = v;
           }
       }
     }
@@ -383,9 +399,10 @@ __global__ __launch_bounds__(512, 2) void kron_pair64_f64_kernel(const StepArgs 
 bool pairMfmaSupported(const StepArgs& a, DType dt) {
   if (a.nf != 2) return false;
   const uint32_t P = a.p[0];
-  if ((P != 64 && P != 32) || a.q[0] != P || a.p[1] != P || a.q[1] != P) return false;
+  if ((P != 64 && (P < 17 || P > 32)) || a.q[0] != P || a.p[1] != P || a.q[1] != P) return false;
   if (a.Kin != (uint64_t)P * P || a.Kout != a.Kin) return false;
   if (a.in_ldc != 1 || a.out_ldc != 1 || (a.y && a.y_ldc != 1)) return false;
+  if (P < 32) return a.batch <= 65535;                                                // padded form: element-wise accesses
   const uint64_t vmask = 16 / dtypeSize(dt) - 1;                                      // 128-bit loads
   if (((uintptr_t)a.in & 15) || ((uint64_t)a.in_ldm & vmask) || (a.in_batch & vmask)) return false;
   if (dt == DType::F64 && P == 64) {                                                  // and 128-bit stores / Y loads
@@ -395,7 +412,7 @@ bool pairMfmaSupported(const StepArgs& a, DType dt) {
   return a.batch <= 65535;
 }
 
-template <typename T, int P>
+template <typename T, int P, bool EXACT = true>
 static hipError_t launchPairT(const StepArgs& a, hipStream_t stream) {
   const int cus = deviceCUs();
   const size_t ldsBytes = 2 * P * P * sizeof(T);
@@ -409,15 +426,15 @@ static hipError_t launchPairT(const StepArgs& a, hipStream_t stream) {
   const int devIdx = launchDeviceIndex();
   const bool y = a.y && a.epilogue;
   if (!attrOnce[y].done(devIdx)) {
-    hipError_t e = y ? hipFuncSetAttribute((const void*)kron_pair_kernel<T, P, true>,
+    hipError_t e = y ? hipFuncSetAttribute((const void*)kron_pair_kernel<T, P, true, EXACT>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes)
-                     : hipFuncSetAttribute((const void*)kron_pair_kernel<T, P, false>,
+                     : hipFuncSetAttribute((const void*)kron_pair_kernel<T, P, false, EXACT>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes);
     if (e != hipSuccess) return e;
     attrOnce[y].mark(devIdx);
   }
-  if (y) hipLaunchKernelGGL((kron_pair_kernel<T, P, true>), grid, block, ldsBytes, stream, a);
-  else   hipLaunchKernelGGL((kron_pair_kernel<T, P, false>), grid, block, ldsBytes, stream, a);
+  if (y) hipLaunchKernelGGL((kron_pair_kernel<T, P, true, EXACT>), grid, block, ldsBytes, stream, a);
+  else   hipLaunchKernelGGL((kron_pair_kernel<T, P, false, EXACT>), grid, block, ldsBytes, stream, a);
   return hipGetLastError();
 }
 
@@ -447,6 +464,7 @@ static hipError_t launchPair64(const StepArgs& a, hipStream_t stream) {
 
 hipError_t launchPairMfma(const StepArgs& a, DType dt, hipStream_t stream) {
   if (!pairMfmaSupported(a, dt)) return hipErrorInvalidValue;
+  if (a.p[0] < 32) return dt == DType::F64 ? launchPairT<double, 32, false>(a, stream) : launchPairT<float, 32, false>(a, stream);
   if (dt == DType::F64) return a.p[0] == 64 ? launchPair64(a, stream) : launchPairT<double, 32>(a, stream);
   return a.p[0] == 64 ? launchPairT<float, 64>(a, stream) : launchPairT<float, 32>(a, stream);
 }

@@ -735,3 +735,18 @@ def test_wave_per_block_kernel_with_factors_of_9_to_15(fk, M, Ps, launches, dt):
     check(fk, ko.MKM, M, Ps, Ps, dt, alpha=1.0, beta=1.0, seed=903, batch=3, share_f=True)
     check(fk, ko.MKM, M, Ps, Ps, dt, alpha=2.0, beta=0.0, seed=904, batch=2)
     check(fk, ko.MKM, M, Ps, Ps, dt, alpha=1.0, beta=1.0, seed=905, integer=True)
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+@pytest.mark.parametrize("M,Ps,launches", [(16, [24, 24], 1), (5, [31, 31], 1), (7, [17, 17], 1), (3, [24] * 3, 2),
+                                           (2, [20] * 4, 3), (40, [28, 28], 1)])
+def test_pair_kernel_with_factors_of_17_to_31(fk, M, Ps, launches, dt):
+    """Two fused PxP factors, 17 <= P <= 31, on the 32x32 pair kernel with zero-padded operands (the reference fuses
+    square factors up to 32x32, reference src/kernel_db/kernel_db.cpp:164-181); longer chains take it for their two
+    trailing factors and run the leading ones across the blocks."""
+    check(fk, ko.MKM, M, Ps, Ps, dt, alpha=1.5, beta=0.5, seed=181)
+    plan = fk.last_plan()
+    assert len(plan) == launches and "_32x32_32x32_2_1x1024" in plan[0][2], plan
+    check(fk, ko.MKM, M, Ps, Ps, dt, alpha=1.0, beta=0.0, seed=182, opFs=ko.OP_T)
+    check(fk, ko.MKM, M, Ps, Ps, dt, alpha=1.0, beta=1.0, seed=183, batch=2)
+    check(fk, ko.MKM, M, Ps, Ps, dt, alpha=2.0, beta=0.0, seed=184, integer=True)
