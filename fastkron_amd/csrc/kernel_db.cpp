@@ -64,7 +64,7 @@ static hipError_t fusedSmallLaunch(const KernelInfo& k, const StepArgs& a, hipSt
 static bool fusedSmallCheck(const KernelInfo& k, const StepArgs& a) { return fusedSmallSupported(a, k.dt); }
 
 // ---- one factor of any shape up to 256x512 on the matrix cores (zero padded) ----
-static bool stepAnyCanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, uint32_t hi, bool, bool,
+static bool stepAnyCanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
                           const DeviceInfo& dev) {
   if (k.dt != p.dt || lo != hi) return false;
   const uint32_t P = p.P[lo], Q = p.Q[lo];
@@ -72,7 +72,10 @@ static bool stepAnyCanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo
   // Small factors are bound by memory on the plain kernel already; the padded tiles pay off from these sizes on
   // (measured per layout and type: e.g. fp32 MKM 18x18, fp64 MKM 12x12, fp32 KMM 31x31, fp64 KMM 20x20).
   const bool kmm = p.mm == MMType::KMM && p.M > 1;
-  const uint64_t minPQ = kmm ? (p.dt == DType::F32 ? 900 : 400) : (p.dt == DType::F32 ? 256 : 144);
+  uint64_t minPQ = kmm ? (p.dt == DType::F32 ? 900 : 400) : (p.dt == DType::F32 ? 256 : 144);
+  // a first launch that reads a transposed X: the plain kernel's lanes then run across the strided dimension, and the
+  // padded tiles win from 8x8 on (tuned plans: 16x16 chains with op(X) = T 2.6 times faster)
+  if (first && p.opX == 2) minPQ = 64;
   return ((uint64_t)P * Q >= minPQ || !dev.rulesOfThumb) && P >= 4;
 }
 static hipError_t stepAnyLaunch(const KernelInfo& k, const StepArgs& a, hipStream_t s) {
@@ -215,6 +218,9 @@ static bool pairCanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, u
   for (uint32_t i = lo; i <= hi; i++) if (p.P[i] != P || p.Q[i] != P) return false;
   if (p.colsBefore(hi) != (uint64_t)P * P) return false;
   if (first && p.opX == 2) return false;
+  // one wave per 64x64 block: with few blocks two single-factor launches, whose tiles are 16 times smaller, fill the
+  // device better (tuned plans at 256 blocks: 1.4 times faster in fp32, 1.9 times in fp64; at 1024 blocks the pair wins)
+  if (dev.rulesOfThumb && P == 64 && (uint64_t)p.M * p.batch < 512) return false;
   return dev.ldsPerBlock >= (int)(2 * k.P * k.P * 8 + 8 * 8192);
 }
 static hipError_t pairLaunch(const KernelInfo& k, const StepArgs& a, hipStream_t s) { return launchPairMfma(a, k.dt, s); }
@@ -380,7 +386,11 @@ void registerRowKernels(std::vector<KernelInfo>& out) {
     kd.canRun = stepF64CanRun; kd.launch = stepF64Launch; kd.check = stepF64Check;
     // fp32 16x16 in the KMM layout: the plain kernel's 256-byte accesses along M beat the 64-byte tile rows
     // and for 128x128 the padded step (factor in LDS instead of split over wave tasks) is a third faster
-    kd.tunerOnly = (variant == 1 && dt == DType::F32 && (P == 16 || P == 128));
+    // ... fp32 64x64 in that layout likewise (1.15 times), 16x16 in either type, and fp64 128x128 in both layouts (the
+    // padded step with the factor in LDS is 1.5 times faster than the factor split over eight wave tasks): all measured
+    // by tuning the reference's published shape table
+    kd.tunerOnly = (variant == 1 && P == 16) || (variant == 1 && dt == DType::F32 && (P == 64 || P == 128)) ||
+                   (dt == DType::F64 && P == 128);
     out.push_back(kd);
   }
 }

@@ -109,7 +109,7 @@ VECTOR_CASES = [
     ("row16x3d", "mkm", "d", 64, [16] * 3, [16] * 3, None, 0.5, "_d_16x16_16x16_3_1x4096"),
     ("row32x3", "mkm", "s", 128, [32] * 3, [32] * 3, None, 0.5, "_32x32_32x32_3_1x32768"),
     ("pair32", "mkm", "s", 64, [32] * 2, [32] * 2, None, 0.5, "_32x32_32x32_2_1x1024"),
-    ("pair64d", "mkm", "d", 64, [64] * 2, [64] * 2, None, 0.5, "_d_64x64_64x64_2_1x4096"),
+    ("pair64d", "mkm", "d", 512, [64] * 2, [64] * 2, None, 0.5, "_d_64x64_64x64_2_1x4096"),
     ("step64", "mkm", "s", 64, [64], [64], None, 0.5, "_64x64_64x64_1_"),
     ("kmm64d", "kmm", "d", 64, [64], [64], None, 0.5, "kmm_hip_gfx950_256_d_64x64_64x64_1_64x64"),
     ("row8x5", "mkm", "s", 64, [8] * 5, [8] * 5, None, 0.5, "_8x8_8x8_5_1x32768"),
@@ -222,8 +222,8 @@ def test_transposed_x_is_copied_first_when_the_whole_row_kernels_then_apply(plan
 
 
 def test_transposed_x_is_read_in_place_when_a_copy_does_not_pay_or_does_not_fit(planner):
-    # one factor: the stride-general kernels read the transposed X directly, a copy would add a pass
-    e, names, _ = plan(planner, "mkm", "s", 64, [64], [64], opX=capi.OP_T)
+    # one small factor: the plain kernel reads the transposed X directly, a copy would add a pass
+    e, names, _ = plan(planner, "mkm", "s", 64, [8], [8], opX=capi.OP_T)
     assert e == capi.SUCCESS and not any(n.startswith("transpose_") for n in names), names
     # shrinking chain: X (M x 32768) is larger than a temporary (M x 16384)
     e, names, _ = plan(planner, "mkm", "s", 64, [32] * 3, [16] * 3, opX=capi.OP_T)
