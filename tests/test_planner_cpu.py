@@ -235,3 +235,80 @@ def test_transposed_x_is_read_in_place_when_a_copy_does_not_pay_or_does_not_fit(
     e, names, launches = plan(planner, "mkm", "s", 64, [8] * 5, [8] * 5, opX=capi.OP_T, temp2=False)
     assert e == capi.SUCCESS and names[0].startswith("transpose_") and len(names) == 2, names
     assert int(launches[0]["in"], 16) == BASE + 3 * GAP
+
+
+# ---- the plans that ship with the library (fastkron_amd/gfx950_plans.txt) ----
+def _parse_key(key):
+    """'MxK*(PxQ^N)_NN_f' / '(PxQ^N)*KxM_TT_d' (factor lists as 'AxB(x)CxD') -> (mm, dt, M, Ps, Qs, opX, opF)."""
+    import re
+    m = re.match(r"^(\d+)x(\d+)\*\((.*)\)_([NT])([NT])_([fd])$", key)
+    if m:
+        mm, M, facs, ox, of, dt = "mkm", int(m.group(1)), m.group(3), m.group(4), m.group(5), m.group(6)
+    else:
+        m = re.match(r"^\((.*)\)\*(\d+)x(\d+)_([NT])([NT])_([fd])$", key)
+        assert m, key
+        mm, M, facs, ox, of, dt = "kmm", int(m.group(3)), m.group(1), m.group(4), m.group(5), m.group(6)
+    Ps, Qs = [], []
+    for f in facs.split("(x)"):
+        pq, _, n = f.partition("^")
+        p, q = pq.split("x")
+        Ps += [int(p)] * int(n or 1)
+        Qs += [int(q)] * int(n or 1)
+    op = {"N": capi.OP_N, "T": capi.OP_T}
+    return mm, ("s" if dt == "f" else "d"), M, Ps, Qs, op[ox], op[of]
+
+
+def _shipped_records():
+    import os
+    path = os.path.join(os.path.dirname(capi.LIB_PATH), "..", "gfx950_plans.txt")
+    recs = []
+    for line in open(path):
+        if line.startswith("#") or not line.strip():
+            continue
+        tok = line.split()
+        i = 2
+        flags = {}
+        while tok[i][0] in "MSX":
+            flags[tok[i][0]] = int(tok[i][1:])
+            i += 1
+        n = int(tok[i])
+        steps = [(int(tok[i + 1 + 3 * k]), int(tok[i + 2 + 3 * k]), tok[i + 3 + 3 * k]) for k in range(n)]
+        recs.append((tok[0], flags, steps))
+    return recs
+
+
+def test_every_shipped_plan_is_what_a_default_handle_runs(planner):
+    recs = _shipped_records()
+    assert len(recs) >= 10
+    for key, flags, steps in recs:
+        if "stridedBatched" in key:
+            continue
+        mm, dt, M, Ps, Qs, opX, opF = _parse_key(key)
+        e, names, launches = plan(planner, mm, dt, M, Ps, Qs, opX=opX, opF=opF)
+        assert e == capi.SUCCESS, key
+        want = [k for _, _, k in steps]
+        got = [n for n in names if not n.startswith("transpose_")]
+        assert got == want, (key, names, want)
+        assert any(n.startswith("transpose_") for n in names) == bool(flags.get("X", 0)), (key, names)
+
+
+def test_shipped_plans_can_be_switched_off(monkeypatch):
+    """FASTKRON_SHIPPED_PLANS=0: a handle created then selects online, as if the file were not there."""
+    import ctypes
+    recs = [r for r in _shipped_records() if "stridedBatched" not in r[0]]
+    monkeypatch.setenv("FASTKRON_SHIPPED_PLANS", "0")
+    lib = capi.load()
+    h = ctypes.c_void_p()
+    assert lib.fastKronInit(ctypes.byref(h), capi.BACKEND_HIP) == capi.SUCCESS
+    assert lib.fastKronSetPlanOnly(h, 1) == capi.SUCCESS
+    try:
+        differ = 0
+        for key, flags, steps in recs:
+            mm, dt, M, Ps, Qs, opX, opF = _parse_key(key)
+            e, names, _ = plan((lib, h), mm, dt, M, Ps, Qs, opX=opX, opF=opF)
+            assert e == capi.SUCCESS
+            got = [n for n in names if not n.startswith("transpose_")]
+            differ += got != [k for _, _, k in steps] or any(n.startswith("transpose_") for n in names) != bool(flags.get("X", 0))
+        assert differ == len(recs)          # every record is there because tuning beat the online plan
+    finally:
+        lib.fastKronDestroy(h)
