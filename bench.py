@@ -220,6 +220,35 @@ def measure(fk, name, steps, warmup, ramp_seconds, nsets, ev, stream, calibrate_
             "gflops": flop / (wall / steps) / 1e9, "roofline": roof, "dims": (M, Ps, Qs, alpha, beta, batch)}
 
 
+# reference documents/performance.md:5-137, the shapes of its A100 tables, "M_PxP^N"
+PUBLISHED_GPU_SHAPES = [(1024, 8, 5), (1024, 8, 6), (1024, 16, 4), (1024, 16, 5), (1024, 32, 3), (1024, 32, 4), (1024, 64, 2),
+                        (1024, 64, 3), (1024, 128, 2), (320, 128, 3), (16, 8, 8), (16, 16, 6), (16, 32, 5), (16, 64, 4),
+                        (16, 128, 3)]
+
+
+def shape_table(fk):
+    """Times every shape of the reference's published GPU table through the handle as a user gets it (online rules
+    plus the tuned plans that ship), operands rotated so that no cache holds them; wall clock around batches of
+    calls with a device synchronisation on both sides."""
+    import torch
+    from fastkron_amd.capi import OP_N, OP_T
+    from fastkron_amd.tune import _Case
+    for mm in ("mkm", "kmm"):
+        for dtype, dn in ((torch.float32, "float"), (torch.float64, "double")):
+            for ops, on in (((OP_N, OP_N), "NN"), ((OP_T, OP_T), "TT")):
+                for M, P, N in PUBLISHED_GPU_SHAPES:
+                    try:
+                        case = _Case(fk, mm, M, [P] * N, [P] * N, dtype)
+                    except torch.cuda.OutOfMemoryError:
+                        continue
+                    ms = case.time(fk, *ops, runs=20, samples=4)
+                    print(json.dumps({"mmtype": mm, "type": dn, "ops": on, "shape": f"{M}_{P}x{P}^{N}", "ms": round(ms, 5),
+                                      "gflops": round(case.gflops(ms), 1),
+                                      "launches": [k for _, _, k in fk.last_plan()]}), flush=True)
+                    del case
+                    torch.cuda.empty_cache()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -236,6 +265,10 @@ def main():
     ap.add_argument("--sets", type=int, default=3,
                     help="least number of operand sets rotated between steps; raised per workload until the sets add up "
                          "to 640 MB, so that the 256 MB Infinity Cache serves none of the traffic")
+    ap.add_argument("--shape-table", action="store_true",
+                    help="instead of the benchmark line: time the shapes of the reference's published GPU table "
+                         "(reference documents/performance.md:5-137: M_PxP^N for MKM and KMM, float and double, operands "
+                         "untransposed and transposed) with cold operands and print one JSON line per shape")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run 4 plain device copies of 256 MiB (a known-size kernel for scaling rocprof counters)")
     args = ap.parse_args()
@@ -252,6 +285,9 @@ def main():
     ev = HipEvents()
     sp = ctypes.c_void_p(stream.cuda_stream)
 
+    if args.shape_table:
+        shape_table(fk)
+        return
     head = measure(fk, args.config, args.steps, args.warmup, args.ramp_seconds, args.sets, ev, sp, args.calibrate_copy)
     out = {
         "metric": "GeMKM/GeKMM GFLOP/s on 1 MI355X (FastKron FLOP count 2*M*sum Kin_i*Q_i)",

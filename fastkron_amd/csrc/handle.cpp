@@ -231,6 +231,7 @@ bool Handle::transposedProblem(const KronProblem& p, void* temp1, void* temp2, K
   *pn = p;
   pn->opX = fastKronOp_N;
   pn->X = *xt;
+  pn->xJustWritten = true;
   pn->strideX = (p.batch > 1 && p.strideX != 0) ? (uint64_t)p.M * p.K() : 0;
   return true;
 }
@@ -453,6 +454,7 @@ bool Handle::buildSplit(const KronProblem& p, uint32_t g, void* temp1, void* tem
   }
   q1.Z = temp1; q1.strideZ = (uint64_t)p.M * K;
   q1.Y = nullptr; q1.strideY = 0; q1.alpha = 1.0; q1.beta = 0.0;
+  q1.zReadNext = true;
 
   // part 2: leading factors as a KMM over every row block; P x Q storage is the transpose of KMM's Q x P
   KronProblem q2 = p;
@@ -460,6 +462,7 @@ bool Handle::buildSplit(const KronProblem& p, uint32_t g, void* temp1, void* tem
   q2.opF = (p.opF == fastKronOp_N) ? fastKronOp_T : fastKronOp_N;
   q2.opX = fastKronOp_N;
   q2.X = temp1; q2.strideX = K;
+  q2.xJustWritten = true;
   q2.strideZ = K; q2.strideY = K;
   q2.batch = p.batch * p.M; q2.strided = true;
   for (uint32_t i = 0; i < g; i++) q2.strideF[i] = 0;
@@ -651,6 +654,19 @@ fastKronError Handle::execute(const KronProblem& p, const Plan& plan, void* temp
       }
       if (a.out == nullptr) return fastKronInvalidArgument;
     }
+    {
+      // Non-temporal hints (StepArgs::stream_in / stream_out).  Measured: an intermediate of 134 MB is read back
+      // from the memory-side cache by the next launch (non-temporal stores cost 4 % there), one of 268 MB is not
+      // (they gain 2 %); X and Z of a launch that moves 268 MB or more with nothing cached gain 2.5 to 4 %, also
+      // when Z itself is small (8 x 512 x (32x16)^3: 67 MB of Z behind 537 MB of X, 126.2 -> 121.9 us).
+      constexpr uint64_t kStreamFrom = 96ull << 20, kBeyondCache = 192ull << 20;
+      const uint64_t es8 = dtypeSize(p.dt);
+      const uint64_t inBytes = (uint64_t)p.M * a.Kin * p.batch * es8, outBytes = (uint64_t)p.M * a.Kout * p.batch * es8;
+      const uint64_t moved = inBytes + outBytes + (a.y ? outBytes : 0);
+      const bool inFromCaller = first && !p.xJustWritten, outToCaller = (last || p.forward) && !p.zReadNext;
+      a.stream_in = inFromCaller ? (moved >= kStreamFrom && inBytes >= kStreamFrom / 2) : inBytes > kBeyondCache;
+      a.stream_out = outToCaller ? moved >= kStreamFrom : outBytes > kBeyondCache;
+    }
     if (logLevel() >= 2)
       printf("[fastkron]   launch %zu: factors [%u,%u] Kin=%llu Kout=%llu kernel %s\n", l, s.lo, s.hi,
              (unsigned long long)a.Kin, (unsigned long long)a.Kout, k.name.c_str());
@@ -670,9 +686,10 @@ fastKronError Handle::execute(const KronProblem& p, const Plan& plan, void* temp
         if (planOnly_) {
           char line[768];
           int n = snprintf(line, sizeof(line), "kernel=%s lo=%u hi=%u M=%u batch=%u Kin=%llu Kout=%llu in=%p out=%p y=%p "
-                           "in_batch=%llu out_batch=%llu y_batch=%llu f_batch=", k.name.c_str(), s.lo, s.hi, c.M, c.batch,
+                           "in_batch=%llu out_batch=%llu y_batch=%llu stream_in=%u stream_out=%u f_batch=", k.name.c_str(), s.lo, s.hi, c.M, c.batch,
                            (unsigned long long)c.Kin, (unsigned long long)c.Kout, c.in, c.out, c.y,
-                           (unsigned long long)c.in_batch, (unsigned long long)c.out_batch, (unsigned long long)c.y_batch);
+                           (unsigned long long)c.in_batch, (unsigned long long)c.out_batch, (unsigned long long)c.y_batch,
+                           c.stream_in, c.stream_out);
           launchLog_.append(line, n > 0 ? (size_t)n : 0);
           for (uint32_t j = 0; j < c.nf && j < kMaxFused; j++)
             launchLog_ += (j ? "," : "") + std::to_string(c.f_batch[j]);

@@ -216,7 +216,7 @@ constexpr int kPair64Waves = 8;                     // one workgroup of 8 waves 
 constexpr int kPair64XWords = 16 * 64;              // doubles of X staging per wave: 16 rows of the tile
 constexpr size_t kPair64LdsBytes = (2 * kP64 * kP64 + kPair64Waves * kPair64XWords) * sizeof(double);
 
-template <bool HAS_Y>
+template <bool HAS_Y, int NT>
 __global__ __launch_bounds__(512, 2) void kron_pair64_f64_kernel(const StepArgs a) {
   constexpr int P = kP64;
   extern __shared__ double pairLds[];
@@ -262,7 +262,7 @@ __global__ __launch_bounds__(512, 2) void kron_pair64_f64_kernel(const StepArgs 
   auto loadPart = [&](uint32_t row, int tb) {
     const double* xp = inB + (size_t)row * a.in_ldm + 2 * l0 + tb * 1024;
 #pragma unroll
-    for (int j = 0; j < 8; j++) x[j] = *(const pd2*)(xp + j * 128);
+    for (int j = 0; j < 8; j++) x[j] = FK_LD(NT, (const pd2*)(xp + j * 128));
   };
 
   auto computeRow = [&](uint32_t row, uint32_t next) {
@@ -377,7 +377,7 @@ __global__ __launch_bounds__(512, 2) void kron_pair64_f64_kernel(const StepArgs 
           for (int h = 0; h < 2; h++) {
             pd2 v = {acc[uh + uu][2 * h] * alpha, acc[uh + uu][2 * h + 1] * alpha};
             if (HAS_Y) v += beta * yv[uu][h];
-            *(pd2*)(out + o0 + 4 * (uh + uu) * 64 + 32 * h) = v;
+            FK_ST(NT, v, (pd2*)(out + o0 + 4 * (uh + uu) * 64 + 32 * h));
           }
       }
     }
@@ -446,19 +446,22 @@ static hipError_t launchPair64(const StepArgs& a, hipStream_t stream) {
   if (wgs > need) wgs = need;
   if (wgs == 0) wgs = 1;
   dim3 grid(wgs, a.batch), block(64 * kPair64Waves);
-  static PerDeviceOnce attrOnce[2];
+  static PerDeviceOnce attrOnce;
   const int devIdx = launchDeviceIndex();
-  const bool y = a.y && a.epilogue;
-  if (!attrOnce[y].done(devIdx)) {
-    hipError_t e = y ? hipFuncSetAttribute((const void*)kron_pair64_f64_kernel<true>,
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)kPair64LdsBytes)
-                     : hipFuncSetAttribute((const void*)kron_pair64_f64_kernel<false>,
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)kPair64LdsBytes);
-    if (e != hipSuccess) return e;
-    attrOnce[y].mark(devIdx);
+  using Kernel = void (*)(const StepArgs);
+  static const Kernel kernels[2][3] = {
+      {kron_pair64_f64_kernel<false, 0>, kron_pair64_f64_kernel<false, 1>, kron_pair64_f64_kernel<false, 2>},
+      {kron_pair64_f64_kernel<true, 0>, kron_pair64_f64_kernel<true, 1>, kron_pair64_f64_kernel<true, 2>}};
+  if (!attrOnce.done(devIdx)) {
+    for (int y = 0; y < 2; y++)
+      for (int nt = 0; nt < 3; nt++) {
+        hipError_t e = hipFuncSetAttribute((const void*)kernels[y][nt], hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           (int)kPair64LdsBytes);
+        if (e != hipSuccess) return e;
+      }
+    attrOnce.mark(devIdx);
   }
-  if (y) hipLaunchKernelGGL((kron_pair64_f64_kernel<true>), grid, block, kPair64LdsBytes, stream, a);
-  else   hipLaunchKernelGGL((kron_pair64_f64_kernel<false>), grid, block, kPair64LdsBytes, stream, a);
+  hipLaunchKernelGGL(kernels[(a.y && a.epilogue) ? 1 : 0][streamMode(a)], grid, block, kPair64LdsBytes, stream, a);
   return hipGetLastError();
 }
 

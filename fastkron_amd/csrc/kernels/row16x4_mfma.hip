@@ -64,7 +64,7 @@ constexpr int kFacWords = 320;            // a staged factor: element (p, q) at 
                                           // reading rows 4k + c, k = lane/16, cover all 64 banks)
 constexpr int kLdsWords = 2 * kQuarterWords + 4 * kFacWords + 256;   // two quarters + the four factors + F2 transposed
 
-template <bool HAS_Y>
+template <bool HAS_Y, int NT>
 __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a, const uint32_t blocksPerBatch,
                                                                const uint32_t totalItems, const uint32_t staggerTicks) {
   extern __shared__ __align__(16) float lds[];
@@ -119,7 +119,7 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a,
   {
     const float* xp = slicePtr(item);
 #pragma unroll
-    for (int t = 0; t < kCarry; t++) xw[t] = *(const f4*)(xp + (laneOff + t * 256));
+    for (int t = 0; t < kCarry; t++) xw[t] = FK_LD(NT, (const f4*)(xp + (laneOff + t * 256)));
   }
   __syncthreads();
 
@@ -169,7 +169,7 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a,
       }
       const float* const xcur = slicePtr(item);
 #pragma unroll
-      for (int t = kCarry; t < kWin; t++) xw[t] = *(const f4*)(xcur + (laneOff + t * 256));
+      for (int t = kCarry; t < kWin; t++) xw[t] = FK_LD(NT, (const f4*)(xcur + (laneOff + t * 256)));
       // behind the last item the requests go to one cached kilobyte of the current row instead, and are dropped
       const float* const xnext = slicePtr(nx < totalItems ? nx : item);
       const int nextStride = nx < totalItems ? 256 : 0;
@@ -180,8 +180,8 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a,
 #pragma unroll
         for (int r = 0; r < 4; r++) d = MFMA16(xw[t % kWin][r], FB[r], d);     // d[k3][q4]
         // the slot is free: request the slice that comes kWin later
-        if (t + kWin < 16) xw[t % kWin] = *(const f4*)(xcur + (laneOff + (t + kWin) * 256));
-        else if (t + kWin - 16 < kCarry) xw[t % kWin] = *(const f4*)(xnext + (laneOff + (t + kWin - 16) * nextStride));
+        if (t + kWin < 16) xw[t % kWin] = FK_LD(NT, (const f4*)(xcur + (laneOff + (t + kWin) * 256)));
+        else if (t + kWin - 16 < kCarry) xw[t % kWin] = FK_LD(NT, (const f4*)(xnext + (laneOff + (t + kWin - 16) * nextStride)));
         f4 e = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int r = 0; r < 4; r++) e = MFMA16(d[r], FA[r], e);        // e[q4][q3]: e[r] = T[k2=t][q3=i][q4=4kb+r]
@@ -246,7 +246,7 @@ __global__ __launch_bounds__(1024, 1) void kron_row16x4_kernel(const StepArgs a,
       for (int r = 0; r < 4; r++) {
         f4 o = (f4){D[0][r], D[1][r], D[2][r], D[3][r]} * alpha;
         if (HAS_Y) o = o + yv[r] * beta;
-        *(GlobalF4*)(Z + (col + r * 4096)) = o;
+        FK_ST(NT, o, (GlobalF4*)(Z + (col + r * 4096)));
       }
     };
 
@@ -294,13 +294,16 @@ hipError_t launchRow16x4(const StepArgs& a, hipStream_t stream) {
   static PerDeviceOnce attrOnce;
   const int devIdx = launchDeviceIndex();
   const size_t ldsBytes = kLdsWords * sizeof(float);
+  using Kernel = void (*)(const StepArgs, const uint32_t, const uint32_t, const uint32_t);
+  static const Kernel kernels[2][3] = {
+      {kron_row16x4_kernel<false, 0>, kron_row16x4_kernel<false, 1>, kron_row16x4_kernel<false, 2>},
+      {kron_row16x4_kernel<true, 0>, kron_row16x4_kernel<true, 1>, kron_row16x4_kernel<true, 2>}};
   if (!attrOnce.done(devIdx)) {
-    hipError_t e = hipFuncSetAttribute((const void*)kron_row16x4_kernel<true>,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes);
-    if (e != hipSuccess) return e;
-    e = hipFuncSetAttribute((const void*)kron_row16x4_kernel<false>,
-                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes);
-    if (e != hipSuccess) return e;
+    for (int y = 0; y < 2; y++)
+      for (int nt = 0; nt < 3; nt++) {
+        hipError_t e = hipFuncSetAttribute((const void*)kernels[y][nt], hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes);
+        if (e != hipSuccess) return e;
+      }
     attrOnce.mark(devIdx);
   }
   const int cus = deviceCUs();
@@ -311,10 +314,8 @@ hipError_t launchRow16x4(const StepArgs& a, hipStream_t stream) {
   const uint32_t wgs = total < (uint64_t)cus ? (uint32_t)total : (uint32_t)cus;
   const uint32_t stagger = total >= 2ull * wgs ? kStaggerTicks : 0;
   dim3 grid(wgs), block(1024);
-  if (a.y && a.epilogue)
-    hipLaunchKernelGGL(kron_row16x4_kernel<true>, grid, block, ldsBytes, stream, a, blocksPerBatch, (uint32_t)total, stagger);
-  else
-    hipLaunchKernelGGL(kron_row16x4_kernel<false>, grid, block, ldsBytes, stream, a, blocksPerBatch, (uint32_t)total, stagger);
+  hipLaunchKernelGGL(kernels[(a.y && a.epilogue) ? 1 : 0][streamMode(a)], grid, block, ldsBytes, stream, a, blocksPerBatch,
+                     (uint32_t)total, stagger);
   return hipGetLastError();
 }
 

@@ -33,6 +33,10 @@ typedef float f4 __attribute__((ext_vector_type(4)));
 
 
 constexpr int kRow8Len = 32768;
+// The two workgroups of a CU would load, compute and store in lockstep; the later one starts 5 us behind (measured
+// on 1024 x 8^5 with cold operands: 59.5 us without, 57.7 with 5 us, 57.9 with 6, 58.0 with 7, 63 with 12; 512 rows
+// 31.1 -> 29.3 us, 768 rows 52.8 -> 47.8, 4096 rows 213.3 -> 211.7; one workgroup per CU is not delayed).
+constexpr uint32_t kRow8SlotDelayTicks = 500;
 constexpr int kRow8LdsWords = 16384 + 5 * 64;     // one half row + the five factors
 
 // Factor operand of the 4x4x1 products for this lane: fa[p][qq] = F[p][4*qq + (lane & 3)].
@@ -73,8 +77,8 @@ __device__ __forceinline__ void contractSecond(float (&x)[8][8], const float (&f
   }
 }
 
-template <bool HAS_Y>
-__global__ __launch_bounds__(512, 4) void kron_row8x5_kernel(const StepArgs a) {
+template <bool HAS_Y, int NT>
+__global__ __launch_bounds__(512, 4) void kron_row8x5_kernel(const StepArgs a, const uint32_t firstRound, const uint32_t delayTicks) {
   extern __shared__ __align__(16) float lds[];
   float* fl = lds + 16384;                       // factors: fl[f*64 + p*8 + q], f = 0 is F1
   const int tid = threadIdx.x;
@@ -90,6 +94,7 @@ __global__ __launch_bounds__(512, 4) void kron_row8x5_kernel(const StepArgs a) {
   // loads must not queue behind 128 KB of row data).  a.f[0] is the last factor F5 ... a.f[nf-1] the first.  With fewer than five
   // factors the leading digits are row indices (8^(5-nf) consecutive rows form the same contiguous
   // 32768-element block) and their factor slots hold the identity.
+  delayLaterWorkgroupOfCU(firstRound, delayTicks);
   if (tid < 320) {
     const int f = tid >> 6, e = tid & 63, p = e >> 3, q = e & 7;
     const int j = 4 - f;
@@ -108,7 +113,7 @@ __global__ __launch_bounds__(512, 4) void kron_row8x5_kernel(const StepArgs a) {
 #pragma unroll
     for (int j = 0; j < 8; j++)
 #pragma unroll
-      for (int i = 0; i < 8; i++) x[i][j] = xp[i * 4096 + j * 512];
+      for (int i = 0; i < 8; i++) x[i][j] = FK_LD(NT, &xp[i * 4096 + j * 512]);
   }
   __syncthreads();
 
@@ -209,7 +214,7 @@ __global__ __launch_bounds__(512, 4) void kron_row8x5_kernel(const StepArgs a) {
         v *= alpha;
         if (HAS_Y) v += beta * Y[col];
       }
-      Z[col] = v;
+      FK_ST(NT, v, &Z[col]);
     }
 }
 
@@ -233,20 +238,22 @@ hipError_t launchRow8x5(const StepArgs& a, hipStream_t stream) {
   static PerDeviceOnce attrOnce;
   const int devIdx = launchDeviceIndex();
   const size_t ldsBytes = kRow8LdsWords * sizeof(float);
+  using Kernel = void (*)(const StepArgs, const uint32_t, const uint32_t);
+  static const Kernel kernels[2][3] = {
+      {kron_row8x5_kernel<false, 0>, kron_row8x5_kernel<false, 1>, kron_row8x5_kernel<false, 2>},
+      {kron_row8x5_kernel<true, 0>, kron_row8x5_kernel<true, 1>, kron_row8x5_kernel<true, 2>}};
   if (!attrOnce.done(devIdx)) {
-    hipError_t e = hipFuncSetAttribute((const void*)kron_row8x5_kernel<true>,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes);
-    if (e != hipSuccess) return e;
-    e = hipFuncSetAttribute((const void*)kron_row8x5_kernel<false>,
-                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes);
-    if (e != hipSuccess) return e;
+    for (int y = 0; y < 2; y++)
+      for (int nt = 0; nt < 3; nt++) {
+        hipError_t e = hipFuncSetAttribute((const void*)kernels[y][nt], hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes);
+        if (e != hipSuccess) return e;
+      }
     attrOnce.mark(devIdx);
   }
   dim3 grid(a.M / row8Rows(a), a.batch), block(512);
-  if (a.y && a.epilogue)
-    hipLaunchKernelGGL(kron_row8x5_kernel<true>, grid, block, ldsBytes, stream, a);
-  else
-    hipLaunchKernelGGL(kron_row8x5_kernel<false>, grid, block, ldsBytes, stream, a);
+  const uint32_t firstRound = 2u * (uint32_t)deviceCUs();
+  hipLaunchKernelGGL(kernels[(a.y && a.epilogue) ? 1 : 0][streamMode(a)], grid, block, ldsBytes, stream, a, firstRound,
+                     kRow8SlotDelayTicks);
   return hipGetLastError();
 }
 

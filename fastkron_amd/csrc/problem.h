@@ -37,6 +37,9 @@ struct KronProblem {
   void* inter[kMaxFactors];           // forward only: inter[j] = output of the step of factor j+1
   uint64_t strideInter[kMaxFactors];
   bool haveStrideInter;
+  // Set for the parts of a call that the library runs as problems of their own: X was written by a launch of this
+  // call just before (a transposed copy, the first part of a two-part plan) / Z is read by the next launch.
+  bool xJustWritten, zReadNext;
 
   uint64_t K() const { uint64_t k = 1; for (uint32_t i = 0; i < N; i++) k *= P[i]; return k; }
   uint64_t L() const { uint64_t l = 1; for (uint32_t i = 0; i < N; i++) l *= Q[i]; return l; }
@@ -73,6 +76,10 @@ struct StepArgs {
   uint64_t in_batch, out_batch, y_batch;
   double   alpha, beta;
   uint32_t epilogue;                   // 1: out = alpha*acc + beta*y (beta term skipped when y is null)
+  // Hints for the kernels that have non-temporal variants: the input is large and was not written just before by
+  // a launch of this call / the output is large and no launch of this call reads it back (or it is larger than
+  // the memory-side cache anyway).  Such data gains nothing from being kept in the caches.
+  uint32_t stream_in, stream_out;
 };
 
 // Merging of adjacent small factors into their Kronecker product (kernels/merge_factors.hip).

@@ -312,3 +312,50 @@ def test_shipped_plans_can_be_switched_off(monkeypatch):
         assert differ == len(recs)          # every record is there because tuning beat the online plan
     finally:
         lib.fastKronDestroy(h)
+
+
+# ---- non-temporal hints: what a launch is told about its input and output ----
+def _hints(launches):
+    return [(int(r["stream_in"]), int(r["stream_out"])) for r in launches]
+
+
+def test_large_cold_operands_are_streamed(planner):
+    """One launch over 134 MB in and out (sgemkm 1024 x 8^5): both hints; the same call on 256 rows: none."""
+    e, names, launches = plan(planner, "mkm", "s", 1024, [8] * 5, [8] * 5)
+    assert e == capi.SUCCESS and len(launches) == 1 and _hints(launches) == [(1, 1)]
+    e, names, launches = plan(planner, "mkm", "s", 256, [8] * 5, [8] * 5)
+    assert e == capi.SUCCESS and _hints(launches) == [(0, 0)]
+
+
+def test_intermediates_that_fit_the_memory_side_cache_are_not_streamed(planner):
+    """sgemkm 128 x 8^6 runs two launches around an intermediate of 134 MB: the first launch streams X in but stores
+    ordinarily, the second loads ordinarily and streams Z out.  With 256 rows (268 MB) everything is streamed."""
+    e, names, launches = plan(planner, "mkm", "s", 128, [8] * 6, [8] * 6)
+    assert e == capi.SUCCESS and len(launches) == 2 and _hints(launches) == [(1, 0), (0, 1)]
+    e, names, launches = plan(planner, "mkm", "s", 256, [8] * 6, [8] * 6)
+    assert e == capi.SUCCESS and len(launches) == 2 and _hints(launches) == [(1, 1), (1, 1)]
+
+
+def test_a_transposed_copy_is_not_streamed_back_in(planner):
+    """op(X) = T behind a transposed copy: the copy (134 MB) was written a moment ago, so the launch that reads it
+    loads ordinarily."""
+    e, names, launches = plan(planner, "mkm", "s", 1024, [8] * 5, [8] * 5, opX=capi.OP_T, opF=capi.OP_T)
+    assert e == capi.SUCCESS and names[0].startswith("transpose_") and len(launches) == 1
+    assert _hints(launches) == [(0, 1)]
+
+
+def test_two_part_plans_keep_their_intermediate_ordinary(planner):
+    """sgemkm 16 x 16^6 (two-part plan, 1 GB per buffer): beyond the cache everything streams; 2 x 16^5 (8 MB): nothing."""
+    e, names, launches = plan(planner, "mkm", "s", 2, [16] * 5, [16] * 5)
+    assert e == capi.SUCCESS and all(h == (0, 0) for h in _hints(launches))
+    e, names, launches = plan(planner, "mkm", "s", 32, [16] * 5, [16] * 5)     # 134 MB per buffer
+    assert e == capi.SUCCESS and len(launches) >= 2
+    hints = _hints(launches)
+    assert hints[0][0] == 1 and hints[-1][1] == 1                  # X in and Z out are streamed
+    assert all(h[1] == 0 for h in hints[:-1]) and all(h[0] == 0 for h in hints[1:])   # nothing in between is
+
+
+def test_a_small_result_behind_a_large_input_is_streamed_out(planner):
+    """8 x 512 x (32x16)^3 with Y: 537 MB of X, 67 MB of Z; the launch moves far more than the caches hold."""
+    e, names, launches = plan(planner, "mkm", "s", 512, [32] * 3, [16] * 3, batch=8, beta=1.0, with_y=True)
+    assert e == capi.SUCCESS and len(launches) == 1 and _hints(launches) == [(1, 1)]
