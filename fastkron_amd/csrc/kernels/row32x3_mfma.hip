@@ -34,7 +34,8 @@ constexpr int kR32Len = 32768;
 constexpr int kR32QuarterWords = 32 * 256;                         // 32 rows k1 of 256 columns
 constexpr int kR32LdsWords = 2 * kR32QuarterWords + 3 * 1024;      // two quarters + the three factors
 
-template <bool HAS_Y>
+// NT: 0 = ordinary stores, 1 = non-temporal stores (1024 x 32^3: 85.0 -> 78.0 us; non-temporal loads of X: 81.6)
+template <bool HAS_Y, int NT>
 __global__ __launch_bounds__(512, 4) void kron_row32x3_kernel(const StepArgs a) {
   extern __shared__ __align__(16) float r32lds[];
   float* const fl = r32lds + 2 * kR32QuarterWords;                 // fl[j*1024 + p*32 + q]; j = 0: F3, 1: F2, 2: F1
@@ -165,7 +166,7 @@ __global__ __launch_bounds__(512, 4) void kron_row32x3_kernel(const StepArgs a) 
     for (int r = 0; r < 4; r++) {
       r3f4 o = (r3f4){D[0][r], D[1][r], D[2][r], D[3][r]} * alpha;
       if (HAS_Y) o = o + yv[r] * beta;
-      *(r3f4*)(Z + (col + r * 1024)) = o;
+      FK_ST(NT, o, (r3f4*)(Z + (col + r * 1024)));
     }
   };
 
@@ -199,20 +200,19 @@ hipError_t launchRow32x3(const StepArgs& a, hipStream_t stream) {
   static PerDeviceOnce attrOnce;
   const int devIdx = launchDeviceIndex();
   const size_t ldsBytes = kR32LdsWords * sizeof(float);
+  using Kernel = void (*)(const StepArgs);
+  static const Kernel kernels[2][2] = {{kron_row32x3_kernel<false, 0>, kron_row32x3_kernel<false, 1>},
+                                       {kron_row32x3_kernel<true, 0>, kron_row32x3_kernel<true, 1>}};
   if (!attrOnce.done(devIdx)) {
-    hipError_t e = hipFuncSetAttribute((const void*)kron_row32x3_kernel<true>,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes);
-    if (e != hipSuccess) return e;
-    e = hipFuncSetAttribute((const void*)kron_row32x3_kernel<false>,
-                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes);
-    if (e != hipSuccess) return e;
+    for (int y = 0; y < 2; y++)
+      for (int nt = 0; nt < 2; nt++) {
+        hipError_t e = hipFuncSetAttribute((const void*)kernels[y][nt], hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes);
+        if (e != hipSuccess) return e;
+      }
     attrOnce.mark(devIdx);
   }
   dim3 grid(a.M, a.batch), block(512);
-  if (a.y && a.epilogue)
-    hipLaunchKernelGGL(kron_row32x3_kernel<true>, grid, block, ldsBytes, stream, a);
-  else
-    hipLaunchKernelGGL(kron_row32x3_kernel<false>, grid, block, ldsBytes, stream, a);
+  hipLaunchKernelGGL(kernels[(a.y && a.epilogue) ? 1 : 0][a.stream_out ? 1 : 0], grid, block, ldsBytes, stream, a);
   return hipGetLastError();
 }
 
