@@ -86,7 +86,7 @@ static bool stepAnyCheck(const KernelInfo& k, const StepArgs& a) { return stepAn
 void registerGenericKernels(std::vector<KernelInfo>& out) {
   for (DType dt : {DType::F32, DType::F64}) {
     KernelInfo k{};
-    k.name = std::string("gekmm_hip_gfx950_256_") + (dt == DType::F32 ? "f" : "d") + "_anyxany_256x512_1_16xany_mfma16x16x4";
+    k.name = std::string("gekmm_hip_gfx950_512_") + (dt == DType::F32 ? "f" : "d") + "_anyxany_256x512_1_16xany_mfma16x16x4";
     k.dt = dt; k.P = 1; k.Q = 1; k.fused = 1; k.tileM = 0; k.tileK = 0; k.threads = 256; k.variant = 0;
     k.canRun = stepAnyCanRun; k.launch = stepAnyLaunch; k.check = stepAnyCheck;
     out.push_back(k);
