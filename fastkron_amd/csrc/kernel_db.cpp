@@ -194,6 +194,20 @@ static bool row32x3CanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo
 static hipError_t row32x3Launch(const KernelInfo&, const StepArgs& a, hipStream_t s) { return launchRow32x3(a, s); }
 static bool row32x3Check(const KernelInfo&, const StepArgs& a) { return row32x3Supported(a); }
 
+// ---- single-factor fp32 step for 64x64 and 128x128, whole-line accesses through LDS (variant 3: MKM, 4: KMM) ----
+static bool stepWideCanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
+                           const DeviceInfo&) {
+  const MMType mm = (k.variant == 4) ? MMType::KMM : MMType::MKM;
+  if (p.dt != DType::F32 || p.mm != mm || lo != hi) return false;
+  if (p.P[lo] != k.P || p.Q[lo] != k.Q) return false;
+  if (first && p.opX == 2) return false;
+  // whole tiles of 4096 input elements: slices of a row (MKM), columns of a slice (KMM)
+  const uint64_t TS = 4096 / k.P;
+  return mm == MMType::KMM ? p.M % TS == 0 : (p.colsBefore(hi) / k.P) % TS == 0;
+}
+static hipError_t stepWideLaunch(const KernelInfo&, const StepArgs& a, hipStream_t s) { return launchStepWide(a, s); }
+static bool stepWideCheck(const KernelInfo&, const StepArgs& a) { return stepWideSupported(a); }
+
 // ---- single-factor MFMA step (fp64 and fp32) ----
 static bool stepF64CanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
                           const DeviceInfo& dev) {
@@ -370,6 +384,18 @@ void registerRowKernels(std::vector<KernelInfo>& out) {
     kk.dt = DType::F64; kk.P = 64; kk.Q = 64; kk.fused = 1; kk.tileM = 64; kk.tileK = 64; kk.threads = 256; kk.variant = 2;
     kk.canRun = kmm64CanRun; kk.launch = kmm64Launch; kk.check = kmm64Check;
     out.push_back(kk);
+  }
+
+  for (uint32_t variant : {3u, 4u})
+  for (uint32_t P : {64u, 128u}) {
+    KernelInfo kw{};
+    const std::string ps = std::to_string(P), ts = std::to_string(4096 / P);
+    kw.name = std::string(variant == 4 ? "kmm" : "mkm") + "_hip_gfx950_256_f_" + ps + "x" + ps + "_" + ps + "x" + ps + "_1_" +
+              (variant == 4 ? ts + "x" + ps : "1x4096") + "_mfma16x16x4_NN_strided_0_3";
+    kw.dt = DType::F32; kw.P = P; kw.Q = P; kw.fused = 1; kw.tileM = variant == 4 ? 4096 / P : 1;
+    kw.tileK = variant == 4 ? P : 4096; kw.threads = 256; kw.variant = variant;
+    kw.canRun = stepWideCanRun; kw.launch = stepWideLaunch; kw.check = stepWideCheck;
+    out.push_back(kw);
   }
 
   // variant 1 = the same kernel on the KMM layout (tiles of 16 consecutive m)

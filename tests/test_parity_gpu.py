@@ -273,7 +273,8 @@ def test_misaligned_buffers_fall_back_to_the_generic_plan(fk):
 
 @pytest.mark.parametrize("which", ["x", "y", "z"])
 @pytest.mark.parametrize("M,Ps,dt", [(96, [16] * 4, np.float32), (16, [16] * 3, np.float32), (100, [32] * 3, np.float32),
-                                     (8, [64, 64], np.float64), (8, [32, 32], np.float32), (64, [64], np.float64)])
+                                     (8, [64, 64], np.float64), (8, [32, 32], np.float32), (64, [64], np.float64),
+                                     (4, [128, 128], np.float32), (6, [64, 64], np.float32)])
 def test_one_misaligned_operand_at_a_time(fk, which, M, Ps, dt):
     """X, Y or Z alone starts one element past a 256-byte boundary: kernels with 16-byte accesses to that operand
     must not be chosen, and the answer must still be right."""
@@ -753,3 +754,24 @@ def test_pair_kernel_with_factors_of_17_to_31(fk, M, Ps, launches, dt):
     check(fk, ko.MKM, M, Ps, Ps, dt, alpha=1.0, beta=0.0, seed=182, opFs=ko.OP_T)
     check(fk, ko.MKM, M, Ps, Ps, dt, alpha=1.0, beta=1.0, seed=183, batch=2)
     check(fk, ko.MKM, M, Ps, Ps, dt, alpha=2.0, beta=0.0, seed=184, integer=True)
+
+
+# ---- single steps with 64x64 / 128x128 fp32 factors on tiles of 4096 contiguous elements (both layouts) ----
+@pytest.mark.parametrize("mm,M,Ps,kw", [
+    (ko.MKM, 4, [128, 128], {}), (ko.MKM, 3, [64, 64], dict(alpha=1.5, beta=0.5)),
+    (ko.MKM, 5, [128, 128], dict(alpha=2.0, beta=-1.0, batch=2, opFs=ko.OP_T)), (ko.MKM, 2, [64, 64, 64], {}),
+    (ko.MKM, 1, [128, 128, 128], dict(beta=1.0)), (ko.MKM, 600, [128, 128], {}),
+    (ko.KMM, 64, [128, 128], {}), (ko.KMM, 128, [64, 64], dict(alpha=1.5, beta=0.5)),
+    (ko.KMM, 32, [128, 128], dict(alpha=2.0, beta=-1.0, batch=2, opFs=ko.OP_T)), (ko.KMM, 192, [64, 64, 64], {}),
+    (ko.KMM, 64, [128, 128], dict(batch=3, share_f=True, beta=1.0, share_y=True)),
+    (ko.MKM, 7, [128, 128], dict(use_temp2=False, beta=0.25))])
+def test_wide_step_kernel(fk, mm, M, Ps, kw):
+    check(fk, mm, M, Ps, Ps, np.float32, seed=71, **kw)
+    assert all("_1_1x4096_" in k or "_1_32x128_" in k or "_1_64x64_" in k for _, _, k in fk.last_plan()), fk.last_plan()
+
+
+@pytest.mark.parametrize("mm,M,Ps", [(ko.KMM, 16, [128, 128]), (ko.KMM, 48, [64, 64]), (ko.KMM, 100, [128, 128])])
+def test_wide_step_kernel_needs_whole_tiles(fk, mm, M, Ps):
+    """Fewer columns than a tile's 32 (64) in the KMM layout, or not a multiple of it: the streaming step runs."""
+    check(fk, mm, M, Ps, Ps, np.float32, seed=72, alpha=1.5, beta=0.5)
+    assert not any("_1_32x128_" in k or "_1_64x64_mfma16" in k for _, _, k in fk.last_plan()), fk.last_plan()
