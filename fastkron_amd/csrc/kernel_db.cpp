@@ -198,15 +198,15 @@ static bool row32x3Check(const KernelInfo&, const StepArgs& a) { return row32x3S
 static bool stepWideCanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
                            const DeviceInfo&) {
   const MMType mm = (k.variant == 4) ? MMType::KMM : MMType::MKM;
-  if (p.dt != DType::F32 || p.mm != mm || lo != hi) return false;
+  if (p.dt != k.dt || p.mm != mm || lo != hi) return false;
   if (p.P[lo] != k.P || p.Q[lo] != k.Q) return false;
   if (first && p.opX == 2) return false;
-  // whole tiles of 4096 input elements: slices of a row (MKM), columns of a slice (KMM)
-  const uint64_t TS = 4096 / k.P;
+  // whole tiles of 16 KB of input: slices of a row (MKM), columns of a slice (KMM)
+  const uint64_t TS = 16384 / dtypeSize(k.dt) / k.P;
   return mm == MMType::KMM ? p.M % TS == 0 : (p.colsBefore(hi) / k.P) % TS == 0;
 }
-static hipError_t stepWideLaunch(const KernelInfo&, const StepArgs& a, hipStream_t s) { return launchStepWide(a, s); }
-static bool stepWideCheck(const KernelInfo&, const StepArgs& a) { return stepWideSupported(a); }
+static hipError_t stepWideLaunch(const KernelInfo& k, const StepArgs& a, hipStream_t s) { return launchStepWide(a, k.dt, s); }
+static bool stepWideCheck(const KernelInfo& k, const StepArgs& a) { return stepWideSupported(a, k.dt); }
 
 // ---- single-factor MFMA step (fp64 and fp32) ----
 static bool stepF64CanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
@@ -387,13 +387,15 @@ void registerRowKernels(std::vector<KernelInfo>& out) {
   }
 
   for (uint32_t variant : {3u, 4u})
+  for (DType dt : {DType::F32, DType::F64})
   for (uint32_t P : {64u, 128u}) {
     KernelInfo kw{};
-    const std::string ps = std::to_string(P), ts = std::to_string(4096 / P);
-    kw.name = std::string(variant == 4 ? "kmm" : "mkm") + "_hip_gfx950_256_f_" + ps + "x" + ps + "_" + ps + "x" + ps + "_1_" +
-              (variant == 4 ? ts + "x" + ps : "1x4096") + "_mfma16x16x4_NN_strided_0_3";
-    kw.dt = DType::F32; kw.P = P; kw.Q = P; kw.fused = 1; kw.tileM = variant == 4 ? 4096 / P : 1;
-    kw.tileK = variant == 4 ? P : 4096; kw.threads = 256; kw.variant = variant;
+    const uint32_t E = 16384 / (uint32_t)dtypeSize(dt);
+    const std::string ps = std::to_string(P), ts = std::to_string(E / P);
+    kw.name = std::string(variant == 4 ? "kmm" : "mkm") + "_hip_gfx950_256_" + (dt == DType::F32 ? "f_" : "d_") + ps + "x" + ps +
+              "_" + ps + "x" + ps + "_1_" + (variant == 4 ? ts + "x" + ps : "1x" + std::to_string(E)) + "_mfma16x16x4lds_NN_strided_0_3";
+    kw.dt = dt; kw.P = P; kw.Q = P; kw.fused = 1; kw.tileM = variant == 4 ? E / P : 1;
+    kw.tileK = variant == 4 ? P : E; kw.threads = 256; kw.variant = variant;
     kw.canRun = stepWideCanRun; kw.launch = stepWideLaunch; kw.check = stepWideCheck;
     out.push_back(kw);
   }

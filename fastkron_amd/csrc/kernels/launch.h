@@ -80,9 +80,9 @@ hipError_t launchRow32x3(const StepArgs& a, hipStream_t stream);
 bool pairMfmaSupported(const StepArgs& a, DType dt);
 hipError_t launchPairMfma(const StepArgs& a, DType dt, hipStream_t stream);
 
-// One step with a 64x64 or 128x128 fp32 factor in the MKM layout, tiles of 4096 contiguous elements through LDS.
-bool stepWideSupported(const StepArgs& a);
-hipError_t launchStepWide(const StepArgs& a, hipStream_t stream);
+// One step with a 64x64 or 128x128 factor, either type and layout, tiles of 16 KB passed through LDS.
+bool stepWideSupported(const StepArgs& a, DType dt);
+hipError_t launchStepWide(const StepArgs& a, DType dt, hipStream_t stream);
 
 // One step with a 16x16 ... 128x128 factor on the matrix cores, fp64 or fp32, MKM or KMM layout.
 bool stepMfmaSupported(const StepArgs& a, DType dt);

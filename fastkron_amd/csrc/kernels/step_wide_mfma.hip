@@ -1,5 +1,5 @@
-// One sliced-multiply step with a square fp32 factor of 64x64 or 128x128, MKM or KMM layout, every global access a
-// whole 128-byte line or more.
+// One sliced-multiply step with a square factor of 64x64 or 128x128, fp32 or fp64, MKM or KMM layout, every global
+// access a whole 128-byte line or more.
 //
 //   MKM  out[m, q*S + s] = sum_p in[m, s*P + p] * F[p, q]          S = Kin / P
 //   KMM  out[(q*S + s), m] = sum_p in[(s*P + p), m] * F[p, q]      (the M index contiguous)
@@ -7,18 +7,18 @@
 // The streaming step kernel (step_mfma.hip) gives a wave 16 slices and lets every lane read its own 16-byte pieces
 // and write 4-byte elements: its load instructions touch 64 lines each and its stores write 64-byte halves of lines,
 // which costs a third of the time once the operands are far larger than the caches (sgemkm 320 x 128^3: 6.3 ms
-// against 4.4 ms here; 1024 x 128^2: 120 against 85 us).  Here a workgroup of four waves owns a tile of 4096 input
-// elements: in the MKM layout TS = 4096/P consecutive slices of a row (contiguous), in the KMM layout the P rows
-// of a slice by TS consecutive columns m.
+// against 4.4 ms here; 1024 x 128^2: 120 against 85 us).  Here a workgroup of four waves owns a tile of 16 KB of input
+// (E = 4096 fp32 or 2048 fp64 elements): in the MKM layout TS = E/P consecutive slices of a row (contiguous), in the
+// KMM layout the P rows of a slice by TS consecutive columns m.
 //   * The tile is read with 16-byte accesses, consecutive lanes on consecutive addresses, one tile ahead into
 //     registers, and passed on through LDS (two buffers, one barrier per tile).
 //   * Wave w owns the output columns q in [w*P/4, (w+1)*P/4): its part of the factor stays in registers as the A
-//     operands of V_MFMA_F32_16X16X4_F32, D[q][j] += F^T[q][p] * X^T[p][j].  The 16 columns j of product e are the
+//     operands of V_MFMA_F32_16X16X4_F32 / V_MFMA_F64_16X16X4_F64, D[q][j] += F^T[q][p] * X^T[p][j].  The 16 columns j of product e are the
 //     slices (MKM) or columns m (KMM) JH*lane + e, JH = TS/16: a lane's results for one q are then JH consecutive
-//     output elements, and 16 lanes store 128 (128x128) or 256 (64x64) contiguous bytes.
+//     output elements, and 16 lanes store 128 (128x128) or 256 (64x64) contiguous bytes in either type.
 //   * MKM: the contraction index of product c in lane group k is p = (P/4)*k + c, so a lane's B operands are P/4
-//     consecutive elements of its slice, read from LDS 16 bytes at a time; 16-byte chunk `ch` of slice `s` sits at
-//     chunk s*(P/4) + (ch ^ ((s / JH) % 16)), which keeps the writers, eight lanes with consecutive chunks, and the
+//     consecutive elements of its slice, read from LDS 16 bytes at a time; 16-byte chunk `ch` of slice `s` (of CPS
+//     chunks) sits at chunk s*CPS + (ch ^ ((s / JH) % 16)), which keeps the writers, eight lanes with consecutive chunks, and the
 //     readers, sixteen lanes with the same chunk of slices JH apart, on distinct banks.
 //     KMM: p = 4*c + k, a lane reads its JH consecutive columns of row p; rows are TS elements apart, which puts
 //     the lane groups of one read on distinct banks without padding.
@@ -37,25 +37,56 @@ namespace fk {
 
 typedef float swf4 __attribute__((ext_vector_type(4)));
 typedef float swf2 __attribute__((ext_vector_type(2)));
+typedef double swd2 __attribute__((ext_vector_type(2)));
+typedef double swd4 __attribute__((ext_vector_type(4)));
 
-constexpr int kSwTile = 4096;                 // input elements per tile
+constexpr int kSwTileBytes = 16384;           // input bytes per tile
 constexpr int kSwWaves = 4;
-constexpr size_t kSwLdsBytes = 2 * kSwTile * sizeof(float);
+constexpr size_t kSwLdsBytes = 2 * kSwTileBytes;
 
-template <int JH> struct SwVec;
-template <> struct SwVec<4> { using type = swf4; };
-template <> struct SwVec<2> { using type = swf2; };
+template <typename T> struct SwType;
+template <> struct SwType<float> {
+  using Acc = swf4;
+  using Chunk = swf4;                          // 16 bytes
+  static __device__ __forceinline__ Acc mma(float a, float b, Acc c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
+  static __device__ __forceinline__ int row(int r, int hi) { return 4 * hi + r; }   // row of accumulator register r
+};
+template <> struct SwType<double> {
+  using Acc = swd4;
+  using Chunk = swd2;
+  static __device__ __forceinline__ Acc mma(double a, double b, Acc c) { return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0); }
+  static __device__ __forceinline__ int row(int r, int hi) { return 4 * r + hi; }
+};
+// JH consecutive output elements of a lane
+template <typename T, int JH> struct SwVec { typedef T type __attribute__((ext_vector_type(JH))); };
+template <typename T> struct SwVec<T, 1> { using type = T; };
+template <typename V, int JH> struct SwLane {
+  template <typename T> static __device__ __forceinline__ T get(const V& v, int e) { return v[e]; }
+  template <typename T> static __device__ __forceinline__ void set(V& v, int e, T x) { v[e] = x; }
+};
+template <typename V> struct SwLane<V, 1> {
+  template <typename T> static __device__ __forceinline__ T get(const V& v, int) { return v; }
+  template <typename T> static __device__ __forceinline__ void set(V& v, int, T x) { v = x; }
+};
 
-template <int P, bool KMM, bool HAS_Y>
+template <typename T, int P, bool KMM, bool HAS_Y>
 __global__ __launch_bounds__(256, 2) void kron_step_wide_kernel(const StepArgs a, const uint32_t tilesPerLine,
                                                                 const uint32_t totalTiles) {
-  constexpr int PC = P / 4;                   // products per column block; 16-byte chunks per slice (MKM)
-  constexpr int TS = kSwTile / P;             // slices (MKM) or columns m (KMM) per tile
+  using ST = SwType<T>;
+  using Acc = typename ST::Acc;
+  using Chunk = typename ST::Chunk;
+  constexpr int EPC = 16 / sizeof(T);         // elements per 16-byte chunk
+  constexpr int E = kSwTileBytes / sizeof(T); // elements per tile
+  constexpr int PC = P / 4;                   // products per column block, elements per lane and slice
+  constexpr int CPS = P / EPC;                // 16-byte chunks per slice (MKM)
+  constexpr int TS = E / P;                   // slices (MKM) or columns m (KMM) per tile
   constexpr int JH = TS / 16;                 // column blocks per tile = consecutive output elements per lane and q
   constexpr int NBW = P / 64;                 // 16-column blocks of the factor per wave
   constexpr int RW = 16 * NBW;                // output columns q per wave
-  using Vec = typename SwVec<JH>::type;
-  extern __shared__ __align__(16) float swLds[];
+  using Vec = typename SwVec<T, JH>::type;
+  using VL = SwLane<Vec, JH>;
+  extern __shared__ __align__(16) unsigned char swLdsRaw[];
+  T* swLds = (T*)swLdsRaw;
   const int tid = threadIdx.x;
   const int l = tid & 63;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -63,15 +94,15 @@ __global__ __launch_bounds__(256, 2) void kron_step_wide_kernel(const StepArgs a
   const uint32_t bt = blockIdx.y;
   const uint64_t S = a.Kin / P;
 
-  const float* inB = (const float*)a.in + (size_t)bt * a.in_batch;
-  float* outB = (float*)a.out + (size_t)bt * a.out_batch;
-  const float* YB = HAS_Y ? (const float*)a.y + (size_t)bt * a.y_batch : nullptr;
-  const float alpha = a.epilogue ? (float)a.alpha : 1.f, beta = (float)a.beta;   // multiplying by 1 is exact
+  const T* inB = (const T*)a.in + (size_t)bt * a.in_batch;
+  T* outB = (T*)a.out + (size_t)bt * a.out_batch;
+  const T* YB = HAS_Y ? (const T*)a.y + (size_t)bt * a.y_batch : nullptr;
+  const T alpha = a.epilogue ? (T)a.alpha : (T)1, beta = (T)a.beta;   // multiplying by 1 is exact
 
   // this wave's columns of the factor as A operands: fa[c][ib] = F[p(c, hi)][RW*w + 16*ib + lo]
-  float fa[PC][NBW];
+  T fa[PC][NBW];
   {
-    const float* F = (const float*)a.f[0] + (size_t)bt * a.f_batch[0];
+    const T* F = (const T*)a.f[0] + (size_t)bt * a.f_batch[0];
 #pragma unroll
     for (int c = 0; c < PC; c++)
 #pragma unroll
@@ -82,84 +113,83 @@ __global__ __launch_bounds__(256, 2) void kron_step_wide_kernel(const StepArgs a
   }
 
   // tile t: MKM row t / tilesPerLine, slices TS*(t % tilesPerLine) ...; KMM slice t / tilesPerLine, columns likewise
-  swf4 pre[4];
+  Chunk pre[4];
   auto request = [&](uint32_t t) {
     const size_t line = t / tilesPerLine, part = t % tilesPerLine;
 #pragma unroll
     for (int i = 0; i < 4; i++) {
       const int g = 256 * i + tid;                             // 16-byte chunk of the tile
       if (KMM) {
-        const int p = g / (TS / 4), ch = g % (TS / 4);
-        pre[i] = *(const swf4*)(inB + (line * P + p) * (size_t)a.in_ldc + part * TS + 4 * ch);
+        const int p = g / (TS / EPC), ch = g % (TS / EPC);
+        pre[i] = *(const Chunk*)(inB + (line * P + p) * (size_t)a.in_ldc + part * TS + EPC * ch);
       } else {
-        pre[i] = *(const swf4*)(inB + line * (size_t)a.in_ldm + part * kSwTile + 4 * g);
+        pre[i] = *(const Chunk*)(inB + line * (size_t)a.in_ldm + part * E + EPC * g);
       }
     }
   };
   auto nextOf = [&](uint32_t t) { return t + gridDim.x < totalTiles ? t + gridDim.x : t; };
 
   auto computeTile = [&](uint32_t t, int buf) {
-    float* xs = swLds + buf * kSwTile;
+    T* xs = swLds + buf * E;
 #pragma unroll
     for (int i = 0; i < 4; i++) {
       const int g = 256 * i + tid;
       if (KMM) {
-        *(swf4*)&xs[4 * g] = pre[i];                           // row p = g / (TS/4), TS elements per row
+        *(Chunk*)&xs[EPC * g] = pre[i];                        // row p = g / (TS/EPC), TS elements per row
       } else {
-        const int s = g / PC, ch = g % PC;
-        *(swf4*)&xs[4 * (s * PC + (ch ^ ((s / JH) & 15)))] = pre[i];
+        const int s = g / CPS, ch = g % CPS;
+        *(Chunk*)&xs[EPC * (s * CPS + (ch ^ ((s / JH) & 15)))] = pre[i];
       }
     }
     request(nextOf(t));                                        // the next tile streams in under the products
     __syncthreads();
     // B operands: x[e][c] = X[p(c, hi)][column JH*lo + e]
-    float x[JH][PC];
+    T x[JH][PC];
     if (KMM) {
 #pragma unroll
       for (int c = 0; c < PC; c++) {
         const Vec v = *(const Vec*)&xs[(4 * c + hi) * TS + JH * lo];
 #pragma unroll
-        for (int e = 0; e < JH; e++) x[e][c] = v[e];
+        for (int e = 0; e < JH; e++) x[e][c] = VL::template get<T>(v, e);
       }
     } else {
 #pragma unroll
       for (int e = 0; e < JH; e++)
 #pragma unroll
-        for (int c4 = 0; c4 < PC / 4; c4++) {
-          const int ch = (PC / 4) * hi + c4;
-          const swf4 v = *(const swf4*)&xs[4 * ((JH * lo + e) * PC + (ch ^ lo))];
+        for (int c4 = 0; c4 < PC / EPC; c4++) {
+          const int ch = (PC / EPC) * hi + c4;
+          const Chunk v = *(const Chunk*)&xs[EPC * ((JH * lo + e) * CPS + (ch ^ lo))];
 #pragma unroll
-          for (int k = 0; k < 4; k++) x[e][4 * c4 + k] = v[k];
+          for (int k = 0; k < EPC; k++) x[e][EPC * c4 + k] = v[k];
         }
     }
 
-    swf4 acc[NBW][JH];
+    Acc acc[NBW][JH];
 #pragma unroll
     for (int ib = 0; ib < NBW; ib++)
 #pragma unroll
-      for (int e = 0; e < JH; e++) acc[ib][e] = (swf4){0.f, 0.f, 0.f, 0.f};
+      for (int e = 0; e < JH; e++) acc[ib][e] = (Acc){0, 0, 0, 0};
 #pragma unroll
     for (int c = 0; c < PC; c++)
 #pragma unroll
       for (int ib = 0; ib < NBW; ib++)
 #pragma unroll
-        for (int e = 0; e < JH; e++)
-          acc[ib][e] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[c][ib], x[e][c], acc[ib][e], 0, 0, 0);
+        for (int e = 0; e < JH; e++) acc[ib][e] = ST::mma(fa[c][ib], x[e][c], acc[ib][e]);
 
-    // accumulator register r of lane (hi, lo) and product e: output column q = RW*w + 16*ib + 4*hi + r, element
+    // accumulator register r of lane (hi, lo) and product e: output column q = RW*w + 16*ib + row(r, hi), element
     // JH*lo + e of the tile's TS
     const size_t line = t / tilesPerLine, part = t % tilesPerLine;
     const size_t qStride = KMM ? S * (size_t)a.out_ldc : S, yStride = KMM ? S * (size_t)a.y_ldc : S;
-    float* out = KMM ? outB + line * (size_t)a.out_ldc + part * TS + JH * lo
-                     : outB + line * (size_t)a.out_ldm + part * TS + JH * lo;
-    const float* Y = nullptr;
+    T* out = KMM ? outB + line * (size_t)a.out_ldc + part * TS + JH * lo
+                 : outB + line * (size_t)a.out_ldm + part * TS + JH * lo;
+    const T* Y = nullptr;
     if (HAS_Y) Y = KMM ? YB + line * (size_t)a.y_ldc + part * TS + JH * lo : YB + line * (size_t)a.y_ldm + part * TS + JH * lo;
     Vec yv[NBW][4];
     if (HAS_Y) {
 #pragma unroll
       for (int ib = 0; ib < NBW; ib++)
 #pragma unroll
-        for (int r = 0; r < 4; r++) yv[ib][r] = *(const Vec*)(Y + (size_t)(RW * w + 16 * ib + 4 * hi + r) * yStride);
+        for (int r = 0; r < 4; r++) yv[ib][r] = *(const Vec*)(Y + (size_t)(RW * w + 16 * ib + ST::row(r, hi)) * yStride);
     }
 #pragma unroll
     for (int ib = 0; ib < NBW; ib++)
@@ -167,9 +197,9 @@ __global__ __launch_bounds__(256, 2) void kron_step_wide_kernel(const StepArgs a
       for (int r = 0; r < 4; r++) {
         Vec v;
 #pragma unroll
-        for (int e = 0; e < JH; e++) v[e] = acc[ib][e][r] * alpha;
+        for (int e = 0; e < JH; e++) VL::template set<T>(v, e, acc[ib][e][r] * alpha);
         if (HAS_Y) v += yv[ib][r] * beta;
-        *(Vec*)(out + (size_t)(RW * w + 16 * ib + 4 * hi + r) * qStride) = v;
+        *(Vec*)(out + (size_t)(RW * w + 16 * ib + ST::row(r, hi)) * qStride) = v;
       }
   };
 
@@ -183,33 +213,33 @@ __global__ __launch_bounds__(256, 2) void kron_step_wide_kernel(const StepArgs a
 
 static bool stepWideIsKmm(const StepArgs& a) { return a.in_ldm == 1 && a.in_ldc != 1; }
 
-bool stepWideSupported(const StepArgs& a) {
+bool stepWideSupported(const StepArgs& a, DType dt) {
   if (a.nf != 1) return false;
   const uint32_t P = a.p[0];
   if ((P != 64 && P != 128) || a.q[0] != P) return false;
   if (a.Kin % P || a.Kout != a.Kin) return false;
-  const uint64_t S = a.Kin / P, TS = kSwTile / P;
+  const uint64_t es = dtypeSize(dt), E = kSwTileBytes / es, S = a.Kin / P, TS = E / P, vm = 16 / es - 1;
   if (stepWideIsKmm(a)) {
     if (a.out_ldm != 1 || (a.y && a.y_ldm != 1)) return false;
     if (a.M % TS) return false;                               // whole tiles
-    if (((uintptr_t)a.in & 15) || (a.in_ldc & 3) || (a.in_batch & 3)) return false;
-    if (((uintptr_t)a.out & 15) || (a.out_ldc & 3) || (a.out_batch & 3)) return false;
-    if (a.y && (((uintptr_t)a.y & 15) || (a.y_ldc & 3) || (a.y_batch & 3))) return false;
+    if (((uintptr_t)a.in & 15) || ((uint64_t)a.in_ldc & vm) || (a.in_batch & vm)) return false;
+    if (((uintptr_t)a.out & 15) || ((uint64_t)a.out_ldc & vm) || (a.out_batch & vm)) return false;
+    if (a.y && (((uintptr_t)a.y & 15) || ((uint64_t)a.y_ldc & vm) || (a.y_batch & vm))) return false;
     return S * (a.M / TS) < (1ull << 31) && a.batch <= 65535;
   }
   if (S % TS) return false;
   if (a.in_ldc != 1 || a.out_ldc != 1 || (a.y && a.y_ldc != 1)) return false;
   // 16-byte accesses: rows and batch entries start on 16-byte boundaries
-  if (((uintptr_t)a.in & 15) || (a.in_ldm & 3) || (a.in_batch & 3)) return false;
-  if (((uintptr_t)a.out & 15) || (a.out_ldm & 3) || (a.out_batch & 3)) return false;
-  if (a.y && (((uintptr_t)a.y & 15) || (a.y_ldm & 3) || (a.y_batch & 3))) return false;
-  return (a.Kin / kSwTile) * a.M < (1ull << 31) && a.batch <= 65535;
+  if (((uintptr_t)a.in & 15) || ((uint64_t)a.in_ldm & vm) || (a.in_batch & vm)) return false;
+  if (((uintptr_t)a.out & 15) || ((uint64_t)a.out_ldm & vm) || (a.out_batch & vm)) return false;
+  if (a.y && (((uintptr_t)a.y & 15) || ((uint64_t)a.y_ldm & vm) || (a.y_batch & vm))) return false;
+  return (a.Kin / E) * a.M < (1ull << 31) && a.batch <= 65535;
 }
 
-template <int P, bool KMM>
+template <typename T, int P, bool KMM>
 static hipError_t launchStepWideT(const StepArgs& a, hipStream_t stream) {
-  const uint32_t TS = kSwTile / P;
-  const uint32_t tilesPerLine = KMM ? a.M / TS : (uint32_t)(a.Kin / kSwTile);
+  const uint32_t E = kSwTileBytes / sizeof(T), TS = E / P;
+  const uint32_t tilesPerLine = KMM ? a.M / TS : (uint32_t)(a.Kin / E);
   const uint32_t totalTiles = KMM ? (uint32_t)(a.Kin / P) * tilesPerLine : tilesPerLine * a.M;
   uint32_t wgs = 2u * (uint32_t)deviceCUs();                   // persistent, two workgroups per CU
   if (a.batch > 1) wgs = (wgs + a.batch - 1) / a.batch;
@@ -217,16 +247,21 @@ static hipError_t launchStepWideT(const StepArgs& a, hipStream_t stream) {
   if (wgs == 0) wgs = 1;
   dim3 grid(wgs, a.batch), block(64 * kSwWaves);
   if (a.y && a.epilogue)
-    hipLaunchKernelGGL((kron_step_wide_kernel<P, KMM, true>), grid, block, kSwLdsBytes, stream, a, tilesPerLine, totalTiles);
+    hipLaunchKernelGGL((kron_step_wide_kernel<T, P, KMM, true>), grid, block, kSwLdsBytes, stream, a, tilesPerLine, totalTiles);
   else
-    hipLaunchKernelGGL((kron_step_wide_kernel<P, KMM, false>), grid, block, kSwLdsBytes, stream, a, tilesPerLine, totalTiles);
+    hipLaunchKernelGGL((kron_step_wide_kernel<T, P, KMM, false>), grid, block, kSwLdsBytes, stream, a, tilesPerLine, totalTiles);
   return hipGetLastError();
 }
 
-hipError_t launchStepWide(const StepArgs& a, hipStream_t stream) {
-  if (!stepWideSupported(a)) return hipErrorInvalidValue;
-  if (stepWideIsKmm(a)) return a.p[0] == 128 ? launchStepWideT<128, true>(a, stream) : launchStepWideT<64, true>(a, stream);
-  return a.p[0] == 128 ? launchStepWideT<128, false>(a, stream) : launchStepWideT<64, false>(a, stream);
+template <typename T>
+static hipError_t launchStepWideD(const StepArgs& a, hipStream_t stream) {
+  if (stepWideIsKmm(a)) return a.p[0] == 128 ? launchStepWideT<T, 128, true>(a, stream) : launchStepWideT<T, 64, true>(a, stream);
+  return a.p[0] == 128 ? launchStepWideT<T, 128, false>(a, stream) : launchStepWideT<T, 64, false>(a, stream);
+}
+
+hipError_t launchStepWide(const StepArgs& a, DType dt, hipStream_t stream) {
+  if (!stepWideSupported(a, dt)) return hipErrorInvalidValue;
+  return dt == DType::F32 ? launchStepWideD<float>(a, stream) : launchStepWideD<double>(a, stream);
 }
 
 }  // namespace fk

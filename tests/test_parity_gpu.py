@@ -765,13 +765,18 @@ def test_pair_kernel_with_factors_of_17_to_31(fk, M, Ps, launches, dt):
     (ko.KMM, 32, [128, 128], dict(alpha=2.0, beta=-1.0, batch=2, opFs=ko.OP_T)), (ko.KMM, 192, [64, 64, 64], {}),
     (ko.KMM, 64, [128, 128], dict(batch=3, share_f=True, beta=1.0, share_y=True)),
     (ko.MKM, 7, [128, 128], dict(use_temp2=False, beta=0.25))])
-def test_wide_step_kernel(fk, mm, M, Ps, kw):
-    check(fk, mm, M, Ps, Ps, np.float32, seed=71, **kw)
-    assert all("_1_1x4096_" in k or "_1_32x128_" in k or "_1_64x64_" in k for _, _, k in fk.last_plan()), fk.last_plan()
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_wide_step_kernel(fk, mm, M, Ps, kw, dt):
+    if dt == np.float64 and mm == ko.KMM:
+        M = M // 2                      # fp64 tiles hold half as many columns
+    check(fk, mm, M, Ps, Ps, dt, seed=71, **kw)
+    if dt == np.float64 and Ps[0] == 64 and mm == ko.KMM:
+        return                          # the 4x4x4 KMM step is preferred for fp64 64x64
+    assert all("mfma16x16x4lds" in k for _, _, k in fk.last_plan()), fk.last_plan()
 
 
 @pytest.mark.parametrize("mm,M,Ps", [(ko.KMM, 16, [128, 128]), (ko.KMM, 48, [64, 64]), (ko.KMM, 100, [128, 128])])
 def test_wide_step_kernel_needs_whole_tiles(fk, mm, M, Ps):
     """Fewer columns than a tile's 32 (64) in the KMM layout, or not a multiple of it: the streaming step runs."""
     check(fk, mm, M, Ps, Ps, np.float32, seed=72, alpha=1.5, beta=0.5)
-    assert not any("_1_32x128_" in k or "_1_64x64_mfma16" in k for _, _, k in fk.last_plan()), fk.last_plan()
+    assert not any("mfma16x16x4lds" in k for _, _, k in fk.last_plan()), fk.last_plan()
