@@ -388,7 +388,7 @@ void registerRowKernels(std::vector<KernelInfo>& out) {
 
   for (uint32_t variant : {3u, 4u})
   for (DType dt : {DType::F32, DType::F64})
-  for (uint32_t P : {64u, 128u}) {
+  for (uint32_t P : {32u, 64u, 128u}) {
     KernelInfo kw{};
     const uint32_t E = 16384 / (uint32_t)dtypeSize(dt);
     const std::string ps = std::to_string(P), ts = std::to_string(E / P);

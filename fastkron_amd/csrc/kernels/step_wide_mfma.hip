@@ -18,7 +18,7 @@
 //     output elements, and 16 lanes store 128 (128x128) or 256 (64x64) contiguous bytes in either type.
 //   * MKM: the contraction index of product c in lane group k is p = (P/4)*k + c, so a lane's B operands are P/4
 //     consecutive elements of its slice, read from LDS 16 bytes at a time; 16-byte chunk `ch` of slice `s` (of CPS
-//     chunks) sits at chunk s*CPS + (ch ^ ((s / JH) % 16)), which keeps the writers, eight lanes with consecutive chunks, and the
+//     chunks) sits at chunk s*CPS + (ch ^ ((s / JH) % min(CPS, 16))), which keeps the writers, eight lanes with consecutive chunks, and the
 //     readers, sixteen lanes with the same chunk of slices JH apart, on distinct banks.
 //     KMM: p = 4*c + k, a lane reads its JH consecutive columns of row p; rows are TS elements apart, which puts
 //     the lane groups of one read on distinct banks without padding.
@@ -69,6 +69,11 @@ template <typename V> struct SwLane<V, 1> {
   template <typename T> static __device__ __forceinline__ void set(V& v, int, T x) { v = x; }
 };
 
+// MKM tiles in LDS: slice s of CPS 16-byte chunks.  With 8 chunks per slice the sixteen lanes of a read (slices 4
+// apart) would meet on two bank groups of eight: slices 32 apart swap places with their neighbours, which moves the
+// upper eight lanes to the other group.
+template <int CPS> __device__ __forceinline__ int swSlot(int s) { return CPS < 16 ? s ^ ((s >> 5) & 1) : s; }
+
 template <typename T, int P, bool KMM, bool HAS_Y>
 __global__ __launch_bounds__(256, 2) void kron_step_wide_kernel(const StepArgs a, const uint32_t tilesPerLine,
                                                                 const uint32_t totalTiles) {
@@ -80,9 +85,12 @@ __global__ __launch_bounds__(256, 2) void kron_step_wide_kernel(const StepArgs a
   constexpr int PC = P / 4;                   // products per column block, elements per lane and slice
   constexpr int CPS = P / EPC;                // 16-byte chunks per slice (MKM)
   constexpr int TS = E / P;                   // slices (MKM) or columns m (KMM) per tile
-  constexpr int JH = TS / 16;                 // column blocks per tile = consecutive output elements per lane and q
-  constexpr int NBW = P / 64;                 // 16-column blocks of the factor per wave
+  // the four waves split the factor's columns q into QG groups and the tile's TS slices / columns into JG parts
+  constexpr int QG = P >= 64 ? 4 : P / 16, JG = 4 / QG;
+  constexpr int JH = TS / 16 / JG;            // column blocks per wave = consecutive output elements per lane and q
+  constexpr int NBW = P / 16 / QG;            // 16-column blocks of the factor per wave
   constexpr int RW = 16 * NBW;                // output columns q per wave
+  constexpr int KEY = (CPS < 16 ? CPS : 16) - 1;
   using Vec = typename SwVec<T, JH>::type;
   using VL = SwLane<Vec, JH>;
   extern __shared__ __align__(16) unsigned char swLdsRaw[];
@@ -91,6 +99,7 @@ __global__ __launch_bounds__(256, 2) void kron_step_wide_kernel(const StepArgs a
   const int l = tid & 63;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lo = l & 15, hi = l >> 4;
+  const int qg = w % QG, j0 = (w / QG) * (TS / JG);            // this wave's column group and first slice / column
   const uint32_t bt = blockIdx.y;
   const uint64_t S = a.Kin / P;
 
@@ -99,7 +108,7 @@ __global__ __launch_bounds__(256, 2) void kron_step_wide_kernel(const StepArgs a
   const T* YB = HAS_Y ? (const T*)a.y + (size_t)bt * a.y_batch : nullptr;
   const T alpha = a.epilogue ? (T)a.alpha : (T)1, beta = (T)a.beta;   // multiplying by 1 is exact
 
-  // this wave's columns of the factor as A operands: fa[c][ib] = F[p(c, hi)][RW*w + 16*ib + lo]
+  // this wave's columns of the factor as A operands: fa[c][ib] = F[p(c, hi)][RW*qg + 16*ib + lo]
   T fa[PC][NBW];
   {
     const T* F = (const T*)a.f[0] + (size_t)bt * a.f_batch[0];
@@ -108,7 +117,7 @@ __global__ __launch_bounds__(256, 2) void kron_step_wide_kernel(const StepArgs a
 #pragma unroll
       for (int ib = 0; ib < NBW; ib++) {
         const int p = KMM ? 4 * c + hi : PC * hi + c;
-        fa[c][ib] = F[(int64_t)p * a.f_sp[0] + (int64_t)(RW * w + 16 * ib + lo) * a.f_sq[0]];
+        fa[c][ib] = F[(int64_t)p * a.f_sp[0] + (int64_t)(RW * qg + 16 * ib + lo) * a.f_sq[0]];
       }
   }
 
@@ -138,17 +147,17 @@ __global__ __launch_bounds__(256, 2) void kron_step_wide_kernel(const StepArgs a
         *(Chunk*)&xs[EPC * g] = pre[i];                        // row p = g / (TS/EPC), TS elements per row
       } else {
         const int s = g / CPS, ch = g % CPS;
-        *(Chunk*)&xs[EPC * (s * CPS + (ch ^ ((s / JH) & 15)))] = pre[i];
+        *(Chunk*)&xs[EPC * (swSlot<CPS>(s) * CPS + (ch ^ ((s / JH) & KEY)))] = pre[i];
       }
     }
     request(nextOf(t));                                        // the next tile streams in under the products
     __syncthreads();
-    // B operands: x[e][c] = X[p(c, hi)][column JH*lo + e]
+    // B operands: x[e][c] = X[p(c, hi)][column j0 + JH*lo + e]
     T x[JH][PC];
     if (KMM) {
 #pragma unroll
       for (int c = 0; c < PC; c++) {
-        const Vec v = *(const Vec*)&xs[(4 * c + hi) * TS + JH * lo];
+        const Vec v = *(const Vec*)&xs[(4 * c + hi) * TS + j0 + JH * lo];
 #pragma unroll
         for (int e = 0; e < JH; e++) x[e][c] = VL::template get<T>(v, e);
       }
@@ -158,7 +167,7 @@ __global__ __launch_bounds__(256, 2) void kron_step_wide_kernel(const StepArgs a
 #pragma unroll
         for (int c4 = 0; c4 < PC / EPC; c4++) {
           const int ch = (PC / EPC) * hi + c4;
-          const Chunk v = *(const Chunk*)&xs[EPC * ((JH * lo + e) * CPS + (ch ^ lo))];
+          const Chunk v = *(const Chunk*)&xs[EPC * (swSlot<CPS>(j0 + JH * lo + e) * CPS + (ch ^ (lo & KEY)))];
 #pragma unroll
           for (int k = 0; k < EPC; k++) x[e][EPC * c4 + k] = v[k];
         }
@@ -176,20 +185,20 @@ __global__ __launch_bounds__(256, 2) void kron_step_wide_kernel(const StepArgs a
 #pragma unroll
         for (int e = 0; e < JH; e++) acc[ib][e] = ST::mma(fa[c][ib], x[e][c], acc[ib][e]);
 
-    // accumulator register r of lane (hi, lo) and product e: output column q = RW*w + 16*ib + row(r, hi), element
-    // JH*lo + e of the tile's TS
+    // accumulator register r of lane (hi, lo) and product e: output column q = RW*qg + 16*ib + row(r, hi), element
+    // j0 + JH*lo + e of the tile's TS
     const size_t line = t / tilesPerLine, part = t % tilesPerLine;
     const size_t qStride = KMM ? S * (size_t)a.out_ldc : S, yStride = KMM ? S * (size_t)a.y_ldc : S;
-    T* out = KMM ? outB + line * (size_t)a.out_ldc + part * TS + JH * lo
-                 : outB + line * (size_t)a.out_ldm + part * TS + JH * lo;
+    T* out = KMM ? outB + line * (size_t)a.out_ldc + part * TS + j0 + JH * lo
+                 : outB + line * (size_t)a.out_ldm + part * TS + j0 + JH * lo;
     const T* Y = nullptr;
-    if (HAS_Y) Y = KMM ? YB + line * (size_t)a.y_ldc + part * TS + JH * lo : YB + line * (size_t)a.y_ldm + part * TS + JH * lo;
+    if (HAS_Y) Y = KMM ? YB + line * (size_t)a.y_ldc + part * TS + j0 + JH * lo : YB + line * (size_t)a.y_ldm + part * TS + j0 + JH * lo;
     Vec yv[NBW][4];
     if (HAS_Y) {
 #pragma unroll
       for (int ib = 0; ib < NBW; ib++)
 #pragma unroll
-        for (int r = 0; r < 4; r++) yv[ib][r] = *(const Vec*)(Y + (size_t)(RW * w + 16 * ib + ST::row(r, hi)) * yStride);
+        for (int r = 0; r < 4; r++) yv[ib][r] = *(const Vec*)(Y + (size_t)(RW * qg + 16 * ib + ST::row(r, hi)) * yStride);
     }
 #pragma unroll
     for (int ib = 0; ib < NBW; ib++)
@@ -199,7 +208,7 @@ __global__ __launch_bounds__(256, 2) void kron_step_wide_kernel(const StepArgs a
 #pragma unroll
         for (int e = 0; e < JH; e++) VL::template set<T>(v, e, acc[ib][e][r] * alpha);
         if (HAS_Y) v += yv[ib][r] * beta;
-        *(Vec*)(out + (size_t)(RW * w + 16 * ib + ST::row(r, hi)) * qStride) = v;
+        *(Vec*)(out + (size_t)(RW * qg + 16 * ib + ST::row(r, hi)) * qStride) = v;
       }
   };
 
@@ -216,7 +225,7 @@ static bool stepWideIsKmm(const StepArgs& a) { return a.in_ldm == 1 && a.in_ldc 
 bool stepWideSupported(const StepArgs& a, DType dt) {
   if (a.nf != 1) return false;
   const uint32_t P = a.p[0];
-  if ((P != 64 && P != 128) || a.q[0] != P) return false;
+  if ((P != 32 && P != 64 && P != 128) || a.q[0] != P) return false;
   if (a.Kin % P || a.Kout != a.Kin) return false;
   const uint64_t es = dtypeSize(dt), E = kSwTileBytes / es, S = a.Kin / P, TS = E / P, vm = 16 / es - 1;
   if (stepWideIsKmm(a)) {
@@ -241,7 +250,17 @@ static hipError_t launchStepWideT(const StepArgs& a, hipStream_t stream) {
   const uint32_t E = kSwTileBytes / sizeof(T), TS = E / P;
   const uint32_t tilesPerLine = KMM ? a.M / TS : (uint32_t)(a.Kin / E);
   const uint32_t totalTiles = KMM ? (uint32_t)(a.Kin / P) * tilesPerLine : tilesPerLine * a.M;
-  uint32_t wgs = 2u * (uint32_t)deviceCUs();                   // persistent, two workgroups per CU
+  // persistent workgroups, as many per CU as registers and LDS allow (two for 128x128, more for the smaller factors)
+  static std::atomic<int> occCache[kMaxDevices];
+  const int devIdx = launchDeviceIndex();
+  int occ = occCache[devIdx].load(std::memory_order_relaxed);
+  if (occ == 0) {
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, (const void*)kron_step_wide_kernel<T, P, KMM, false>, 64 * kSwWaves,
+                                                     kSwLdsBytes) != hipSuccess || occ < 1) occ = 2;
+    if (occ > 4) occ = 4;
+    occCache[devIdx].store(occ, std::memory_order_relaxed);
+  }
+  uint32_t wgs = (uint32_t)occ * (uint32_t)deviceCUs();
   if (a.batch > 1) wgs = (wgs + a.batch - 1) / a.batch;
   if (wgs > totalTiles) wgs = totalTiles;
   if (wgs == 0) wgs = 1;
@@ -255,8 +274,12 @@ static hipError_t launchStepWideT(const StepArgs& a, hipStream_t stream) {
 
 template <typename T>
 static hipError_t launchStepWideD(const StepArgs& a, hipStream_t stream) {
-  if (stepWideIsKmm(a)) return a.p[0] == 128 ? launchStepWideT<T, 128, true>(a, stream) : launchStepWideT<T, 64, true>(a, stream);
-  return a.p[0] == 128 ? launchStepWideT<T, 128, false>(a, stream) : launchStepWideT<T, 64, false>(a, stream);
+  const uint32_t P = a.p[0];
+  if (stepWideIsKmm(a))
+    return P == 128 ? launchStepWideT<T, 128, true>(a, stream) : P == 64 ? launchStepWideT<T, 64, true>(a, stream)
+                                                                         : launchStepWideT<T, 32, true>(a, stream);
+  return P == 128 ? launchStepWideT<T, 128, false>(a, stream) : P == 64 ? launchStepWideT<T, 64, false>(a, stream)
+                                                                        : launchStepWideT<T, 32, false>(a, stream);
 }
 
 hipError_t launchStepWide(const StepArgs& a, DType dt, hipStream_t stream) {

@@ -756,7 +756,7 @@ def test_pair_kernel_with_factors_of_17_to_31(fk, M, Ps, launches, dt):
     check(fk, ko.MKM, M, Ps, Ps, dt, alpha=2.0, beta=0.0, seed=184, integer=True)
 
 
-# ---- single steps with 64x64 / 128x128 fp32 factors on tiles of 4096 contiguous elements (both layouts) ----
+# ---- single steps with 32x32 / 64x64 / 128x128 factors on tiles of 16 KB passed through LDS (both layouts and types) ----
 @pytest.mark.parametrize("mm,M,Ps,kw", [
     (ko.MKM, 4, [128, 128], {}), (ko.MKM, 3, [64, 64], dict(alpha=1.5, beta=0.5)),
     (ko.MKM, 5, [128, 128], dict(alpha=2.0, beta=-1.0, batch=2, opFs=ko.OP_T)), (ko.MKM, 2, [64, 64, 64], {}),
@@ -764,7 +764,8 @@ def test_pair_kernel_with_factors_of_17_to_31(fk, M, Ps, launches, dt):
     (ko.KMM, 64, [128, 128], {}), (ko.KMM, 128, [64, 64], dict(alpha=1.5, beta=0.5)),
     (ko.KMM, 32, [128, 128], dict(alpha=2.0, beta=-1.0, batch=2, opFs=ko.OP_T)), (ko.KMM, 192, [64, 64, 64], {}),
     (ko.KMM, 64, [128, 128], dict(batch=3, share_f=True, beta=1.0, share_y=True)),
-    (ko.MKM, 7, [128, 128], dict(use_temp2=False, beta=0.25))])
+    (ko.MKM, 7, [128, 128], dict(use_temp2=False, beta=0.25)),
+    (ko.KMM, 256, [32, 32], dict(alpha=1.5, beta=0.5)), (ko.KMM, 128, [32, 32, 32], dict(batch=2, opFs=ko.OP_T, beta=1.0))])
 @pytest.mark.parametrize("dt", [np.float32, np.float64])
 def test_wide_step_kernel(fk, mm, M, Ps, kw, dt):
     if dt == np.float64 and mm == ko.KMM:
@@ -775,8 +776,9 @@ def test_wide_step_kernel(fk, mm, M, Ps, kw, dt):
     assert all("mfma16x16x4lds" in k for _, _, k in fk.last_plan()), fk.last_plan()
 
 
-@pytest.mark.parametrize("mm,M,Ps", [(ko.KMM, 16, [128, 128]), (ko.KMM, 48, [64, 64]), (ko.KMM, 100, [128, 128])])
+@pytest.mark.parametrize("mm,M,Ps", [(ko.KMM, 16, [128, 128]), (ko.KMM, 48, [64, 64]), (ko.KMM, 100, [128, 128]),
+                                     (ko.KMM, 64, [32, 32])])
 def test_wide_step_kernel_needs_whole_tiles(fk, mm, M, Ps):
-    """Fewer columns than a tile's 32 (64) in the KMM layout, or not a multiple of it: the streaming step runs."""
+    """Fewer columns than a tile's 32 (64, 128) in the KMM layout, or not a multiple of it: the streaming step runs."""
     check(fk, mm, M, Ps, Ps, np.float32, seed=72, alpha=1.5, beta=0.5)
     assert not any("mfma16x16x4lds" in k for _, _, k in fk.last_plan()), fk.last_plan()
