@@ -275,9 +275,10 @@ bool Handle::transposeFirstOnline(const KronProblem& p, const KronProblem& pn, v
   size_t nT = 0, nN = 0;
   const bool okT = runOnline(p, temp1, temp2, ws) == fastKronSuccess;
   nT = countLaunches(lastPlan_);
-  // a first launch that reads a transposed M-major X through the padded step with a large factor counts twice (tuned
-  // plans: 128x128 chains run 1.3 to 3.3 times faster behind a transposed copy; 64x64 pairs do not gain)
-  if (okT && p.mm == MMType::MKM && p.P[p.N - 1] >= 128) {
+  // a first launch that reads a transposed X through the padded step with a large factor counts twice (tuned plans:
+  // 128x128 chains run 1.3 to 3.3 times faster behind a transposed copy, 64x64 and 128x128 pairs of single steps
+  // 1.2 to 1.4 times in either layout and type)
+  if (okT && p.P[p.N - 1] >= 64) {
     const size_t s0 = lastPlan_.find(':');
     if (s0 != std::string::npos && lastPlan_.compare(s0 + 1, 6, "gekmm_") == 0 &&
         lastPlan_.find("anyxany", s0) < lastPlan_.find(';', s0)) nT++;
@@ -327,15 +328,24 @@ fastKronError Handle::runOnline(KronProblem p, void* temp1, void* temp2, const C
       }
     }
   }
-  // Kernel-specific requirements on the actual buffers (alignment, strides): when the chosen plan
-  // cannot run on them, fall back to one generic launch per factor.
-  e = execute(p, plan, temp1, temp2, true);
-  if (e == fastKronKernelNotFound) {
-    plan.clear();
-    for (int i = (int)p.N - 1; i >= 0; i--) plan.push_back(PlanStep{(uint32_t)i, (uint32_t)i, db_.genericKernel(p.dt)});
-  } else if (e != fastKronSuccess) {
-    return e;
+  // Kernel-specific requirements on the actual buffers (alignment, strides): a kernel that refuses them is left out
+  // and the selection repeated (the 16-byte accesses of the whole-row and wide kernels need aligned operands, the
+  // streaming kernels behind them in the list do not); one generic launch per factor is the last resort.
+  std::vector<int> refusedKernels;
+  for (int attempt = 0;; attempt++) {
+    int refused = -1;
+    e = execute(p, plan, temp1, temp2, true, &refused);
+    if (e != fastKronKernelNotFound) break;
+    if (refused < 0 || attempt >= 8 || db_.kernels()[refused].P == 0) {
+      plan.clear();
+      for (int i = (int)p.N - 1; i >= 0; i--) plan.push_back(PlanStep{(uint32_t)i, (uint32_t)i, db_.genericKernel(p.dt)});
+      e = fastKronSuccess;
+      break;
+    }
+    refusedKernels.push_back(refused);
+    plan = db_.selectOnline(p, dev_, useFusion(), &refusedKernels);
   }
+  if (e != fastKronSuccess) return e;
   lastPlan_ = key;
   for (auto& s : plan)
     lastPlan_ += ";" + std::to_string(s.lo) + "-" + std::to_string(s.hi) + ":" + db_.kernels()[s.kernel].name;
@@ -614,7 +624,8 @@ StepArgs makeStepArgs(const KronProblem& p, uint32_t lo, uint32_t hi, bool first
 
 // With dryRun the launches are only validated (kernel-specific checks on the concrete buffers);
 // fastKronKernelNotFound then means "this plan cannot run on these buffers".
-fastKronError Handle::execute(const KronProblem& p, const Plan& plan, void* temp1, void* temp2, bool dryRun) {
+fastKronError Handle::execute(const KronProblem& p, const Plan& plan, void* temp1, void* temp2, bool dryRun,
+                              int* refused) {
   const size_t n = plan.size();
   if (n == 0) return fastKronKernelNotFound;
   const uint64_t L = p.L();
@@ -682,7 +693,10 @@ fastKronError Handle::execute(const KronProblem& p, const Plan& plan, void* temp
       for (uint32_t j = 0; j < a.nf && j < kMaxFused; j++)
         c.f[j] = (const char*)a.f[j] + (size_t)b0 * a.f_batch[j] * es;
       if (dryRun) {
-        if (k.check && !k.check(k, c)) return fastKronKernelNotFound;   // every chunk: its base pointers differ
+        if (k.check && !k.check(k, c)) {                                // every chunk: its base pointers differ
+          if (refused) *refused = s.kernel;
+          return fastKronKernelNotFound;
+        }
         if (planOnly_) {
           char line[768];
           int n = snprintf(line, sizeof(line), "kernel=%s lo=%u hi=%u M=%u batch=%u Kin=%llu Kout=%llu in=%p out=%p y=%p "

@@ -45,7 +45,9 @@ class Handle {
   fastKronError xgemm(KronProblem p, fastKronBackend backend, void* temp1, void* temp2, const CallWorkspace* ws = nullptr);
 
   // Runs `plan` on the stream; temps may be null when the plan has a single launch.
-  fastKronError execute(const KronProblem& p, const Plan& plan, void* temp1, void* temp2, bool dryRun = false);
+  // dryRun: only the kernels' checks of the concrete buffers run; *refused then names the kernel that said no
+  fastKronError execute(const KronProblem& p, const Plan& plan, void* temp1, void* temp2, bool dryRun = false,
+                        int* refused = nullptr);
   // What a tuned record prescribes for a problem: merge small factors or not, two-part plan with `split` leading
   // factors or one chain (0), and the launches (numbered in the chain after merging; for a two-part plan the
   // trailing part's steps, on factors >= split, come first).

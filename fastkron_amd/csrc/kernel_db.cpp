@@ -234,7 +234,8 @@ static bool pairCanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, u
   if (first && p.opX == 2) return false;
   // one wave per 64x64 block: with few blocks two single-factor launches, whose tiles are 16 times smaller, fill the
   // device better (tuned plans at 256 blocks: 1.4 times faster in fp32, 1.9 times in fp64; at 1024 blocks the pair wins)
-  if (dev.rulesOfThumb && P == 64 && (uint64_t)p.M * p.batch < 512) return false;
+  // (fp64: two single steps on tiles passed through LDS also win at 1024 blocks, 36 against 44 us)
+  if (dev.rulesOfThumb && P == 64 && (uint64_t)p.M * p.batch < (p.dt == DType::F64 ? 2048u : 512u)) return false;
   return dev.ldsPerBlock >= (int)(2 * k.P * k.P * 8 + 8 * 8192);
 }
 static hipError_t pairLaunch(const KernelInfo& k, const StepArgs& a, hipStream_t s) { return launchPairMfma(a, k.dt, s); }
@@ -242,9 +243,13 @@ static bool pairCheck(const KernelInfo& k, const StepArgs& a) { return pairMfmaS
 
 // ---- KMM-layout step with a 64x64 fp64 factor ----
 static bool kmm64CanRun(const KernelInfo&, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
-                        const DeviceInfo&) {
+                        const DeviceInfo& dev) {
   if (p.dt != DType::F64 || p.mm != MMType::KMM || lo != hi || p.P[lo] != 64 || p.Q[lo] != 64) return false;
   if (first && p.opX == 2) return false;
+  // made for the leading factors of long MKM chains (many batch entries of 4096 contiguous columns); a KMM problem
+  // proper, one entry of a few hundred columns, runs 1.1 to 1.8 times faster on the tiles passed through LDS
+  // (up to 1 GB of X; at 2 GB this kernel is 4 % ahead again)
+  if (dev.rulesOfThumb && p.batch < 8 && (uint64_t)p.M * p.K() < (1ull << 27)) return false;
   return p.M % 64 == 0;
 }
 static hipError_t kmm64Launch(const KernelInfo&, const StepArgs& a, hipStream_t s) { return launchKmm64F64(a, s); }
@@ -280,10 +285,13 @@ static bool kmm4x6Check(const KernelInfo&, const StepArgs& a) { return kmm4x6Sup
 
 // ---- KMM-layout register kernel: NF fused PxP fp32 factors with P^NF = 64 ----
 static bool kmmRegCanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
-                         const DeviceInfo&) {
+                         const DeviceInfo& dev) {
   if (p.dt != DType::F32 || p.mm != MMType::KMM || hi - lo + 1 != k.fused || p.forward) return false;
   for (uint32_t i = lo; i <= hi; i++) if (p.P[i] != k.P || p.Q[i] != k.Q) return false;
   if (first && p.opX == 2) return false;
+  // lanes run along M: with 16 columns a quarter of each wave works, and one plain launch per factor is 1.3 times
+  // faster than half as many launches here (sgekmm 16 x 8^8; three fused factors still pay)
+  if (dev.rulesOfThumb && p.M < 32 && k.fused <= 2) return false;
   return p.colsBefore(hi) % k.tileK == 0 && p.M >= 16;
 }
 static hipError_t kmmRegLaunch(const KernelInfo&, const StepArgs& a, hipStream_t s) { return launchKmmReg(a, s); }
@@ -447,7 +455,12 @@ std::vector<int> KernelDB::candidates(const KronProblem& p, uint32_t lo, uint32_
   return r;
 }
 
-Plan KernelDB::selectOnline(const KronProblem& p, const DeviceInfo& dev, bool allowFusion) const {
+Plan KernelDB::selectOnline(const KronProblem& p, const DeviceInfo& dev, bool allowFusion,
+                            const std::vector<int>* excluded) const {
+  auto barred = [&](int k) {
+    if (excluded) for (int x : *excluded) if (x == k) return true;
+    return false;
+  };
   Plan plan;
   int hi = (int)p.N - 1;
   while (hi >= 0) {
@@ -457,7 +470,7 @@ Plan KernelDB::selectOnline(const KronProblem& p, const DeviceInfo& dev, bool al
       for (int lo = (hi + 1 >= (int)maxDepth) ? hi + 1 - (int)maxDepth : 0; lo <= hi; lo++) {
         auto c = candidates(p, (uint32_t)lo, (uint32_t)hi, hi == (int)p.N - 1, lo == 0, dev);
         int pick = -1;
-        for (int k : c) if (kernels_[k].P != 0 && !kernels_[k].tunerOnly) { pick = k; break; }   // first registered = preferred
+        for (int k : c) if (kernels_[k].P != 0 && !kernels_[k].tunerOnly && !barred(k)) { pick = k; break; }   // first registered = preferred
         if (pick >= 0) { bestLo = lo; bestK = pick; break; }           // deepest fusion wins
       }
     }

@@ -61,7 +61,9 @@ class KernelDB {
   int genericKernel(DType dt) const;
 
   // Online selection (no timing): greedy over the chain, deepest fusion first.
-  Plan selectOnline(const KronProblem& p, const DeviceInfo& dev, bool allowFusion) const;
+  // `excluded`: kernels (indices) that must not be chosen, e.g. because they refused the call's buffers
+  Plan selectOnline(const KronProblem& p, const DeviceInfo& dev, bool allowFusion,
+                    const std::vector<int>* excluded = nullptr) const;
   // All kernels able to run factors [lo, hi] as one launch.
   std::vector<int> candidates(const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool last,
                               const DeviceInfo& dev) const;

@@ -109,9 +109,9 @@ VECTOR_CASES = [
     ("row16x3d", "mkm", "d", 64, [16] * 3, [16] * 3, None, 0.5, "_d_16x16_16x16_3_1x4096"),
     ("row32x3", "mkm", "s", 128, [32] * 3, [32] * 3, None, 0.5, "_32x32_32x32_3_1x32768"),
     ("pair32", "mkm", "s", 64, [32] * 2, [32] * 2, None, 0.5, "_32x32_32x32_2_1x1024"),
-    ("pair64d", "mkm", "d", 512, [64] * 2, [64] * 2, None, 0.5, "_d_64x64_64x64_2_1x4096"),
+    ("pair64d", "mkm", "d", 2048, [64] * 2, [64] * 2, None, 0.5, "_d_64x64_64x64_2_1x4096"),
     ("step64", "mkm", "s", 64, [64], [64], None, 0.5, "_64x64_64x64_1_"),
-    ("kmm64d", "kmm", "d", 64, [64], [64], None, 0.5, "kmm_hip_gfx950_256_d_64x64_64x64_1_64x64"),
+    ("kmm64d", "kmm", "d", 64, [64], [64], 8, 0.5, "kmm_hip_gfx950_256_d_64x64_64x64_1_64x64"),
     ("row8x5", "mkm", "s", 64, [8] * 5, [8] * 5, None, 0.5, "_8x8_8x8_5_1x32768"),
     ("row32x16", "mkm", "s", 64, [32] * 3, [16] * 3, None, 0.5, "_32x16_32x16_3_1x32768"),
     ("kmm4x6", "kmm", "s", 64, [4] * 6, [4] * 6, None, 0.5, "_4x4_4x4_6_8x4096"),
@@ -361,3 +361,14 @@ def test_a_small_result_behind_a_large_input_is_streamed_out(planner):
     """8 x 512 x (32x16)^3 with Y: 537 MB of X, 67 MB of Z; the launch moves far more than the caches hold."""
     e, names, launches = plan(planner, "mkm", "s", 512, [32] * 3, [16] * 3, batch=8, beta=1.0, with_y=True)
     assert e == capi.SUCCESS and len(launches) == 1 and _hints(launches) == [(1, 1)]
+
+
+# ---- a kernel that refuses the call's buffers is replaced by the next one in line ----
+@pytest.mark.parametrize("which,expect", [("z", "_128x128_128x128_1_1x2048_mfma16x16x4_NN"), ("y", "_128x128_128x128_1_1x2048_mfma16x16x4_NN"),
+                                          ("x", "anyxany")])
+def test_a_refusing_kernel_is_replaced_by_the_next_in_line(planner, which, expect):
+    """sgemkm 8 x 128^2: the wide step kernel needs X, Z and Y on 16-byte boundaries, the streaming step only X, the
+    padded step nothing: an operand one element off moves the plan down that list, not to the plain kernel."""
+    e, names, launches = plan(planner, "mkm", "s", 8, [128] * 2, [128] * 2, beta=0.5, with_y=True, offs={which: 4})
+    assert e == capi.SUCCESS and len(launches) == 2
+    assert all(expect in n for n in names), names
