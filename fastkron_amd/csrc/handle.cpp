@@ -275,10 +275,10 @@ bool Handle::transposeFirstOnline(const KronProblem& p, const KronProblem& pn, v
   size_t nT = 0, nN = 0;
   const bool okT = runOnline(p, temp1, temp2, ws) == fastKronSuccess;
   nT = countLaunches(lastPlan_);
-  // a first launch that reads a transposed X through the padded step with a large factor counts twice (tuned plans:
-  // 128x128 chains run 1.3 to 3.3 times faster behind a transposed copy, 64x64 and 128x128 pairs of single steps
-  // 1.2 to 1.4 times in either layout and type)
-  if (okT && p.P[p.N - 1] >= 64) {
+  // a first launch that reads a transposed M-major X through the padded step with a large factor counts twice (tuned
+  // plans: 128x128 chains run 1.3 to 3.3 times faster behind a transposed copy, pairs of single 64x64 steps 1.3 to 1.4
+  // times; in the KMM layout the padded step reads a transposed X along its rows and stays ahead by 5 to 30 %)
+  if (okT && p.mm == MMType::MKM && p.P[p.N - 1] >= 64) {
     const size_t s0 = lastPlan_.find(':');
     if (s0 != std::string::npos && lastPlan_.compare(s0 + 1, 6, "gekmm_") == 0 &&
         lastPlan_.find("anyxany", s0) < lastPlan_.find(';', s0)) nT++;
@@ -288,7 +288,10 @@ bool Handle::transposeFirstOnline(const KronProblem& p, const KronProblem& pn, v
   planOnly_ = wasPlanOnly;
   lastPlan_ = savedPlan; launchLog_ = savedLog;
   // without a second temporary the transposed copy sits in temp1, which a plan of several launches writes
-  bool yes = okN && (!okT || 1 + nN <= nT);
+  // (KMM layout: with equal launch counts the plan that reads the transposed X in its first launch is 6 to 16 %
+  // ahead on 16x16 chains, and 18 to 29 % behind on 8x8 chains, whose first factor fills half a matrix-core tile)
+  const bool tie = p.mm == MMType::MKM || p.P[p.N - 1] < 16;
+  bool yes = okN && (!okT || (tie ? 1 + nN <= nT : 1 + nN < nT));
   if (yes && !temp2 && nN != 1) yes = false;
   transposeCache_[ck] = yes;
   return yes;

@@ -281,7 +281,7 @@ def _shipped_records():
 
 def test_every_shipped_plan_is_what_a_default_handle_runs(planner):
     recs = _shipped_records()
-    assert len(recs) >= 10
+    assert len(recs) >= 3
     for key, flags, steps in recs:
         if "stridedBatched" in key:
             continue

@@ -104,10 +104,12 @@ def test_tuned_plan_of_a_mixed_chain_is_not_slower_than_the_online_one(tmp_path)
 @pytest.mark.parametrize("mm,M,Ps,dt,opX,opF", [
     (ko.MKM, 256, [64, 64], np.float64, ko.OP_T, ko.OP_T), (ko.KMM, 256, [64, 64], np.float64, ko.OP_N, ko.OP_N),
     (ko.MKM, 256, [128, 128], np.float64, ko.OP_N, ko.OP_N), (ko.KMM, 256, [128, 128], np.float32, ko.OP_T, ko.OP_T),
-    (ko.MKM, 256, [128, 128], np.float32, ko.OP_T, ko.OP_T), (ko.MKM, 256, [16] * 4, np.float64, ko.OP_T, ko.OP_T)])
+    (ko.MKM, 256, [128, 128], np.float32, ko.OP_T, ko.OP_T), (ko.MKM, 256, [16] * 4, np.float64, ko.OP_T, ko.OP_T),
+    (ko.KMM, 256, [16] * 4, np.float32, ko.OP_T, ko.OP_T), (ko.KMM, 256, [16] * 4, np.float64, ko.OP_T, ko.OP_T)])
 def test_shapes_with_a_shipped_plan_match_the_oracle(mm, M, Ps, dt, opX, opF):
-    """Shapes of the reference's performance table for which fastkron_amd/gfx950_plans.txt holds a tuned plan: a
-    default handle runs that plan (checked on the host in tests/test_planner_cpu.py) and the result is the oracle's."""
+    """Shapes of the reference's performance table for which fastkron_amd/gfx950_plans.txt holds a tuned plan, or held
+    one until the online rules took it over: a default handle runs the shipped plan where there is one (checked on the
+    host in tests/test_planner_cpu.py) and the result is the oracle's."""
     import fastkron_amd
     h = fastkron_amd.FastKron()
     try:
