@@ -789,3 +789,15 @@ def test_wide_step_kernel_needs_whole_tiles(fk, mm, M, Ps):
     """Fewer columns than a tile's 32 (64, 128) in the KMM layout, or not a multiple of it: the streaming step runs."""
     check(fk, mm, M, Ps, Ps, np.float32, seed=72, alpha=1.5, beta=0.5)
     assert not any("mfma16x16x4lds" in k for _, _, k in fk.last_plan()), fk.last_plan()
+
+
+@pytest.mark.parametrize("M,Ps", [(32, [16, 16]), (96, [16] * 4), (64, [12, 12]), (32, [9, 9, 9, 9]), (48, [16, 16]), (160, [15, 15])])
+def test_kmm_pairs_of_16x16_with_two_columns_per_lane(fk, M, Ps):
+    """sgekmm with pairs of 16x16 (9x9 ... 15x15) factors: with a multiple of 32 columns a lane owns two neighbouring
+    columns and moves them as 8-byte elements (48 columns: one column per lane as before)."""
+    check(fk, ko.KMM, M, Ps, Ps, np.float32, alpha=1.5, beta=0.5, seed=211)
+    assert any("_2_16x256_" in k for _, _, k in fk.last_plan()), fk.last_plan()
+    check(fk, ko.KMM, M, Ps, Ps, np.float32, alpha=1.0, beta=0.0, seed=212, opFs=ko.OP_T)
+    check(fk, ko.KMM, M, Ps, Ps, np.float32, alpha=1.0, beta=1.0, seed=213, batch=3)
+    check(fk, ko.KMM, M, Ps, Ps, np.float32, alpha=2.0, beta=0.0, seed=214, batch=2, share_f=True)
+    check(fk, ko.KMM, M, Ps, Ps, np.float32, alpha=1.0, beta=0.0, seed=215, integer=True, use_temp2=False)
