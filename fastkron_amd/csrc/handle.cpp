@@ -346,7 +346,12 @@ fastKronError Handle::runOnline(KronProblem p, void* temp1, void* temp2, const C
       break;
     }
     refusedKernels.push_back(refused);
-    plan = db_.selectOnline(p, dev_, useFusion(), &refusedKernels);
+    // (cached like the first selection, under the problem and the kernels left out)
+    std::string rk = key + (p.forward ? "_fwd" : "") + (useFusion() ? "" : "_nofuse") + "|without";
+    for (int k : refusedKernels) rk += ":" + std::to_string(k);
+    auto it = planCache_.find(rk);
+    if (it != planCache_.end()) plan = it->second;
+    else { plan = db_.selectOnline(p, dev_, useFusion(), &refusedKernels); planCache_[rk] = plan; }
   }
   if (e != fastKronSuccess) return e;
   lastPlan_ = key;
