@@ -295,6 +295,17 @@ static bool kmmRegCanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo,
   return p.colsBefore(hi) % k.tileK == 0 && p.M >= 16;
 }
 static hipError_t kmmRegLaunch(const KernelInfo&, const StepArgs& a, hipStream_t s) { return launchKmmReg(a, s); }
+
+// ---- KMM layout: three fused 8x8 fp32 factors, 512 rows by 64 columns per workgroup ----
+static bool kmm8x3CanRun(const KernelInfo&, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
+                         const DeviceInfo&) {
+  if (p.dt != DType::F32 || p.mm != MMType::KMM || hi - lo + 1 != 3 || p.forward) return false;
+  for (uint32_t i = lo; i <= hi; i++) if (p.P[i] != 8 || p.Q[i] != 8) return false;
+  if (first && p.opX == 2) return false;
+  return p.colsBefore(hi) % 512 == 0 && p.M % 64 == 0;
+}
+static hipError_t kmm8x3Launch(const KernelInfo&, const StepArgs& a, hipStream_t s) { return launchKmm8x3(a, s); }
+static bool kmm8x3Check(const KernelInfo&, const StepArgs& a) { return kmm8x3Supported(a); }
 static bool kmmRegCheck(const KernelInfo&, const StepArgs& a) { return kmmRegSupported(a); }
 
 void registerRowKernels(std::vector<KernelInfo>& out) {
@@ -353,6 +364,14 @@ void registerRowKernels(std::vector<KernelInfo>& out) {
     k6.dt = DType::F32; k6.P = 4; k6.Q = 4; k6.fused = 6; k6.tileM = 8; k6.tileK = 4096; k6.threads = 512; k6.variant = 0;
     k6.canRun = kmm4x6CanRun; k6.launch = kmm4x6Launch; k6.check = kmm4x6Check;
     out.push_back(k6);
+  }
+
+  {
+    KernelInfo k3{};
+    k3.name = "kmm_hip_gfx950_512_f_8x8_8x8_3_64x512_mfma4x4x1_NN_strided_0_3";
+    k3.dt = DType::F32; k3.P = 8; k3.Q = 8; k3.fused = 3; k3.tileM = 64; k3.tileK = 512; k3.threads = 512; k3.variant = 0;
+    k3.canRun = kmm8x3CanRun; k3.launch = kmm8x3Launch; k3.check = kmm8x3Check;
+    out.push_back(k3);
   }
 
   // deepest fusion first: the online selection takes the first kernel that fits at a given depth

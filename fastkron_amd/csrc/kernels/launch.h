@@ -80,6 +80,10 @@ hipError_t launchRow32x3(const StepArgs& a, hipStream_t stream);
 bool pairMfmaSupported(const StepArgs& a, DType dt);
 hipError_t launchPairMfma(const StepArgs& a, DType dt, hipStream_t stream);
 
+// Three fused 8x8 fp32 factors in the KMM layout, 512 rows by 64 columns per workgroup.
+bool kmm8x3Supported(const StepArgs& a);
+hipError_t launchKmm8x3(const StepArgs& a, hipStream_t stream);
+
 // One step with a 64x64 or 128x128 factor, either type and layout, tiles of 16 KB passed through LDS.
 bool stepWideSupported(const StepArgs& a, DType dt);
 hipError_t launchStepWide(const StepArgs& a, DType dt, hipStream_t stream);

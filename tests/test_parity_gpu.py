@@ -801,3 +801,17 @@ def test_kmm_pairs_of_16x16_with_two_columns_per_lane(fk, M, Ps):
     check(fk, ko.KMM, M, Ps, Ps, np.float32, alpha=1.0, beta=1.0, seed=213, batch=3)
     check(fk, ko.KMM, M, Ps, Ps, np.float32, alpha=2.0, beta=0.0, seed=214, batch=2, share_f=True)
     check(fk, ko.KMM, M, Ps, Ps, np.float32, alpha=1.0, beta=0.0, seed=215, integer=True, use_temp2=False)
+
+
+@pytest.mark.parametrize("mm,M,Ps,launches", [(ko.KMM, 64, [8] * 3, 1), (ko.KMM, 128, [8] * 5, 2), (ko.KMM, 192, [8] * 6, 2),
+                                              (ko.KMM, 64, [4, 8, 8, 8], 2), (ko.MKM, 2, [8] * 8, 2), (ko.KMM, 80, [8] * 3, 2)])
+def test_kmm_three_fused_8x8_factors(fk, mm, M, Ps, launches):
+    """sgekmm chains of 8x8 factors: three per launch on 512 rows by 64 columns per workgroup (a multiple of 64 columns;
+    80 columns keep the two-factor kernel), also for the leading factors of a long sgemkm chain."""
+    check(fk, mm, M, Ps, Ps, np.float32, alpha=1.5, beta=0.5, seed=221)
+    plan = fk.last_plan()
+    assert len(plan) == launches and (M % 64 != 0 and mm == ko.KMM or any("_8x8_8x8_3_64x512_" in k for _, _, k in plan)), plan
+    check(fk, mm, M, Ps, Ps, np.float32, alpha=1.0, beta=0.0, seed=222, opFs=ko.OP_T)
+    check(fk, mm, M, Ps, Ps, np.float32, alpha=1.0, beta=1.0, seed=223, batch=3)
+    check(fk, mm, M, Ps, Ps, np.float32, alpha=2.0, beta=0.0, seed=224, batch=2, share_f=True)
+    check(fk, mm, M, Ps, Ps, np.float32, alpha=1.0, beta=0.0, seed=225, integer=True, use_temp2=False)
