@@ -275,10 +275,12 @@ bool Handle::transposeFirstOnline(const KronProblem& p, const KronProblem& pn, v
   size_t nT = 0, nN = 0;
   const bool okT = runOnline(p, temp1, temp2, ws) == fastKronSuccess;
   nT = countLaunches(lastPlan_);
-  // a first launch that reads a transposed M-major X through the padded step with a large factor counts twice (tuned
-  // plans: 128x128 chains run 1.3 to 3.3 times faster behind a transposed copy, pairs of single 64x64 steps 1.3 to 1.4
-  // times; in the KMM layout the padded step reads a transposed X along its rows and stays ahead by 5 to 30 %)
-  if (okT && p.mm == MMType::MKM && p.P[p.N - 1] >= 64) {
+  // a first launch that reads a transposed X through the padded step with a large factor counts twice: in the MKM layout
+  // always (tuned plans: 128x128 chains run 1.3 to 3.3 times faster behind a transposed copy, pairs of single 64x64
+  // steps 1.3 to 1.4 times); in the KMM layout, where that step reads the transposed X along its rows, only while X
+  // stays in the caches (up to 64 MB the copy is ahead by 8 to 14 %, beyond that behind by 5 to 30 %)
+  const uint64_t xBytes = p.M * p.K() * (p.dt == DType::F32 ? 4 : 8) * (uint64_t)(p.batch ? p.batch : 1);
+  if (okT && p.P[p.N - 1] >= 64 && (p.mm == MMType::MKM || xBytes <= (64ull << 20))) {
     const size_t s0 = lastPlan_.find(':');
     if (s0 != std::string::npos && lastPlan_.compare(s0 + 1, 6, "gekmm_") == 0 &&
         lastPlan_.find("anyxany", s0) < lastPlan_.find(';', s0)) nT++;
@@ -288,10 +290,12 @@ bool Handle::transposeFirstOnline(const KronProblem& p, const KronProblem& pn, v
   planOnly_ = wasPlanOnly;
   lastPlan_ = savedPlan; launchLog_ = savedLog;
   // without a second temporary the transposed copy sits in temp1, which a plan of several launches writes
-  // (KMM layout: with equal launch counts the plan that reads the transposed X in its first launch is 6 to 16 %
-  // ahead on 16x16 chains, and 18 to 29 % behind on 8x8 chains, whose first factor fills half a matrix-core tile)
-  const bool tie = p.mm == MMType::MKM || p.P[p.N - 1] < 16;
-  bool yes = okN && (!okT || (tie ? 1 + nN <= nT : 1 + nN < nT));
+  // with equal counts the copy goes first, except in the KMM layout with fewer than 64 columns, where the copy cannot
+  // run on whole 64-wide tiles with 16-byte accesses (sgekmm 16x16^4 with 256 and 1024 columns: 1.26 times faster
+  // behind the copy; 16 columns, 16x16^6: 1.16 times slower; factors below 16x16 read a transposed X too slowly in any
+  // case)
+  const bool copyOnTie = p.mm == MMType::MKM || p.M >= 64 || p.P[p.N - 1] < 16;
+  bool yes = okN && (!okT || (copyOnTie ? 1 + nN <= nT : 1 + nN < nT));
   if (yes && !temp2 && nN != 1) yes = false;
   transposeCache_[ck] = yes;
   return yes;

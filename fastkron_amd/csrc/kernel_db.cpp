@@ -76,6 +76,8 @@ static bool stepAnyCanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo
   // a first launch that reads a transposed X: the plain kernel's lanes then run across the strided dimension, and the
   // padded tiles win from 8x8 on (tuned plans: 16x16 chains with op(X) = T 2.6 times faster)
   if (first && p.opX == 2) minPQ = 64;
+  // shrinking factors with 16 rows or more (tuned plans: gemkm 1024 x (16x8)^5 1.4 times faster in both types)
+  if (!kmm && P >= 16 && Q < P && minPQ > 128) minPQ = 128;
   return ((uint64_t)P * Q >= minPQ || !dev.rulesOfThumb) && P >= 4;
 }
 static hipError_t stepAnyLaunch(const KernelInfo& k, const StepArgs& a, hipStream_t s) {
@@ -491,6 +493,20 @@ Plan KernelDB::selectOnline(const KronProblem& p, const DeviceInfo& dev, bool al
         int pick = -1;
         for (int k : c) if (kernels_[k].P != 0 && !kernels_[k].tunerOnly && !barred(k)) { pick = k; break; }   // first registered = preferred
         if (pick >= 0) { bestLo = lo; bestK = pick; break; }           // deepest fusion wins
+      }
+      // The LDS-fused kernel taken as deep as it goes can leave one or two factors, which then run one plain launch
+      // each (or a shallow group): two groups of about equal depth are faster (tuned plans: sgemkm 1024 x (2x4)^7 as
+      // 4 + 3 instead of 6 + 1: 1.34 times, sgekmm 1024 x 3^7 as 4 + 3 instead of 5 + 1 + 1: 1.3 times).
+      const int total = hi + 1, depth = hi - bestLo + 1;
+      if (kernels_[bestK].canRun == fusedSmallCanRun && bestLo > 0 && bestLo < depth - 1 && total <= 2 * (int)maxDepth) {
+        auto fusedPick = [&](int lo, int h) {
+          for (int k : candidates(p, (uint32_t)lo, (uint32_t)h, h == (int)p.N - 1, lo == 0, dev))
+            if (kernels_[k].P != 0 && !kernels_[k].tunerOnly && !barred(k)) return kernels_[k].canRun == fusedSmallCanRun ? k : -1;
+          return -1;
+        };
+        const int lo2 = hi + 1 - (total + 1) / 2;
+        const int upper = fusedPick(lo2, hi);
+        if (upper >= 0 && fusedPick(0, lo2 - 1) >= 0) { bestLo = lo2; bestK = upper; }
       }
     }
     plan.push_back(PlanStep{(uint32_t)bestLo, (uint32_t)hi, bestK});

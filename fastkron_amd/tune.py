@@ -12,7 +12,8 @@ reference's src/print_best_kernel_for_shapes.py:13-21,72-83, which drives its be
 the log; here the tuner is called through the C API.
 
 `--table` tunes the shapes of the reference's published performance table (reference documents/performance.md:9-480:
-M_PxP^N for both layouts, both types, untransposed and transposed operands) plus the five benchmark configurations;
+M_PxP^N for both layouts, both types, untransposed and transposed operands), chains with odd, rectangular and differing
+factors of the kinds its tests run, and the five benchmark configurations;
 with `--keep-if-faster F` a record is only kept when the tuned plan beats the online selection by that fraction,
 which is how fastkron_amd/gfx950_plans.txt, the file the library loads by default, was made.
 """
@@ -30,6 +31,14 @@ TABLE = [(1024, 8, 5), (1024, 8, 6), (1024, 16, 4), (1024, 16, 5), (1024, 32, 3)
          (1024, 64, 3), (1024, 128, 2), (320, 128, 3), (16, 8, 8), (16, 16, 6), (16, 32, 5), (16, 64, 4), (16, 128, 3),
          (256, 8, 5), (256, 8, 6), (256, 16, 4), (256, 16, 5), (256, 32, 3), (256, 32, 4), (256, 64, 2), (256, 64, 3),
          (256, 128, 2), (128, 128, 3)]
+
+# chains of the kinds the reference's tests run (reference tests/src/general-tests-NN.cpp:53-100: odd sizes, rectangular
+# factors; :102-160: factors that differ), here with 1024 rows (MKM) or columns (KMM) of X
+IRREGULAR = [([3] * 7, [3] * 7), ([5] * 6, [5] * 6), ([6] * 6, [6] * 6), ([12] * 4, [12] * 4), ([24] * 3, [24] * 3),
+             ([31] * 3, [31] * 3), ([50] * 3, [50] * 3), ([62] * 2, [62] * 2), ([127] * 2, [127] * 2), ([129] * 2, [129] * 2),
+             ([2] * 7, [4] * 7), ([31] * 3, [63] * 3), ([63] * 3, [31] * 3), ([16] * 5, [8] * 5), ([8] * 4, [32] * 4),
+             ([12] * 5, [16] * 5), ([32] * 3, [64] * 3), ([2, 3, 4, 5, 6, 7, 8], [2, 3, 4, 5, 6, 7, 8]),
+             ([8, 16, 32], [8, 16, 32]), ([64, 32, 16, 8], [64, 32, 16, 8])]
 
 
 def _shapes(args):
@@ -125,6 +134,10 @@ def tune_table(db, keep_if_faster, only=None, verbose=True):
             for ops in ((OP_N, OP_N), (OP_T, OP_T)):
                 for M, P, N in TABLE:
                     problems.append((mm, dtype, ops, M, [P] * N, [P] * N, 1.0, 0.0, 1))
+    for mm in ("mkm", "kmm"):
+        for dtype in (torch.float32, torch.float64):
+            for Ps, Qs in IRREGULAR:
+                problems.append((mm, dtype, (OP_N, OP_N), 1024, Ps, Qs, 1.0, 0.0, 1))
     problems += [("mkm", torch.float32, (OP_N, OP_N), 1024, [8] * 5, [8] * 5, 1.0, 0.0, 1),
                  ("kmm", torch.float32, (OP_N, OP_N), 2048, [4] * 6, [4] * 6, 1.5, 0.5, 1),
                  ("mkm", torch.float32, (OP_N, OP_N), 512, [32] * 3, [16] * 3, 1.0, 1.0, 8)]
@@ -134,7 +147,8 @@ def tune_table(db, keep_if_faster, only=None, verbose=True):
     for idx, (mm, dtype, ops, M, Ps, Qs, alpha, beta, batch) in enumerate(problems):
         if only is not None and idx % only[1] != only[0]:
             continue
-        tag = f"{mm} {'f' if dtype == torch.float32 else 'd'} {'NN' if ops[0] == OP_N else 'TT'} {M}_{Ps[0]}x{Qs[0]}^{len(Ps)}"
+        tag = f"{mm} {'f' if dtype == torch.float32 else 'd'} {'NN' if ops[0] == OP_N else 'TT'} {M}_" + \
+              (f"{Ps[0]}x{Qs[0]}^{len(Ps)}" if len(set(zip(Ps, Qs))) == 1 else ",".join(f"{p}x{q}" for p, q in zip(Ps, Qs)))
         try:
             case = _Case(online, mm, M, Ps, Qs, dtype, alpha, beta, batch)
         except torch.cuda.OutOfMemoryError:

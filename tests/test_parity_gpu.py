@@ -474,6 +474,9 @@ def test_kmm_layout_fp64_64x64_step_on_4x4x4_matrix_instruction(fk, M, Ps):
     instruction (single problems of this size run on the tiles passed through LDS)."""
     check(fk, ko.KMM, M, Ps, Ps, np.float64, alpha=1.5, beta=0.5, seed=151, batch=8)
     assert any("mfma4x4x4" in k for _, _, k in fk.last_plan()), fk.last_plan()
+    # (one factor for all entries: the launch walks the tiles of all entries as one sequence)
+    check(fk, ko.KMM, M, Ps, Ps, np.float64, alpha=1.5, beta=0.5, seed=157, batch=9, share_f=True)
+    assert any("mfma4x4x4" in k for _, _, k in fk.last_plan()), fk.last_plan()
     check(fk, ko.KMM, M, Ps, Ps, np.float64, alpha=1.5, beta=0.5, seed=156)
     assert not any("mfma4x4x4" in k for _, _, k in fk.last_plan()), fk.last_plan()
     check(fk, ko.KMM, M, Ps, Ps, np.float64, alpha=1.0, beta=0.0, seed=152, opFs=ko.OP_T)
