@@ -76,6 +76,9 @@ static bool stepAnyCanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo
   // a first launch that reads a transposed X: the plain kernel's lanes then run across the strided dimension, and the
   // padded tiles win from 8x8 on (tuned plans: 16x16 chains with op(X) = T 2.6 times faster)
   if (first && p.opX == 2) minPQ = 64;
+  // fp64 in the KMM layout with more than 128 rows that do not fill the padded groups of four: the plain kernel is
+  // 1.8 times faster (dgekmm 1024 x 129^2 and 200^2; 160^2 the same, 255^2 slower)
+  if (dev.rulesOfThumb && kmm && p.dt == DType::F64 && P > 128 && ((P + 3) / 4) % 4 != 0) return false;
   // shrinking factors with 16 rows or more (tuned plans: gemkm 1024 x (16x8)^5 1.4 times faster in both types)
   if (!kmm && P >= 16 && Q < P && minPQ > 128) minPQ = 128;
   return ((uint64_t)P * Q >= minPQ || !dev.rulesOfThumb) && P >= 4;
