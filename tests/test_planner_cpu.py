@@ -24,6 +24,18 @@ def planner():
     lib.fastKronDestroy(h)
 
 
+@pytest.fixture
+def online_planner(monkeypatch):
+    """A plan-only handle without the shipped tuned plans: the online rules alone."""
+    monkeypatch.setenv("FASTKRON_SHIPPED_PLANS", "0")
+    lib = capi.load()
+    h = ctypes.c_void_p()
+    assert lib.fastKronInit(ctypes.byref(h), capi.BACKEND_HIP) == capi.SUCCESS
+    assert lib.fastKronSetPlanOnly(h, 1) == capi.SUCCESS
+    yield lib, h
+    lib.fastKronDestroy(h)
+
+
 def plan(planner, mm, dt, M, Ps, Qs, batch=None, alpha=1.0, beta=0.0, with_y=False, offs=None, strides=None,
          strideF=None, opX=capi.OP_N, opF=capi.OP_N, temp2=True, y_is_z=False):
     """Runs one call in plan-only mode.  `offs` shifts the fake base pointers of x / z / y / t1 / t2 by bytes,
@@ -237,6 +249,53 @@ def test_transposed_x_is_read_in_place_when_a_copy_does_not_pay_or_does_not_fit(
     e, names, launches = plan(planner, "mkm", "s", 64, [8] * 5, [8] * 5, opX=capi.OP_T, temp2=False)
     assert e == capi.SUCCESS and names[0].startswith("transpose_") and len(names) == 2, names
     assert int(launches[0]["in"], 16) == BASE + 3 * GAP
+
+
+def test_transposition_rules_that_came_from_tuned_plans(online_planner):
+    planner = online_planner
+    copied = lambda names: names[0].startswith("transpose_")
+    # a padded-step first launch on a 128-wide factor counts twice in the MKM layout, also with 16 rows ...
+    e, names, _ = plan(planner, "mkm", "s", 16, [128] * 3, [128] * 3, opX=capi.OP_T)
+    assert e == capi.SUCCESS and copied(names) and len(names) == 4, names
+    # ... in the KMM layout only while X is at most 64 MB
+    e, names, _ = plan(planner, "kmm", "s", 1024, [128] * 2, [128] * 2, opX=capi.OP_T)
+    assert e == capi.SUCCESS and copied(names), names
+    e, names, _ = plan(planner, "kmm", "s", 320, [128] * 3, [128] * 3, opX=capi.OP_T)
+    assert e == capi.SUCCESS and not copied(names) and len(names) == 3, names
+    # equal launch counts: the copy goes first, except in the KMM layout with fewer than 64 columns
+    e, names, _ = plan(planner, "kmm", "s", 256, [16] * 4, [16] * 4, opX=capi.OP_T)
+    assert e == capi.SUCCESS and copied(names) and len(names) == 3, names
+    e, names, _ = plan(planner, "kmm", "s", 16, [16] * 6, [16] * 6, opX=capi.OP_T)
+    assert e == capi.SUCCESS and not copied(names), names
+
+
+# ---- online rules for chains outside the specialised kernels ----
+def test_lds_fused_groups_get_balanced_depth(online_planner):
+    """The LDS-fused kernel taken as deep as it goes would leave a single plain launch (or two): the last two groups share
+    the factors about equally instead."""
+    planner = online_planner
+    e, names, _ = plan(planner, "mkm", "s", 1024, [2] * 7, [4] * 7)
+    assert e == capi.SUCCESS and len(names) == 2 and all("small_fused" in n for n in names), names
+    e, names, _ = plan(planner, "kmm", "s", 1024, [3] * 7, [3] * 7)
+    assert e == capi.SUCCESS and len(names) == 2 and all("small_fused" in n for n in names), names
+    # a chain that one group holds stays one launch
+    e, names, _ = plan(planner, "mkm", "s", 1024, [3] * 7, [3] * 7)
+    assert e == capi.SUCCESS and len(names) == 1 and "small_fused" in names[0], names
+
+
+def test_padded_step_rules_for_rectangular_and_large_odd_factors(online_planner):
+    planner = online_planner
+    # shrinking factors with 16 rows: padded matrix-core step, not the plain kernel
+    for dt in ("s", "d"):
+        e, names, _ = plan(planner, "mkm", dt, 1024, [16] * 5, [8] * 5)
+        assert e == capi.SUCCESS and len(names) == 5 and all("anyxany" in n for n in names), names
+    # fp64, KMM layout, more than 128 rows: plain kernel when the padded groups of four stay part empty
+    e, names, _ = plan(planner, "kmm", "d", 1024, [129] * 2, [129] * 2)
+    assert e == capi.SUCCESS and all("generic" in n for n in names), names
+    e, names, _ = plan(planner, "kmm", "d", 1024, [255] * 2, [255] * 2)
+    assert e == capi.SUCCESS and all("anyxany" in n for n in names), names
+    e, names, _ = plan(planner, "kmm", "s", 1024, [200] * 2, [200] * 2)
+    assert e == capi.SUCCESS and all("anyxany" in n for n in names), names
 
 
 # ---- the plans that ship with the library (fastkron_amd/gfx950_plans.txt) ----
