@@ -34,7 +34,8 @@ constexpr int kR32Len = 32768;
 constexpr int kR32QuarterWords = 32 * 256;                         // 32 rows k1 of 256 columns
 constexpr int kR32LdsWords = 2 * kR32QuarterWords + 3 * 1024;      // two quarters + the three factors
 
-// NT: 0 = ordinary stores, 1 = non-temporal stores (1024 x 32^3: 85.0 -> 78.0 us; non-temporal loads of X: 81.6)
+// NT: 0 = ordinary stores, 1 = streaming stores (1024 x 32^3: 85.0 -> 78.0 us with non-temporal stores, non-temporal loads
+// of X as well: 81.6; at system scope through a descriptor of the row: 4096 rows 286 -> 279 us)
 template <bool HAS_Y, int NT>
 __global__ __launch_bounds__(512, 4) void kron_row32x3_kernel(const StepArgs a) {
   extern __shared__ __align__(16) float r32lds[];
@@ -48,6 +49,7 @@ __global__ __launch_bounds__(512, 4) void kron_row32x3_kernel(const StepArgs a) 
   const float* X = (const float*)a.in + (size_t)bt * a.in_batch + (size_t)m * a.in_ldm;
   float* Z = (float*)a.out + (size_t)bt * a.out_batch + (size_t)m * a.out_ldm;
   const float* Y = HAS_Y ? (const float*)a.y + (size_t)bt * a.y_batch + (size_t)m * a.y_ldm : nullptr;
+  const __amdgpu_buffer_rsrc_t zTarget = streamTarget((void*)Z, 32768 * 4u);
 
   // factors to LDS ahead of the row loads (vector memory operations retire in order); a.f[0] is the factor of the
   // fastest digit (F3), element (p, q) at p*f_sp + q*f_sq
@@ -166,7 +168,8 @@ __global__ __launch_bounds__(512, 4) void kron_row32x3_kernel(const StepArgs a) 
     for (int r = 0; r < 4; r++) {
       r3f4 o = (r3f4){D[0][r], D[1][r], D[2][r], D[3][r]} * alpha;
       if (HAS_Y) o = o + yv[r] * beta;
-      FK_ST(NT, o, (r3f4*)(Z + (col + r * 1024)));
+      if (NT) streamStore16(o, zTarget, (col + r * 1024) * 4u);
+      else *(r3f4*)(Z + (col + r * 1024)) = o;
     }
   };
 

@@ -640,10 +640,13 @@ ANY_SHAPE = [
 @pytest.mark.parametrize("M,Ps,Qs", ANY_SHAPE)
 def test_any_shape_step_on_the_matrix_cores(fk, mm, M, Ps, Qs, dt):
     check(fk, mm, M, Ps, Qs, dt, alpha=1.5, beta=0.5, seed=401)
-    assert any("anyxany" in k for _, _, k in fk.last_plan()), fk.last_plan()
+    # (online rule: fp64 factors of more than 128 rows that leave the padded groups of four part empty run on the plain
+    # kernel in the KMM layout; 255 rows stay here)
+    ruled_out = mm == ko.KMM and dt == np.float64 and all(p > 128 and ((p + 3) // 4) % 4 for p in Ps)
+    assert ruled_out or any("anyxany" in k for _, _, k in fk.last_plan()), fk.last_plan()
     check(fk, mm, M, Ps, Qs, dt, alpha=1.0, beta=0.0, seed=402, opFs=ko.OP_T)
     check(fk, mm, M, Ps, Qs, dt, alpha=1.0, beta=0.0, seed=403, opX=ko.OP_T)       # X stored transposed
-    assert any("anyxany" in k for _, _, k in fk.last_plan()), fk.last_plan()
+    assert ruled_out or any("anyxany" in k for _, _, k in fk.last_plan()), fk.last_plan()
     check(fk, mm, M, Ps, Qs, dt, alpha=2.0, beta=1.0, seed=404, batch=3)
     check(fk, mm, M, Ps, Qs, dt, alpha=1.0, beta=1.0, seed=405, integer=True)
     check(fk, mm, M, Ps, Qs, dt, alpha=1.0, beta=0.0, seed=406, use_temp2=False)
