@@ -184,7 +184,9 @@ fastKronError Handle::xgemm(KronProblem p, fastKronBackend backend, void* temp1,
   if (!p.forward) {
     Choice c;
     bool have = lookupChoice(p, &c);
-    if (!have && canTune() && !planOnly_ && !ws) {
+    // (a GeKMM that runs as a GeMKM is tuned as that GeMKM, below)
+    const bool asMKM = p.mm == MMType::KMM && useFusion() && temp2 && viaMKMOnline(p);
+    if (!have && canTune() && !planOnly_ && !ws && !asMKM) {
       e = tune(p, temp2 != nullptr, &c);
       if (e != fastKronSuccess && e != fastKronKernelNotFound) return e;
       have = (e == fastKronSuccess);
@@ -195,7 +197,14 @@ fastKronError Handle::xgemm(KronProblem p, fastKronBackend backend, void* temp1,
     }
   }
 
-  // 2. Online selection.  With op(X) = T first the question whether to transpose X ahead of the launches.
+  // 2. Online selection.  A GeKMM whose X is stored transposed is the GeMKM of that buffer with a transposed result:
+  //    the whole-row GeMKM kernels then apply, and one transposition at the end writes Z.
+  //    With few columns that pays even when X has to be transposed first.
+  if (p.mm == MMType::KMM && !p.forward && useFusion() && temp2 && viaMKMOnline(p)) {
+    e = runViaMKM(p, backend, temp1, temp2, ws);
+    if (e != fastKronKernelNotFound) return e;
+  }
+  //    With op(X) = T otherwise the question whether to transpose X ahead of the launches.
   if (p.opX == fastKronOp_T && !p.forward && useFusion()) {
     KronProblem pn;
     void* xt = nullptr;
@@ -210,6 +219,88 @@ fastKronError Handle::xgemm(KronProblem p, fastKronBackend backend, void* temp1,
     }
   }
   return runOnline(p, temp1, temp2, ws);
+}
+
+// Online rule for a GeKMM with op(X) = T: as the GeMKM of the same buffer plus a transposition of the result.
+// FASTKRON_KMM_VIA_MKM=0 / 1 forces the answer.
+bool Handle::viaMKMOnline(const KronProblem& p) const {
+  static const int forced = [] { const char* e = getenv("FASTKRON_KMM_VIA_MKM"); return e ? atoi(e) : -1; }();
+  if (p.L() >= (1ull << 32) || p.M < 2) return false;
+  if (forced >= 0) return forced != 0;
+  if (p.opX != fastKronOp_T) {
+    // X has to be transposed as well, two more passes over the data: fp32 with fewer than 64 columns, square factors up
+    // to 32x32 and at least 64 MB of X (sgekmm 16 x 8^8 2.91 -> 1.55 ms, 16 x 16^6 1.86 -> 1.55, 16 x 32^5 5.67 -> 4.36;
+    // 32 x 8^6, 33 MB: no difference, 48 x 16^4, 13 MB: 23 -> 37 us; fp64 loses 1.1 to 1.6 times)
+    if (p.dt != DType::F32 || p.M >= 64 || (uint64_t)p.M * p.K() * 4 < (64ull << 20)) return false;
+    for (uint32_t i = 0; i < p.N; i++) if (p.P[i] != p.Q[i] || p.P[i] > 32) return false;
+    return true;
+  }
+  // Measured on the reference's published shapes with both operands transposed.  Square factors up to 32x32 gain 1.3
+  // to 2.8 times in fp32 (sgekmm 1024 x 8^5 171 -> 112 us, 16 x 8^8 3.34 -> 1.20 ms) and up to 1.2 times in fp64.  With
+  // fewer than 64 columns the GeKMM kernels move short pieces and larger factors gain as well (sgekmm 16 x 64^4 and
+  // 16 x 128^3 1.27 times, fp64 up to 1.12 times); from 64 columns on, 64x64 and 128x128 factors are within 3 % in
+  // fp32 or lose up to 10 % (320 x 128^3), fp64 chains of three 64x64 factors gain 1.1 times.
+  uint32_t maxP = 0;
+  for (uint32_t i = 0; i < p.N; i++) {
+    if (p.P[i] != p.Q[i]) return false;
+    if (p.P[i] > maxP) maxP = p.P[i];
+  }
+  return maxP <= 32 || p.M < 64 || (p.dt == DType::F64 && maxP == 64 && p.N >= 3);
+}
+
+// Z (L x M) = transpose(R) + beta * Y with R (M x L) = alpha * X^T (F_1 (x) ... (x) F_N) computed by the GeMKM path
+// into temp1; the GeMKM uses temp2 and, when Z is free to be overwritten and large enough, Z as its temporaries.
+fastKronError Handle::runViaMKM(const KronProblem& p, fastKronBackend backend, void* temp1, void* temp2, const CallWorkspace* ws) {
+  size_t yElems = 0, tmpElems = 0;
+  if (sizes(p.M, p.N, p.P, p.Q, &yElems, &tmpElems) != fastKronSuccess) return fastKronKernelNotFound;
+  const uint64_t ML = (uint64_t)p.M * p.L();
+  KronProblem q = p;
+  q.mm = MMType::MKM;
+  q.opF = (p.opF == fastKronOp_N) ? fastKronOp_T : fastKronOp_N;      // KMM factors are stored Q x P
+  q.opX = fastKronOp_N;
+  q.Z = temp1; q.strideZ = p.batch > 1 ? ML : 0;
+  q.Y = nullptr; q.strideY = 0; q.beta = 0.0;
+  q.zReadNext = true;
+  const bool zFree = !(p.Y == p.Z && p.beta != 0.0);
+  void* zTemp = (zFree && tmpElems <= ML && (p.batch == 1 || p.strideZ >= ML)) ? p.Z : nullptr;
+  fastKronError e;
+  const bool copyX = p.opX != fastKronOp_T;
+  if (copyX) {
+    // X (K x M) goes to temp2 as M x K first; the GeMKM then has Z and, once its first launch has read it, temp2
+    const uint64_t MK = (uint64_t)p.M * p.K();
+    if (!zTemp || MK > tmpElems || p.K() >= (1ull << 32)) return fastKronKernelNotFound;
+    const uint32_t nb = (p.batch > 1 && p.strideX != 0) ? p.batch : 1;         // a shared X is transposed once
+    q.X = temp2; q.strideX = nb > 1 ? MK : 0; q.xJustWritten = true;
+    if (!planOnly_) {
+      constexpr uint32_t kMaxGridBatch = 65535;
+      const size_t es = dtypeSize(p.dt);
+      for (uint32_t b0 = 0; b0 < nb; b0 += kMaxGridBatch) {
+        const uint32_t n = nb - b0 < kMaxGridBatch ? nb - b0 : kMaxGridBatch;
+        if (launchTranspose((const char*)p.X + (size_t)b0 * p.strideX * es, (char*)temp2 + (size_t)b0 * MK * es, (uint32_t)p.K(), p.M, n,
+                            p.strideX, MK, p.dt, stream_) != hipSuccess) return fastKronInvalidArgument;
+      }
+    }
+    e = xgemm(q, backend, zTemp, temp2, ws);
+  } else {
+    e = xgemm(q, backend, temp2, zTemp, ws);
+  }
+  if (e != fastKronSuccess) return e;
+  const size_t semi = lastPlan_.find(';');
+  const std::string ty = p.dt == DType::F32 ? "f" : "d";
+  lastPlan_ = p.str() + (copyX ? ";" + std::to_string(p.N - 1) + "-" + std::to_string(p.N - 1) + ":transpose_hip_gfx950_256_" + ty + "_x" : "") +
+              (semi == std::string::npos ? "" : lastPlan_.substr(semi)) + ";0-0:transpose_hip_gfx950_256_" + ty + "_z";
+  if (planOnly_) return fastKronSuccess;
+  constexpr uint32_t kMaxGridBatch = 65535;
+  const size_t es = dtypeSize(p.dt);
+  const void* y = (p.beta != 0.0) ? p.Y : nullptr;
+  for (uint32_t b0 = 0; b0 < p.batch; b0 += kMaxGridBatch) {
+    const uint32_t n = p.batch - b0 < kMaxGridBatch ? p.batch - b0 : kMaxGridBatch;
+    hipError_t he = launchTransposeAdd((const char*)temp1 + (size_t)b0 * ML * es, (char*)p.Z + (size_t)b0 * p.strideZ * es, p.M,
+                                       (uint32_t)p.L(), n, ML, p.strideZ, y ? (const char*)y + (size_t)b0 * p.strideY * es : nullptr,
+                                       p.strideY, p.beta, p.dt, stream_);
+    if (he != hipSuccess) return fastKronInvalidArgument;
+  }
+  return fastKronSuccess;
 }
 
 // How many launches the last planned call makes (entries of lastPlan_).

@@ -62,6 +62,9 @@ class Handle {
   bool transposeFirstOnline(const KronProblem& p, const KronProblem& pn, void* temp1, void* temp2, const CallWorkspace* ws);
   hipError_t launchTransposeX(const KronProblem& p, void* xt, uint64_t xtStride);
   void noteTranspose(const KronProblem& p);
+  // GeKMM with op(X) = T as the GeMKM of the same buffer and a transposition of the result
+  bool viaMKMOnline(const KronProblem& p) const;
+  fastKronError runViaMKM(const KronProblem& p, fastKronBackend backend, void* temp1, void* temp2, const CallWorkspace* ws);
   bool lookupChoice(const KronProblem& p, Choice* c) const;
   fastKronError runChoice(const KronProblem& p, const Choice& c, void* temp1, void* temp2, const CallWorkspace* ws);
   bool buildSplit(const KronProblem& p, uint32_t g, void* temp1, void* temp2, KronProblem* q1, KronProblem* q2) const;

@@ -7,6 +7,9 @@
 // TR * TC = 4096): lanes run along c when reading (contiguous, or the whole tile contiguous when C <= 64) and along
 // r when writing (TR >= 64 contiguous elements); the LDS rows are padded by one element, so both sides are free of
 // bank conflicts.  Algorithmic traffic: R*C elements read and written.
+//
+// The same kernels finish a GeKMM that ran as the GeMKM of its transposed operands: out = transpose(in) + beta * Y,
+// Y laid out like out (HAS_Y).
 #include <hip/hip_runtime.h>
 #include "../problem.h"
 #include "launch.h"
@@ -15,16 +18,18 @@ namespace fk {
 
 constexpr int kTrTile = 4096;
 
-template <typename T>
-__global__ __launch_bounds__(256) void kron_transpose_kernel(const T* __restrict__ in, T* __restrict__ out, uint32_t R,
+template <typename T, bool HAS_Y>
+__global__ __launch_bounds__(256) void kron_transpose_kernel(const T* __restrict__ in, T* out, uint32_t R,
                                                              uint32_t C, uint32_t tcLog, uint32_t tilesC,
-                                                             uint64_t inBatch, uint64_t outBatch) {
+                                                             uint64_t inBatch, uint64_t outBatch, const T* y, uint64_t yBatch,
+                                                             T beta) {
   __shared__ T tile[kTrTile + kTrTile / 4];            // TR rows of TC + 1 elements, TC >= 4
   const uint32_t TC = 1u << tcLog, TR = kTrTile >> tcLog;
   const uint32_t tr = blockIdx.x / tilesC, tc = blockIdx.x % tilesC;
   const uint32_t r0 = tr * TR, c0 = tc * TC;
   const T* src = in + (size_t)blockIdx.y * inBatch;
   T* dst = out + (size_t)blockIdx.y * outBatch;
+  const T* ysrc = HAS_Y ? y + (size_t)blockIdx.y * yBatch : nullptr;
   for (uint32_t i = threadIdx.x; i < (uint32_t)kTrTile; i += 256) {
     const uint32_t r = i >> tcLog, c = i & (TC - 1);
     if (r0 + r < R && c0 + c < C) tile[r * (TC + 1) + c] = src[(size_t)(r0 + r) * C + c0 + c];
@@ -33,27 +38,35 @@ __global__ __launch_bounds__(256) void kron_transpose_kernel(const T* __restrict
   const uint32_t trLog = 12 - tcLog;
   for (uint32_t i = threadIdx.x; i < (uint32_t)kTrTile; i += 256) {
     const uint32_t c = i >> trLog, r = i & (TR - 1);
-    if (r0 + r < R && c0 + c < C) dst[(size_t)(c0 + c) * R + r0 + r] = tile[r * (TC + 1) + c];
+    if (r0 + r < R && c0 + c < C) {
+      T v = tile[r * (TC + 1) + c];
+      if (HAS_Y) v += beta * ysrc[(size_t)(c0 + c) * R + r0 + r];
+      dst[(size_t)(c0 + c) * R + r0 + r] = v;
+    }
   }
 }
 
-// The same with 16-byte global accesses and square tiles of TD x TD elements (128 x 128 in fp32, 64 x 64 in fp64:
-// 512-byte pieces on both sides), for R and C multiples of the vector length and 16-byte aligned buffers.  LDS rows
-// are TD + 1 elements, written and read element by element: a wave's writes go to (row, 4*c4 + k) with 16 lanes
-// along c4, its reads to (4*r4 + k, col) with 16 lanes along r4, both on 64 distinct banks.
-template <typename T, int TD>
-__global__ __launch_bounds__(TD == 128 ? 1024 : 256) void kron_transpose_vec_kernel(const T* __restrict__ in, T* __restrict__ out,
-                                                                                   uint32_t R, uint32_t C, uint32_t tilesC,
-                                                                                   uint64_t inBatch, uint64_t outBatch) {
-  constexpr int VE = 16 / sizeof(T), NTH = TD == 128 ? 1024 : 256, VPR = TD / VE;      // vectors per tile row
+// The same with 16-byte global accesses on tiles of TDR x TDC elements through LDS, for R and C multiples of the vector
+// length and 16-byte aligned buffers: 128 x 128 in fp32 and 64 x 64 in fp64 (512-byte pieces on both sides), and
+// tall or wide tiles of 16 KB for matrices with fewer than 64 rows or columns (16 or 32 columns: a tile is one
+// contiguous piece of the input and 16 or 32 contiguous pieces of the output; 16 or 32 rows: the reverse).  LDS rows
+// are TDC + 1 elements, written and read element by element.
+template <typename T, int TDR, int TDC, bool HAS_Y>
+__global__ __launch_bounds__(TDR * TDC * sizeof(T) >= 65536 ? 1024 : 256) void kron_transpose_vec_kernel(
+    const T* __restrict__ in, T* out, uint32_t R, uint32_t C, uint32_t tilesC, uint64_t inBatch, uint64_t outBatch, const T* y,
+    uint64_t yBatch, T beta) {
+  constexpr int VE = 16 / sizeof(T), NTH = TDR * TDC * sizeof(T) >= 65536 ? 1024 : 256;
+  constexpr int VPR = TDC / VE, VPC = TDR / VE;            // vectors per tile row (input side) / per tile column (output side)
   typedef T VT __attribute__((ext_vector_type(VE)));
   extern __shared__ __align__(16) unsigned char trLds[];
-  T* tile = (T*)trLds;                                                   // TD rows of TD + 1 elements
+  T* tile = (T*)trLds;                                                   // TDR rows of TDC + 1 elements
   const uint32_t tr = blockIdx.x / tilesC, tc = blockIdx.x % tilesC;
-  const uint32_t r0 = tr * TD, c0 = tc * TD;
+  const uint32_t r0 = tr * TDR, c0 = tc * TDC;
   const T* src = in + (size_t)blockIdx.y * inBatch;
   T* dst = out + (size_t)blockIdx.y * outBatch;
-  constexpr int PER = TD * VPR / NTH;
+  const T* ysrc = HAS_Y ? y + (size_t)blockIdx.y * yBatch : nullptr;
+  constexpr int PER = TDR * VPR / NTH;
+  static_assert(TDR * VPR % NTH == 0 && PER >= 1, "whole vectors per thread");
   VT v[PER];
 #pragma unroll
   for (int i = 0; i < PER; i++) {
@@ -66,47 +79,55 @@ __global__ __launch_bounds__(TD == 128 ? 1024 : 256) void kron_transpose_vec_ker
   for (int i = 0; i < PER; i++) {
     const uint32_t idx = threadIdx.x + i * NTH, row = idx / VPR, c4 = idx % VPR;
 #pragma unroll
-    for (int k = 0; k < VE; k++) tile[row * (TD + 1) + VE * c4 + k] = v[i][k];
+    for (int k = 0; k < VE; k++) tile[row * (TDC + 1) + VE * c4 + k] = v[i][k];
   }
   __syncthreads();
 #pragma unroll
   for (int i = 0; i < PER; i++) {
-    const uint32_t idx = threadIdx.x + i * NTH, col = idx / VPR, r4 = idx % VPR;
+    const uint32_t idx = threadIdx.x + i * NTH, col = idx / VPC, r4 = idx % VPC;
     VT o;
 #pragma unroll
-    for (int k = 0; k < VE; k++) o[k] = tile[(VE * r4 + k) * (TD + 1) + col];
-    if (c0 + col < C && r0 + VE * r4 < R) *(VT*)(dst + (size_t)(c0 + col) * R + r0 + VE * r4) = o;
+    for (int k = 0; k < VE; k++) o[k] = tile[(VE * r4 + k) * (TDC + 1) + col];
+    if (c0 + col < C && r0 + VE * r4 < R) {
+      if (HAS_Y) o += beta * *(const VT*)(ysrc + (size_t)(c0 + col) * R + r0 + VE * r4);
+      *(VT*)(dst + (size_t)(c0 + col) * R + r0 + VE * r4) = o;
+    }
   }
 }
 
-template <typename T, int TD>
+template <typename T, int TDR, int TDC, bool HAS_Y>
 static hipError_t launchTransposeVec(const void* in, void* out, uint32_t R, uint32_t C, uint32_t batch, uint64_t inBatch,
-                                     uint64_t outBatch, hipStream_t stream) {
-  const uint64_t tilesC = (C + TD - 1) / TD, tilesR = (R + TD - 1) / TD;
+                                     uint64_t outBatch, const void* y, uint64_t yBatch, double beta, hipStream_t stream) {
+  const uint64_t tilesC = (C + TDC - 1) / TDC, tilesR = (R + TDR - 1) / TDR;
   if (tilesC * tilesR >= (1ull << 31)) return hipErrorInvalidValue;
-  const size_t lds = (size_t)TD * (TD + 1) * sizeof(T);
+  const size_t lds = (size_t)TDR * (TDC + 1) * sizeof(T);
   static PerDeviceOnce attrOnce;
   const int devIdx = launchDeviceIndex();
   if (!attrOnce.done(devIdx)) {
-    hipError_t e = hipFuncSetAttribute((const void*)kron_transpose_vec_kernel<T, TD>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipError_t e = hipFuncSetAttribute((const void*)kron_transpose_vec_kernel<T, TDR, TDC, HAS_Y>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
     attrOnce.mark(devIdx);
   }
-  dim3 grid((uint32_t)(tilesC * tilesR), batch), block(TD == 128 ? 1024 : 256);
-  hipLaunchKernelGGL((kron_transpose_vec_kernel<T, TD>), grid, block, lds, stream, (const T*)in, (T*)out, R, C, (uint32_t)tilesC,
-                     inBatch, outBatch);
+  dim3 grid((uint32_t)(tilesC * tilesR), batch), block(TDR * TDC * sizeof(T) >= 65536 ? 1024 : 256);
+  hipLaunchKernelGGL((kron_transpose_vec_kernel<T, TDR, TDC, HAS_Y>), grid, block, lds, stream, (const T*)in, (T*)out, R, C,
+                     (uint32_t)tilesC, inBatch, outBatch, (const T*)y, yBatch, (T)beta);
   return hipGetLastError();
 }
 
-hipError_t launchTranspose(const void* in, void* out, uint32_t R, uint32_t C, uint32_t batch, uint64_t inBatch,
-                           uint64_t outBatch, DType dt, hipStream_t stream) {
-  if (R == 0 || C == 0 || batch == 0 || batch > 65535) return hipErrorInvalidValue;
-  {
-    const uint32_t ve = dt == DType::F32 ? 4 : 2;
-    const bool vec = R % ve == 0 && C % ve == 0 && R >= 64 && C >= 64 && (((uintptr_t)in | (uintptr_t)out) & 15) == 0 &&
-                     inBatch % ve == 0 && outBatch % ve == 0;
-    if (vec) return dt == DType::F32 ? launchTransposeVec<float, 128>(in, out, R, C, batch, inBatch, outBatch, stream)
-                                     : launchTransposeVec<double, 64>(in, out, R, C, batch, inBatch, outBatch, stream);
+template <typename T, bool HAS_Y>
+static hipError_t launchTransposeT(const void* in, void* out, uint32_t R, uint32_t C, uint32_t batch, uint64_t inBatch,
+                                   uint64_t outBatch, const void* y, uint64_t yBatch, double beta, hipStream_t stream) {
+  constexpr uint32_t ve = 16 / sizeof(T);
+  const bool vec = R % ve == 0 && C % ve == 0 && (((uintptr_t)in | (uintptr_t)out) & 15) == 0 && inBatch % ve == 0 &&
+                   outBatch % ve == 0 && (!HAS_Y || (((uintptr_t)y & 15) == 0 && yBatch % ve == 0));
+  if (vec) {
+    constexpr int SQ = sizeof(T) == 4 ? 128 : 64, E = 16384 / sizeof(T);      // square tile edge; elements of a 16 KB tile
+#define FK_TR(TDR, TDC) launchTransposeVec<T, TDR, TDC, HAS_Y>(in, out, R, C, batch, inBatch, outBatch, y, yBatch, beta, stream)
+    if (R >= 64 && C >= 64) return FK_TR(SQ, SQ);
+    if (C < 64 && C >= 8 && R >= 256) return C <= 16 ? FK_TR(E / 16, 16) : FK_TR(E / 32, 32);
+    if (R < 64 && R >= 8 && C >= 256) return R <= 16 ? FK_TR(16, E / 16) : FK_TR(32, E / 32);
+#undef FK_TR
   }
   uint32_t tcLog = 2;
   while (tcLog < 6 && (1u << tcLog) < C) tcLog++;
@@ -114,13 +135,26 @@ hipError_t launchTranspose(const void* in, void* out, uint32_t R, uint32_t C, ui
   const uint64_t tilesC = (C + TC - 1) / TC, tilesR = (R + TR - 1) / TR;
   if (tilesC * tilesR >= (1ull << 31)) return hipErrorInvalidValue;
   dim3 grid((uint32_t)(tilesC * tilesR), batch), block(256);
-  if (dt == DType::F32)
-    hipLaunchKernelGGL(kron_transpose_kernel<float>, grid, block, 0, stream, (const float*)in, (float*)out, R, C, tcLog,
-                       (uint32_t)tilesC, inBatch, outBatch);
-  else
-    hipLaunchKernelGGL(kron_transpose_kernel<double>, grid, block, 0, stream, (const double*)in, (double*)out, R, C, tcLog,
-                       (uint32_t)tilesC, inBatch, outBatch);
+  hipLaunchKernelGGL((kron_transpose_kernel<T, HAS_Y>), grid, block, 0, stream, (const T*)in, (T*)out, R, C, tcLog,
+                     (uint32_t)tilesC, inBatch, outBatch, (const T*)y, yBatch, (T)beta);
   return hipGetLastError();
+}
+
+// out (C x R) = transpose(in (R x C)) + beta * y (y null: the plain transposed copy), per batch entry
+hipError_t launchTransposeAdd(const void* in, void* out, uint32_t R, uint32_t C, uint32_t batch, uint64_t inBatch,
+                              uint64_t outBatch, const void* y, uint64_t yBatch, double beta, DType dt, hipStream_t stream) {
+  if (R == 0 || C == 0 || batch == 0 || batch > 65535) return hipErrorInvalidValue;
+  const bool hasY = y != nullptr && beta != 0.0;
+  if (dt == DType::F32)
+    return hasY ? launchTransposeT<float, true>(in, out, R, C, batch, inBatch, outBatch, y, yBatch, beta, stream)
+                : launchTransposeT<float, false>(in, out, R, C, batch, inBatch, outBatch, nullptr, 0, 0.0, stream);
+  return hasY ? launchTransposeT<double, true>(in, out, R, C, batch, inBatch, outBatch, y, yBatch, beta, stream)
+              : launchTransposeT<double, false>(in, out, R, C, batch, inBatch, outBatch, nullptr, 0, 0.0, stream);
+}
+
+hipError_t launchTranspose(const void* in, void* out, uint32_t R, uint32_t C, uint32_t batch, uint64_t inBatch,
+                           uint64_t outBatch, DType dt, hipStream_t stream) {
+  return launchTransposeAdd(in, out, R, C, batch, inBatch, outBatch, nullptr, 0, 0.0, dt, stream);
 }
 
 }  // namespace fk

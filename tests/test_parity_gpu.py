@@ -88,9 +88,45 @@ def test_transposed_x_ahead_of_the_whole_row_kernels(fk, mm, M, Ps, dt):
         # KMM layout, a copy that saves no launch: the padded step reads the transposed X in the first launch instead
         assert not plan[0][2].startswith("transpose_"), plan
         return
-    assert plan[0][2].startswith("transpose_"), plan
+    if mm == ko.KMM:
+        # small factors: the GeKMM runs as the GeMKM of the transposed buffer, the result is transposed into Z
+        assert plan[0][2].startswith("mkm_") and plan[-1][2].endswith("_z"), plan
+    else:
+        assert plan[0][2].startswith("transpose_"), plan
     check(fk, mm, M, Ps, Ps, dt, alpha=1.0, beta=0.0, seed=72, opX=ko.OP_T, opFs=ko.OP_N, batch=3, share_f=True)
     check(fk, mm, M, Ps, Ps, dt, alpha=1.0, beta=1.0, seed=73, opX=ko.OP_T, opFs=ko.OP_N, batch=2)
+
+
+@pytest.mark.parametrize("M,Ps,dt", [(64, [8] * 5, np.float32), (16, [8] * 3, np.float32), (100, [16] * 3, np.float32),
+                                     (3, [16] * 4, np.float32), (256, [32] * 3, np.float32), (64, [16] * 3, np.float64),
+                                     (68, [8] * 4, np.float64), (128, [4, 8, 16], np.float32), (20, [8] * 6, np.float32)])
+def test_gekmm_with_transposed_x_as_gemkm(fk, M, Ps, dt):
+    """GeKMM with op(X) = T and square factors up to 32x32: the buffer is the X of a GeMKM with transposed factors; the
+    whole-row GeMKM kernels run on it and one transposition, which also adds beta * Y, writes Z (column counts with and
+    without whole 16-byte tiles, chains that need the two-part plan, batches, shared factors and a shared Y)."""
+    check(fk, ko.KMM, M, Ps, Ps, dt, alpha=1.5, beta=0.5, seed=81, opX=ko.OP_T, opFs=ko.OP_T)
+    plan = fk.last_plan()
+    assert not plan[0][2].startswith(("transpose_", "kmm_")) and plan[-1][2].endswith("_z"), plan
+    check(fk, ko.KMM, M, Ps, Ps, dt, alpha=2.0, beta=0.0, seed=82, opX=ko.OP_T, opFs=ko.OP_N)
+    assert fk.last_plan()[-1][2].endswith("_z"), fk.last_plan()
+    check(fk, ko.KMM, M, Ps, Ps, dt, alpha=1.0, beta=1.0, seed=83, opX=ko.OP_T, opFs=ko.OP_N, batch=3, share_f=True)
+    assert fk.last_plan()[-1][2].endswith("_z"), fk.last_plan()
+    check(fk, ko.KMM, M, Ps, Ps, dt, alpha=1.0, beta=-1.0, seed=84, opX=ko.OP_T, opFs=ko.OP_T, batch=2, share_y=True)
+    check(fk, ko.KMM, M, Ps, Ps, dt, alpha=1.0, beta=1.0, seed=85, opX=ko.OP_T, opFs=ko.OP_N, integer=True)
+    # without a second temporary the call keeps to the GeKMM kernels
+    check(fk, ko.KMM, M, Ps, Ps, dt, alpha=1.0, beta=0.5, seed=86, opX=ko.OP_T, opFs=ko.OP_N, use_temp2=False)
+    assert not fk.last_plan()[-1][2].endswith("_z"), fk.last_plan()
+
+
+@pytest.mark.parametrize("M,Ps", [(16, [8] * 7), (20, [16] * 5)])
+def test_large_gekmm_with_few_columns_as_gemkm(fk, M, Ps):
+    """fp32 GeKMM with fewer than 64 columns, square factors up to 32x32 and 64 MB of X or more: X is transposed into a
+    temporary, the GeMKM kernels run on it and the result is transposed into Z (with beta * Y)."""
+    check(fk, ko.KMM, M, Ps, Ps, np.float32, alpha=1.5, beta=0.5, seed=91)
+    plan = fk.last_plan()
+    assert plan[0][2].endswith("_x") and plan[-1][2].endswith("_z"), plan
+    check(fk, ko.KMM, M, Ps, Ps, np.float32, alpha=1.0, beta=0.0, seed=92, opFs=ko.OP_T)
+    assert fk.last_plan()[-1][2].endswith("_z"), fk.last_plan()
 
 
 @pytest.mark.parametrize("mm", [ko.MKM, ko.KMM])

@@ -231,8 +231,49 @@ def test_transposed_x_is_copied_first_when_the_whole_row_kernels_then_apply(plan
     # the same for the two-part plan of a longer chain and for GeKMM
     e, names, _ = plan(planner, "mkm", "s", 8, [16] * 5, [16] * 5, opX=capi.OP_T)
     assert e == capi.SUCCESS and names[0].startswith("transpose_") and len(names) == 3, names
-    e, names, _ = plan(planner, "kmm", "s", 64, [4] * 6, [4] * 6, opX=capi.OP_T)
-    assert e == capi.SUCCESS and names[0].startswith("transpose_") and "_4x4_4x4_6_8x4096" in names[1], names
+    # GeKMM with 64x64 factors (with small factors it runs as a GeMKM, below)
+    e, names, _ = plan(planner, "kmm", "s", 64, [64] * 2, [64] * 2, opX=capi.OP_T)
+    assert e == capi.SUCCESS and names[0].startswith("transpose_") and names[0].endswith("_x") and len(names) == 3, names
+
+
+def test_gekmm_with_transposed_x_runs_as_the_gemkm_of_that_buffer(online_planner):
+    """op(X) = T in a GeKMM means the buffer holds M x K, the X of a GeMKM with transposed factors: the whole-row GeMKM
+    kernels run on it, their result goes to temp1 and one transposition (with beta * Y) writes Z."""
+    planner = online_planner
+    e, names, launches = plan(planner, "kmm", "s", 64, [8] * 5, [8] * 5, opX=capi.OP_T, beta=0.5, with_y=True)
+    assert e == capi.SUCCESS and "mkm_" in names[0] and "_8x8_8x8_5_1x32768" in names[0] and names[-1].endswith("_z"), names
+    assert len(names) == 2 and len(launches) == 1
+    # the launch reads the caller's X, writes temp1, and leaves alpha in and beta * Y out
+    assert int(launches[0]["in"], 16) == BASE and int(launches[0]["out"], 16) == BASE + 3 * GAP
+    assert launches[0]["y"] == "(nil)"
+    # a longer chain: the two-part GeMKM plan, with temp2 and Z as its temporaries
+    e, names, launches = plan(planner, "kmm", "s", 1024, [8] * 6, [8] * 6, opX=capi.OP_T)
+    assert e == capi.SUCCESS and len(names) == 3 and names[-1].endswith("_z"), names
+    assert int(launches[-1]["out"], 16) == BASE + 3 * GAP
+    # Y in place (Y == Z, beta != 0): Z cannot serve as a temporary
+    e, names, launches = plan(planner, "kmm", "s", 1024, [8] * 6, [8] * 6, opX=capi.OP_T, beta=1.0, y_is_z=True)
+    assert e == capi.SUCCESS and names[-1].endswith("_z"), names
+    assert all(int(r["out"], 16) != BASE + GAP for r in launches), launches
+    # 64x64 factors and larger only with fewer than 64 columns (and fp64 chains of three 64x64 factors)
+    e, names, _ = plan(planner, "kmm", "s", 1024, [64] * 2, [64] * 2, opX=capi.OP_T)
+    assert e == capi.SUCCESS and not names[-1].endswith("_z"), names
+    e, names, _ = plan(planner, "kmm", "s", 16, [128] * 3, [128] * 3, opX=capi.OP_T)
+    assert e == capi.SUCCESS and names[-1].endswith("_z"), names
+    e, names, _ = plan(planner, "kmm", "d", 256, [64] * 3, [64] * 3, opX=capi.OP_T)
+    assert e == capi.SUCCESS and names[-1].endswith("_z"), names
+    e, names, _ = plan(planner, "kmm", "d", 16, [8] * 5, [8] * 5, opX=capi.OP_T)
+    assert e == capi.SUCCESS and names[-1].endswith("_z"), names
+    # X not transposed: only large fp32 problems with fewer than 64 columns go this way, X transposed into temp2 first
+    e, names, launches = plan(planner, "kmm", "s", 16, [8] * 8, [8] * 8)
+    assert e == capi.SUCCESS and names[0].endswith("_x") and names[-1].endswith("_z") and len(names) == 4, names
+    assert int(launches[0]["in"], 16) == BASE + 4 * GAP and int(launches[-1]["out"], 16) == BASE + 3 * GAP, launches
+    e, names, _ = plan(planner, "kmm", "s", 48, [16] * 4, [16] * 4)
+    assert e == capi.SUCCESS and not names[-1].endswith("_z"), names
+    e, names, _ = plan(planner, "kmm", "d", 16, [8] * 8, [8] * 8)
+    assert e == capi.SUCCESS and not names[-1].endswith("_z"), names
+    # rectangular factors stay on the GeKMM kernels
+    e, names, _ = plan(planner, "kmm", "s", 256, [32] * 3, [16] * 3, opX=capi.OP_T)
+    assert e == capi.SUCCESS and not names[-1].endswith("_z"), names
 
 
 def test_transposed_x_is_read_in_place_when_a_copy_does_not_pay_or_does_not_fit(planner):
@@ -263,9 +304,9 @@ def test_transposition_rules_that_came_from_tuned_plans(online_planner):
     e, names, _ = plan(planner, "kmm", "s", 320, [128] * 3, [128] * 3, opX=capi.OP_T)
     assert e == capi.SUCCESS and not copied(names) and len(names) == 3, names
     # equal launch counts: the copy goes first, except in the KMM layout with fewer than 64 columns
-    e, names, _ = plan(planner, "kmm", "s", 256, [16] * 4, [16] * 4, opX=capi.OP_T)
-    assert e == capi.SUCCESS and copied(names) and len(names) == 3, names
-    e, names, _ = plan(planner, "kmm", "s", 16, [16] * 6, [16] * 6, opX=capi.OP_T)
+    e, names, _ = plan(planner, "mkm", "d", 256, [16] * 4, [16] * 4, opX=capi.OP_T)
+    assert e == capi.SUCCESS and copied(names), names
+    e, names, _ = plan(planner, "kmm", "d", 16, [16] * 6, [16] * 6, opX=capi.OP_T)
     assert e == capi.SUCCESS and not copied(names), names
 
 
