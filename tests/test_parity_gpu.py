@@ -342,6 +342,36 @@ def test_one_misaligned_operand_at_a_time(fk, which, M, Ps, dt):
     assert normwise(Z.cpu().numpy(), want) <= TOL[dt], (which, fk.last_plan())
 
 
+@pytest.mark.parametrize("which", ["none", "y", "z"])
+def test_32x16_row_kernel_with_results_off_16_byte_boundaries(fk, which):
+    """The 32x16^3 row kernel writes Z and reads Y 16 bytes per lane when their rows start on 16-byte boundaries, element
+    by element otherwise: either way one launch and the right answer."""
+    import torch
+    M, Ps, Qs = 6, [32] * 3, [16] * 3
+    K, L = 32768, 4096
+    X, Fs, Y = make_case(ko.MKM, M, Ps, Qs, np.float32, seed=63, with_y=True)
+    want = oracle_answer(ko.MKM, M, Ps, Qs, X, Fs, Y, 1.5, 0.5)
+    dev = "cuda:0"
+
+    def place(host, shifted):
+        buf = torch.full((host.size + 64,), float("nan"), dtype=torch.float32, device=dev)
+        v = buf[1:1 + host.size] if shifted else buf[:host.size]
+        v.copy_(torch.from_numpy(host.reshape(-1)))
+        return v
+
+    tX, tY = place(X, False), place(Y, which == "y")
+    Z = place(np.full(M * L, np.nan, np.float32), which == "z")
+    tFs = [torch.from_numpy(f).to(dev) for f in Fs]
+    t1 = torch.empty(M * K, dtype=torch.float32, device=dev)
+    t2 = torch.empty(M * K, dtype=torch.float32, device=dev)
+    e = fk.xgemkm(M, Ps, Qs, tX, tFs, Z, 1.5, 0.5, tY, t1, t2)
+    torch.cuda.synchronize()
+    assert e == 0
+    plan = fk.last_plan()
+    assert len(plan) == 1 and "32x16" in plan[0][2], plan
+    assert normwise(Z.cpu().numpy(), want) <= TOL[np.float32], (which, plan)
+
+
 @pytest.mark.parametrize("M,Ps,dt", [(8, [16] * 5, np.float32), (4, [8] * 6, np.float32), (2, [32] * 4, np.float32),
                                      (8, [16] * 4, np.float64), (2, [64] * 3, np.float64), (16, [4] * 8, np.float32),
                                      (4, [8] * 5, np.float64), (3, [4, 4] + [8] * 5, np.float32)])
