@@ -1,4 +1,4 @@
-"""GPU parity at the full sizes of the five benchmark configurations (and of two more shapes large enough for their
+"""GPU parity at the full sizes of the five benchmark configurations (and of three more shapes large enough for their
 kernels' streaming stores), where the oracle cannot answer the whole problem in seconds.  Two checks per configuration, both against the oracle and both through the C ABI:
 
 * sampled rows (MKM) / columns (KMM): every row of X is an independent chain, so the oracle's answer for a few
@@ -31,9 +31,10 @@ FULL = [
     ("c3", ko.MKM, 256, [64] * 3, [64] * 3, np.float64, 1.0, 0.0, 1),
     ("c4", ko.KMM, 2048, [4] * 6, [4] * 6, np.float32, 1.5, 0.5, 1),
     ("c5", ko.MKM, 512, [32] * 3, [16] * 3, np.float32, 1.0, 1.0, 8),
-    # sizes at which two more kernels stream their results (system-scope 16-byte stores)
+    # sizes at which three more kernels stream their results (system-scope 16-byte stores)
     ("16x16^3 on 8192 rows", ko.MKM, 8192, [16] * 3, [16] * 3, np.float32, 1.5, 0.5, 1),
     ("32x32^3 on 2048 rows", ko.MKM, 2048, [32] * 3, [32] * 3, np.float32, 1.0, 0.0, 1),
+    ("KMM 32x32^3 on 1024 columns", ko.KMM, 1024, [32] * 3, [32] * 3, np.float32, 2.0, 0.0, 1),
 ]
 
 
