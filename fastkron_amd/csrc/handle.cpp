@@ -293,11 +293,13 @@ fastKronError Handle::runViaMKM(const KronProblem& p, fastKronBackend backend, v
   constexpr uint32_t kMaxGridBatch = 65535;
   const size_t es = dtypeSize(p.dt);
   const void* y = (p.beta != 0.0) ? p.Y : nullptr;
+  // Z goes to the caller: streamed from the size on at which the kernels stream their results (Handle::execute)
+  const bool streamZ = !p.zReadNext && (uint64_t)(y ? 3 : 2) * ML * p.batch * es >= (96ull << 20);
   for (uint32_t b0 = 0; b0 < p.batch; b0 += kMaxGridBatch) {
     const uint32_t n = p.batch - b0 < kMaxGridBatch ? p.batch - b0 : kMaxGridBatch;
     hipError_t he = launchTransposeAdd((const char*)temp1 + (size_t)b0 * ML * es, (char*)p.Z + (size_t)b0 * p.strideZ * es, p.M,
                                        (uint32_t)p.L(), n, ML, p.strideZ, y ? (const char*)y + (size_t)b0 * p.strideY * es : nullptr,
-                                       p.strideY, p.beta, p.dt, stream_);
+                                       p.strideY, p.beta, p.dt, stream_, streamZ);
     if (he != hipSuccess) return fastKronInvalidArgument;
   }
   return fastKronSuccess;

@@ -145,7 +145,8 @@ hipError_t launchMergeFactors(const MergeArgs& a, DType dt, hipStream_t stream);
 hipError_t launchTranspose(const void* in, void* out, uint32_t R, uint32_t C, uint32_t batch, uint64_t inBatch,
                            uint64_t outBatch, DType dt, hipStream_t stream);
 hipError_t launchTransposeAdd(const void* in, void* out, uint32_t R, uint32_t C, uint32_t batch, uint64_t inBatch,
-                              uint64_t outBatch, const void* y, uint64_t yBatch, double beta, DType dt, hipStream_t stream);
+                              uint64_t outBatch, const void* y, uint64_t yBatch, double beta, DType dt, hipStream_t stream,
+                              bool streamOut);
 // Fills `elems` elements with values spread over [-1, 1] (data for the tuner's timing runs).
 hipError_t launchFill(void* dst, size_t elems, DType dt, hipStream_t stream);
 

@@ -51,7 +51,9 @@ __global__ __launch_bounds__(256) void kron_transpose_kernel(const T* __restrict
 // tall or wide tiles of 16 KB for matrices with fewer than 64 rows or columns (16 or 32 columns: a tile is one
 // contiguous piece of the input and 16 or 32 contiguous pieces of the output; 16 or 32 rows: the reverse).  LDS rows
 // are TDC + 1 elements, written and read element by element.
-template <typename T, int TDR, int TDC, bool HAS_Y>
+// STREAM: the result goes to the caller and nothing reads it back soon: stores at system scope (launch.h), through a
+// descriptor of the tile's span of the output (the launcher checks that it stays below 2 GB).
+template <typename T, int TDR, int TDC, bool HAS_Y, bool STREAM>
 __global__ __launch_bounds__(TDR * TDC * sizeof(T) >= 65536 ? 1024 : 256) void kron_transpose_vec_kernel(
     const T* __restrict__ in, T* out, uint32_t R, uint32_t C, uint32_t tilesC, uint64_t inBatch, uint64_t outBatch, const T* y,
     uint64_t yBatch, T beta) {
@@ -67,6 +69,8 @@ __global__ __launch_bounds__(TDR * TDC * sizeof(T) >= 65536 ? 1024 : 256) void k
   const T* ysrc = HAS_Y ? y + (size_t)blockIdx.y * yBatch : nullptr;
   constexpr int PER = TDR * VPR / NTH;
   static_assert(TDR * VPR % NTH == 0 && PER >= 1, "whole vectors per thread");
+  const __amdgpu_buffer_rsrc_t oTarget =
+      streamTarget((void*)(dst + (size_t)c0 * R + r0), STREAM ? (uint32_t)(((size_t)(TDC - 1) * R + TDR) * sizeof(T)) : 0u);
   VT v[PER];
 #pragma unroll
   for (int i = 0; i < PER; i++) {
@@ -90,12 +94,13 @@ __global__ __launch_bounds__(TDR * TDC * sizeof(T) >= 65536 ? 1024 : 256) void k
     for (int k = 0; k < VE; k++) o[k] = tile[(VE * r4 + k) * (TDC + 1) + col];
     if (c0 + col < C && r0 + VE * r4 < R) {
       if (HAS_Y) o += beta * *(const VT*)(ysrc + (size_t)(c0 + col) * R + r0 + VE * r4);
-      *(VT*)(dst + (size_t)(c0 + col) * R + r0 + VE * r4) = o;
+      if constexpr (STREAM) streamStore16(o, oTarget, (uint32_t)(((size_t)col * R + VE * r4) * sizeof(T)));
+      else *(VT*)(dst + (size_t)(c0 + col) * R + r0 + VE * r4) = o;
     }
   }
 }
 
-template <typename T, int TDR, int TDC, bool HAS_Y>
+template <typename T, int TDR, int TDC, bool HAS_Y, bool STREAM>
 static hipError_t launchTransposeVec(const void* in, void* out, uint32_t R, uint32_t C, uint32_t batch, uint64_t inBatch,
                                      uint64_t outBatch, const void* y, uint64_t yBatch, double beta, hipStream_t stream) {
   const uint64_t tilesC = (C + TDC - 1) / TDC, tilesR = (R + TDR - 1) / TDR;
@@ -104,18 +109,18 @@ static hipError_t launchTransposeVec(const void* in, void* out, uint32_t R, uint
   static PerDeviceOnce attrOnce;
   const int devIdx = launchDeviceIndex();
   if (!attrOnce.done(devIdx)) {
-    hipError_t e = hipFuncSetAttribute((const void*)kron_transpose_vec_kernel<T, TDR, TDC, HAS_Y>,
+    hipError_t e = hipFuncSetAttribute((const void*)kron_transpose_vec_kernel<T, TDR, TDC, HAS_Y, STREAM>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
     attrOnce.mark(devIdx);
   }
   dim3 grid((uint32_t)(tilesC * tilesR), batch), block(TDR * TDC * sizeof(T) >= 65536 ? 1024 : 256);
-  hipLaunchKernelGGL((kron_transpose_vec_kernel<T, TDR, TDC, HAS_Y>), grid, block, lds, stream, (const T*)in, (T*)out, R, C,
+  hipLaunchKernelGGL((kron_transpose_vec_kernel<T, TDR, TDC, HAS_Y, STREAM>), grid, block, lds, stream, (const T*)in, (T*)out, R, C,
                      (uint32_t)tilesC, inBatch, outBatch, (const T*)y, yBatch, (T)beta);
   return hipGetLastError();
 }
 
-template <typename T, bool HAS_Y>
+template <typename T, bool HAS_Y, bool STREAM>
 static hipError_t launchTransposeT(const void* in, void* out, uint32_t R, uint32_t C, uint32_t batch, uint64_t inBatch,
                                    uint64_t outBatch, const void* y, uint64_t yBatch, double beta, hipStream_t stream) {
   constexpr uint32_t ve = 16 / sizeof(T);
@@ -123,7 +128,7 @@ static hipError_t launchTransposeT(const void* in, void* out, uint32_t R, uint32
                    outBatch % ve == 0 && (!HAS_Y || (((uintptr_t)y & 15) == 0 && yBatch % ve == 0));
   if (vec) {
     constexpr int SQ = sizeof(T) == 4 ? 128 : 64, E = 16384 / sizeof(T);      // square tile edge; elements of a 16 KB tile
-#define FK_TR(TDR, TDC) launchTransposeVec<T, TDR, TDC, HAS_Y>(in, out, R, C, batch, inBatch, outBatch, y, yBatch, beta, stream)
+#define FK_TR(TDR, TDC) launchTransposeVec<T, TDR, TDC, HAS_Y, STREAM>(in, out, R, C, batch, inBatch, outBatch, y, yBatch, beta, stream)
     if (R >= 64 && C >= 64) return FK_TR(SQ, SQ);
     if (C < 64 && C >= 8 && R >= 256) return C <= 16 ? FK_TR(E / 16, 16) : FK_TR(E / 32, 32);
     if (R < 64 && R >= 8 && C >= 256) return R <= 16 ? FK_TR(16, E / 16) : FK_TR(32, E / 32);
@@ -140,21 +145,26 @@ static hipError_t launchTransposeT(const void* in, void* out, uint32_t R, uint32
   return hipGetLastError();
 }
 
-// out (C x R) = transpose(in (R x C)) + beta * y (y null: the plain transposed copy), per batch entry
+// out (C x R) = transpose(in (R x C)) + beta * y (y null: the plain transposed copy), per batch entry; streamOut: the
+// result is not read back soon (stores at system scope where the kernel with 16-byte accesses applies)
 hipError_t launchTransposeAdd(const void* in, void* out, uint32_t R, uint32_t C, uint32_t batch, uint64_t inBatch,
-                              uint64_t outBatch, const void* y, uint64_t yBatch, double beta, DType dt, hipStream_t stream) {
+                              uint64_t outBatch, const void* y, uint64_t yBatch, double beta, DType dt, hipStream_t stream,
+                              bool streamOut) {
   if (R == 0 || C == 0 || batch == 0 || batch > 65535) return hipErrorInvalidValue;
   const bool hasY = y != nullptr && beta != 0.0;
-  if (dt == DType::F32)
-    return hasY ? launchTransposeT<float, true>(in, out, R, C, batch, inBatch, outBatch, y, yBatch, beta, stream)
-                : launchTransposeT<float, false>(in, out, R, C, batch, inBatch, outBatch, nullptr, 0, 0.0, stream);
-  return hasY ? launchTransposeT<double, true>(in, out, R, C, batch, inBatch, outBatch, y, yBatch, beta, stream)
-              : launchTransposeT<double, false>(in, out, R, C, batch, inBatch, outBatch, nullptr, 0, 0.0, stream);
+  // a tile's span of the output, (tile columns) x R elements, has to stay below 2 GB for the descriptor's offsets
+  const bool so = streamOut && (uint64_t)1024 * R * dtypeSize(dt) < (1ull << 31);
+#define FK_TRT(T) (hasY ? (so ? launchTransposeT<T, true, true>(in, out, R, C, batch, inBatch, outBatch, y, yBatch, beta, stream)      \
+                              : launchTransposeT<T, true, false>(in, out, R, C, batch, inBatch, outBatch, y, yBatch, beta, stream))    \
+                        : (so ? launchTransposeT<T, false, true>(in, out, R, C, batch, inBatch, outBatch, nullptr, 0, 0.0, stream)    \
+                              : launchTransposeT<T, false, false>(in, out, R, C, batch, inBatch, outBatch, nullptr, 0, 0.0, stream)))
+  return dt == DType::F32 ? FK_TRT(float) : FK_TRT(double);
+#undef FK_TRT
 }
 
 hipError_t launchTranspose(const void* in, void* out, uint32_t R, uint32_t C, uint32_t batch, uint64_t inBatch,
                            uint64_t outBatch, DType dt, hipStream_t stream) {
-  return launchTransposeAdd(in, out, R, C, batch, inBatch, outBatch, nullptr, 0, 0.0, dt, stream);
+  return launchTransposeAdd(in, out, R, C, batch, inBatch, outBatch, nullptr, 0, 0.0, dt, stream, false);
 }
 
 }  // namespace fk
