@@ -89,6 +89,31 @@ def test_full_size_configuration(fk, name, mm, M, Ps, Qs, dt, alpha, beta, batch
         assert err <= TOL[dt], f"batch {b}: checksum over all chains off by {err:.3e}"
 
 
+@pytest.mark.parametrize("M,Ps,dt", [(1024, [8] * 5, np.float32), (16, [8] * 7, np.float32), (1024, [16] * 3, np.float64)])
+def test_full_size_gekmm_with_transposed_x(fk, M, Ps, dt):
+    """GeKMM with op(X) = T at sizes where the final transposition streams Z: sampled columns and the checksum over all
+    columns against the oracle (X is stored M x K, Z and Y are L x M)."""
+    from tests.gpu_util import oracle_answer
+    K = int(np.prod(Ps))
+    alpha, beta = 1.5, 0.5
+    X = seeded(21, (M * K,), dt)
+    Fs = [seeded(22 + i, (p * p,), dt) for i, p in enumerate(Ps)]
+    Y = seeded(50, (K * M,), dt)
+    Z, e = run_gpu(fk, ko.KMM, M, Ps, Ps, X, Fs, Y, alpha, beta, opX=ko.OP_T)
+    assert e == 0 and not np.isnan(Z).any()
+    assert fk.last_plan()[-1][2].endswith("_z"), fk.last_plan()
+    x2, z2, y2 = X.reshape(M, K), Z.reshape(K, M), Y.reshape(K, M)
+    picks = _rows(M, 6)
+    want = oracle_answer(ko.KMM, len(picks), Ps, Ps, np.ascontiguousarray(x2[picks]), Fs, np.ascontiguousarray(y2[:, picks]),
+                         alpha, beta, opX=ko.OP_T)
+    err = normwise(np.ascontiguousarray(z2[:, picks]).reshape(-1), np.asarray(want).reshape(-1))
+    assert err <= TOL[dt], f"sampled columns off by {err:.3e}"
+    want = oracle_answer(ko.KMM, 1, Ps, Ps, x2.sum(0, dtype=np.float64), [f.astype(np.float64) for f in Fs],
+                         y2.sum(1, dtype=np.float64), alpha, beta, opX=ko.OP_T)
+    err = normwise(z2.sum(1, dtype=np.float64), np.asarray(want).reshape(-1))
+    assert err <= TOL[dt], f"checksum over all columns off by {err:.3e}"
+
+
 @pytest.mark.parametrize("mm,M,Ps,dt", [
     (ko.MKM, 2064, [16] * 5, np.float32),      # 2.16e9 elements: whole-block kernel on virtual rows + leading launch
     (ko.MKM, 1040, [3] * 13, np.float32),      # 1.66e9 elements through the LDS-fused kernel
