@@ -63,6 +63,14 @@ class FastKron:
     def set_options(self, tune=False, fusion=True):
         self.lib.fastKronSetOptions(self.h, (OPT_USE_FUSION if fusion else OPT_NONE) | (OPT_TUNE if tune else 0))
 
+    def sync_error(self):
+        """Error word of the kernels that synchronise their workgroups (0: no wait ran out); cleared by the call."""
+        w = ctypes.c_uint32(0)
+        e = self.lib.fastKronGetSyncError(self.h, ctypes.byref(w))
+        if e != 0:
+            raise RuntimeError(f"fastKronGetSyncError: {e}")
+        return w.value
+
     def last_plan(self):
         """[(lo, hi, kernel name), ...] of the most recent call, in launch order (include/fastkron_ext.h)."""
         buf = ctypes.create_string_buffer(4096)

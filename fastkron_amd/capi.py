@@ -29,7 +29,7 @@ EXPORTS = [
 ]
 
 EXT_EXPORTS = ["fastKronGetLastPlan", "fastKronSetTunedDB", "fastKronSetPlanOnly", "fastKronGetLastLaunches",
-               "sgemkmStaticScratch"]     # include/fastkron_ext.h
+               "sgemkmStaticScratch", "fastKronGetSyncError", "fastKronSetSyncHelpAfter"]     # include/fastkron_ext.h
 
 _lib = None
 
@@ -92,6 +92,8 @@ def load():
     lib.sgemkmStaticScratch.argtypes = [vp, cint, u32, u32, u32p, u32p, vp, cint, vpp, cint, vp, ctypes.c_float,
                                         ctypes.c_float, vp]
     lib.sgemkmStaticScratch.restype = cint
+    lib.fastKronGetSyncError.argtypes = [vp, u32p]
+    lib.fastKronSetSyncHelpAfter.argtypes = [u32]
     lib.fastKronSetPlanOnly.argtypes = [vp, cint]
     lib.fastKronGetLastLaunches.argtypes = [vp, ctypes.c_char_p, ctypes.c_size_t]
     lib.fastKronGetLastLaunches.restype = ctypes.c_size_t

@@ -6,6 +6,7 @@
 #include "../../include/fastkron.h"
 #include "../../include/fastkron_ext.h"
 #include "handle.h"
+#include "kernels/launch.h"
 
 using namespace fk;
 
@@ -97,6 +98,16 @@ size_t fastKronGetLastLaunches(fastKronHandle handle, char* buf, size_t bufLen) 
     buf[n] = 0;
   }
   return s.size();
+}
+
+fastKronError fastKronGetSyncError(fastKronHandle handle, uint32_t* word) {
+  if (!handle || !word) return fastKronInvalidArgument;
+  return H(handle)->syncError(word);
+}
+
+fastKronError fastKronSetSyncHelpAfter(uint32_t polls) {
+  fk::setKmm4x6TwoPhaseHelpAfter(polls);
+  return fastKronSuccess;
 }
 
 fastKronError fastKronSetTunedDB(fastKronHandle handle, const char* path) {

@@ -83,6 +83,7 @@ static bool tuneChain(Handle& h, const KronProblem& q, const TuneBuffers& B, boo
         a.in = B.in[0]; a.in_batch = (uint64_t)q.M * a.Kin;
         a.out = B.out[0]; a.out_batch = (uint64_t)q.M * a.Kout;
         if (a.y) { a.y = B.out[0]; a.y_batch = (uint64_t)q.M * a.Kout; }
+        a.scratch = B.t1; a.scratch_elems = B.elems; a.sync = h.syncArea();
         const float ms = timeLaunch(k, a, B, h.stream());
         if (verbose) printf("[fastkron] tune %s [%d,%d] %s: %.4f ms\n", q.str().c_str(), lo, hi, k.name.c_str(), ms);
         if (ms < bestT[lo][hi]) { bestT[lo][hi] = ms; bestK[lo][hi] = ki; }
@@ -125,6 +126,7 @@ static bool tuneSingle(Handle& h, const KronProblem& q, const TuneBuffers& B, bo
     a.in = B.in[0]; a.in_batch = (uint64_t)q.M * a.Kin;
     a.out = B.out[0]; a.out_batch = (uint64_t)q.M * a.Kout;
     if (a.y) { a.y = B.out[0]; a.y_batch = (uint64_t)q.M * a.Kout; }
+    a.scratch = B.t2; a.scratch_elems = B.elems; a.sync = h.syncArea();
     const float t = timeLaunch(k, a, B, h.stream());
     if (verbose) printf("[fastkron] tune %s [0,%u] %s: %.4f ms\n", q.str().c_str(), q.N - 1, k.name.c_str(), t);
     if (t < best) { best = t; bestK = ki; }

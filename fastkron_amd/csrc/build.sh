@@ -1,7 +1,8 @@
 #!/bin/bash
 # Builds libFastKron.so (the C-ABI library) for gfx950 with hipcc, in-tree.
-#   fastkron_amd/csrc/build.sh [extra hipcc flags]
+#   fastkron_amd/csrc/build.sh           (takes no arguments: the kernels have no build-time switches)
 set -euo pipefail
+if (( $# )); then echo "build.sh takes no arguments" >&2; exit 2; fi
 HERE="$(cd "$(dirname "${BASH_SOURCE[0]}")" && pwd)"
 OUT="$HERE/../lib"
 OBJ="$HERE/../lib/obj"
@@ -9,7 +10,7 @@ mkdir -p "$OUT" "$OBJ"
 HIPCC="${HIPCC:-/opt/rocm/bin/hipcc}"
 # -packed-fp32-ops is switched off: hipcc must not form v_pk_*_f32 from scalar float code.
 FLAGS=(-O3 -std=c++17 -fPIC --offload-arch=gfx950 -Xclang -target-feature -Xclang -packed-fp32-ops
-       -Wall -Wno-unused-function -Wno-unused-value -Wno-unused-result -Wno-unused-command-line-argument -I"$HERE/../../include" "$@")
+       -Wall -Wno-unused-function -Wno-unused-value -Wno-unused-result -Wno-unused-command-line-argument -I"$HERE/../../include")
 SRCS=("$HERE"/api.cpp "$HERE"/handle.cpp "$HERE"/kernel_db.cpp "$HERE"/autotuner.cpp "$HERE"/static_scratch.hip "$HERE"/kernels/*.hip)
 pids=()
 objs=()

@@ -22,7 +22,7 @@ static int logLevel() {
 Handle::Handle(uint32_t backends) : backends_(backends) {
   // the plans that ship with the library first, then the user's own file on top of them
   const std::string shipped = KernelDB::shippedPath();
-  if (!shipped.empty()) db_.loadFile(shipped);
+  if (!shipped.empty()) db_.loadFile(shipped, true);
   dbPath_ = KernelDB::defaultPath();
   if (!dbPath_.empty()) db_.loadFile(dbPath_);
 }
@@ -34,9 +34,13 @@ Handle::~Handle() {
 
 void Handle::setPlanOnly(bool on) {
   planOnly_ = on;
+  if (!on && mergeWs_ && !mergeWsOwned_) {
+    // the stand-in address of plan-only mode must never reach a launch: without it initHIP allocates the real one
+    mergeWs_ = nullptr; mergeWsBytes_ = 0;
+  }
   if (on && !dev_.valid) {
     // the device the library is written for: 256 compute units, 160 KB of LDS per workgroup
-    dev_.cus = 256; dev_.ldsPerBlock = 160 * 1024; dev_.waveSize = 64;
+    dev_.cus = 256; dev_.ldsPerBlock = 160 * 1024; dev_.waveSize = 64; dev_.xcdRoundRobin = true;
   }
   if (on && !mergeWs_) {
     // never dereferenced: in this mode no launch is made
@@ -80,12 +84,37 @@ fastKronError Handle::initHIP(void* ptrToStream) {
   { void* p = nullptr; (void)staticScratchForCurrentDevice(&p); }
   // workspace for merged factors (kMaxMergeGroups products of at most 64x64 doubles); allocated here so that
   // the gemkm / gekmm calls themselves never allocate
+  if (mergeWs_ && !mergeWsOwned_) { mergeWs_ = nullptr; mergeWsBytes_ = 0; }       // plan-only stand-in
   if (!mergeWs_) {
     mergeWsBytes_ = (size_t)kMaxMergeGroups * 64 * 64 * sizeof(double);
-    if (hipMalloc(&mergeWs_, mergeWsBytes_) != hipSuccess) { mergeWs_ = nullptr; mergeWsBytes_ = 0; }
+    // (behind the merged factors: the counter area of the kernels that synchronise their workgroups, zero once and
+    // left zero by every launch that uses it)
+    if (hipMalloc(&mergeWs_, mergeWsBytes_ + kSyncAreaBytes) != hipSuccess ||
+        hipMemset((char*)mergeWs_ + mergeWsBytes_, 0, kSyncAreaBytes) != hipSuccess) {
+      if (mergeWs_) (void)hipFree(mergeWs_);
+      mergeWs_ = nullptr; mergeWsBytes_ = 0;
+    }
     mergeWsOwned_ = mergeWs_ != nullptr;
+    // how the device places workgroups on its XCDs, recorded once (the counter area serves as the 1 KB this needs
+    // and is zeroed again afterwards)
+    if (mergeWs_) {
+      uint32_t* area = (uint32_t*)((char*)mergeWs_ + mergeWsBytes_);
+      dev_.xcdRoundRobin = kmm4x6TwoPhasePlacementHolds(area, stream_);
+      if (hipMemsetAsync(area, 0, kSyncAreaBytes, stream_) != hipSuccess || hipStreamSynchronize(stream_) != hipSuccess)
+        dev_.xcdRoundRobin = false;
+    }
     if (mergeWs_ && hipEventCreateWithFlags(&mergeWsEvent_, hipEventDisableTiming) != hipSuccess) mergeWsEvent_ = nullptr;
   }
+  return fastKronSuccess;
+}
+
+fastKronError Handle::syncError(uint32_t* word) {
+  *word = 0;
+  if (planOnly_ || !mergeWs_ || !mergeWsOwned_) return fastKronSuccess;
+  uint32_t* dev = (uint32_t*)syncArea() + 1;
+  if (hipMemcpyAsync(word, dev, sizeof(uint32_t), hipMemcpyDeviceToHost, stream_) != hipSuccess ||
+      hipMemsetAsync(dev, 0, sizeof(uint32_t), stream_) != hipSuccess || hipStreamSynchronize(stream_) != hipSuccess)
+    return fastKronOtherError;
   return fastKronSuccess;
 }
 
@@ -150,6 +179,7 @@ fastKronError Handle::sizesForward(uint32_t M, uint32_t N, const uint32_t* Ps, c
 }
 
 fastKronError Handle::xgemm(KronProblem p, fastKronBackend backend, void* temp1, void* temp2, const CallWorkspace* ws) {
+  callWs_ = ws != nullptr;
   // argument checks in the order of reference src/handle/handle.cpp:116-122
   if (!p.forward) {
     if (p.Z == nullptr || temp1 == nullptr || !hasBackend(backend)) return fastKronInvalidArgument;
@@ -187,9 +217,9 @@ fastKronError Handle::xgemm(KronProblem p, fastKronBackend backend, void* temp1,
     // (a GeKMM that runs as a GeMKM is tuned as that GeMKM, below)
     const bool asMKM = p.mm == MMType::KMM && useFusion() && temp2 && viaMKMOnline(p);
     if (!have && canTune() && !planOnly_ && !ws && !asMKM) {
-      e = tune(p, temp2 != nullptr, &c);
-      if (e != fastKronSuccess && e != fastKronKernelNotFound) return e;
-      have = (e == fastKronSuccess);
+      // a tuner that cannot run (no memory for its operand sets, no events) leaves the problem without a record:
+      // the call then runs on the online selection, as it would untuned
+      have = tune(p, temp2 != nullptr, &c) == fastKronSuccess;
     }
     if (have) {
       e = runChoice(p, c, temp1, temp2, ws);
@@ -359,39 +389,54 @@ void Handle::noteTranspose(const KronProblem& p) {
 // plan-only mode on the call's own buffers; the answer is kept per problem.
 bool Handle::transposeFirstOnline(const KronProblem& p, const KronProblem& pn, void* temp1, void* temp2,
                                   const CallWorkspace* ws) {
+  // Lays a problem out in plan-only mode on the call's own buffers and counts its launches.
+  auto plannedLaunches = [&](const KronProblem& q, bool* ok) {
+    const bool wasPlanOnly = planOnly_;
+    const std::string savedPlan = lastPlan_, savedLog = launchLog_;
+    planOnly_ = true;
+    *ok = runOnline(q, temp1, temp2, ws) == fastKronSuccess;
+    const size_t n = countLaunches(lastPlan_);
+    const std::string plan = lastPlan_;
+    planOnly_ = wasPlanOnly;
+    lastPlan_ = savedPlan; launchLog_ = savedLog;
+    return std::make_pair(n, plan);
+  };
   const std::string ck = p.str() + (temp2 ? "_t2" : "_t1");
   auto it = transposeCache_.find(ck);
-  if (it != transposeCache_.end()) return it->second;
-  const bool wasPlanOnly = planOnly_;
-  const std::string savedPlan = lastPlan_, savedLog = launchLog_;
-  planOnly_ = true;
-  size_t nT = 0, nN = 0;
-  const bool okT = runOnline(p, temp1, temp2, ws) == fastKronSuccess;
-  nT = countLaunches(lastPlan_);
-  // a first launch that reads a transposed X through the padded step with a large factor counts twice: in the MKM layout
-  // always (tuned plans: 128x128 chains run 1.3 to 3.3 times faster behind a transposed copy, pairs of single 64x64
-  // steps 1.3 to 1.4 times); in the KMM layout, where that step reads the transposed X along its rows, only while X
-  // stays in the caches (up to 64 MB the copy is ahead by 8 to 14 %, beyond that behind by 5 to 30 %)
-  const uint64_t xBytes = p.M * p.K() * (p.dt == DType::F32 ? 4 : 8) * (uint64_t)(p.batch ? p.batch : 1);
-  if (okT && p.P[p.N - 1] >= 64 && (p.mm == MMType::MKM || xBytes <= (64ull << 20))) {
-    const size_t s0 = lastPlan_.find(':');
-    if (s0 != std::string::npos && lastPlan_.compare(s0 + 1, 6, "gekmm_") == 0 &&
-        lastPlan_.find("anyxany", s0) < lastPlan_.find(';', s0)) nT++;
+  bool yes;
+  if (it != transposeCache_.end()) yes = it->second;
+  else {
+    bool okT = false, okN = false;
+    auto planT = plannedLaunches(p, &okT);
+    size_t nT = planT.first;
+    // a first launch that reads a transposed X through the padded step with a large factor counts twice: in the MKM layout
+    // always (tuned plans: 128x128 chains run 1.3 to 3.3 times faster behind a transposed copy, pairs of single 64x64
+    // steps 1.3 to 1.4 times); in the KMM layout, where that step reads the transposed X along its rows, only while X
+    // stays in the caches (up to 64 MB the copy is ahead by 8 to 14 %, beyond that behind by 5 to 30 %)
+    const uint64_t xBytes = p.M * p.K() * (p.dt == DType::F32 ? 4 : 8) * (uint64_t)(p.batch ? p.batch : 1);
+    if (okT && p.P[p.N - 1] >= 64 && (p.mm == MMType::MKM || xBytes <= (64ull << 20))) {
+      const std::string& pl = planT.second;
+      const size_t s0 = pl.find(':');
+      if (s0 != std::string::npos && pl.compare(s0 + 1, 6, "gekmm_") == 0 && pl.find("anyxany", s0) < pl.find(';', s0)) nT++;
+    }
+    const size_t nN = plannedLaunches(pn, &okN).first;
+    // with equal counts the copy goes first, except in the KMM layout with fewer than 64 columns, where the copy cannot
+    // run on whole 64-wide tiles with 16-byte accesses (sgekmm 16x16^4 with 256 and 1024 columns: 1.26 times faster
+    // behind the copy; 16 columns, 16x16^6: 1.16 times slower; factors below 16x16 read a transposed X too slowly in any
+    // case)
+    const bool copyOnTie = p.mm == MMType::MKM || p.M >= 64 || p.P[p.N - 1] < 16;
+    yes = okN && (!okT || (copyOnTie ? 1 + nN <= nT : 1 + nN < nT));
+    transposeCache_[ck] = yes;           // the preference of the shape; the buffers of each call are checked below
   }
-  const bool okN = runOnline(pn, temp1, temp2, ws) == fastKronSuccess;
-  nN = countLaunches(lastPlan_);
-  planOnly_ = wasPlanOnly;
-  lastPlan_ = savedPlan; launchLog_ = savedLog;
-  // without a second temporary the transposed copy sits in temp1, which a plan of several launches writes
-  // with equal counts the copy goes first, except in the KMM layout with fewer than 64 columns, where the copy cannot
-  // run on whole 64-wide tiles with 16-byte accesses (sgekmm 16x16^4 with 256 and 1024 columns: 1.26 times faster
-  // behind the copy; 16 columns, 16x16^6: 1.16 times slower; factors below 16x16 read a transposed X too slowly in any
-  // case)
-  const bool copyOnTie = p.mm == MMType::MKM || p.M >= 64 || p.P[p.N - 1] < 16;
-  bool yes = okN && (!okT || (copyOnTie ? 1 + nN <= nT : 1 + nN < nT));
-  if (yes && !temp2 && nN != 1) yes = false;
-  transposeCache_[ck] = yes;
-  return yes;
+  if (!yes) return false;
+  // Without a second temporary the transposed copy sits in temp1, which a plan of several launches writes while its
+  // first launch still reads the copy.  How many launches the untransposed problem takes depends on the call's own
+  // buffers (a misaligned operand moves it off the whole-row kernels), so this is asked on every call.
+  if (!temp2) {
+    bool okN = false;
+    if (plannedLaunches(pn, &okN).first != 1 || !okN) return false;
+  }
+  return true;
 }
 
 fastKronError Handle::runOnline(KronProblem p, void* temp1, void* temp2, const CallWorkspace* ws) {
@@ -745,6 +790,12 @@ fastKronError Handle::execute(const KronProblem& p, const Plan& plan, void* temp
     if (n == 2) { tmps[1] = nullptr; zIsTmp[1] = false; }     // a 2-launch plan never touches the second one
   }
 
+  // capacity of a temporary by the API's contract: the widest step output of every batch entry
+  uint64_t tempElems = 0;
+  if (!p.forward) {
+    size_t ye = 0, te = 0;
+    if (sizes(p.M, p.N, p.P, p.Q, &ye, &te) == fastKronSuccess) tempElems = (uint64_t)te * p.batch;
+  }
   const void* in = p.X;
   uint64_t inBatch = p.strideX;
   for (size_t l = 0; l < n; l++) {
@@ -783,6 +834,17 @@ fastKronError Handle::execute(const KronProblem& p, const Plan& plan, void* temp
       a.stream_in = inFromCaller ? (moved >= kStreamFrom && inBytes >= kStreamFrom / 2) : inBytes > kBeyondCache;
       a.stream_out = outToCaller ? moved >= kStreamFrom : outBytes > kBeyondCache;
     }
+    {
+      // A temporary that this launch neither reads nor writes, for kernels that keep an intermediate of their own:
+      // the first launch reads X and the last writes Z, so one of the two temporaries is idle then.
+      void* idle = nullptr;
+      if (!p.forward && (first || last)) {
+        for (void* t : {temp1, temp2})
+          if (t && t != a.in && t != a.out && t != (const void*)p.Z && t != p.X && t != p.Y && !idle) idle = t;
+      }
+      a.scratch = idle; a.scratch_elems = idle ? tempElems : 0;
+      a.sync = callWs_ ? nullptr : syncArea();
+    }
     if (logLevel() >= 2)
       printf("[fastkron]   launch %zu: factors [%u,%u] Kin=%llu Kout=%llu kernel %s\n", l, s.lo, s.hi,
              (unsigned long long)a.Kin, (unsigned long long)a.Kout, k.name.c_str());
@@ -815,6 +877,12 @@ fastKronError Handle::execute(const KronProblem& p, const Plan& plan, void* temp
           launchLog_ += "\n";
         }
         continue;
+      }
+      if (k.usesSync) {
+        // the counter area is one more piece of device state of the handle: a later call on another stream is
+        // ordered behind this launch (orderWorkspaceBehind)
+        if (mergeWsUsed_ && mergeWsStream_ != stream_) orderWorkspaceBehind(stream_);
+        mergeWsStream_ = stream_; mergeWsUsed_ = true;
       }
       hipError_t he = k.launch(k, c, stream_);
       if (he != hipSuccess) {

@@ -92,6 +92,10 @@ class Handle {
   KernelDB& db() { return db_; }
   const DeviceInfo& device() const { return dev_; }
   hipStream_t stream() const { return stream_; }
+  // the zero-initialised counter area behind the merged-factor workspace (null before fastKronInitHIP)
+  // Reads and clears the error word of the counter area (synchronises the stream).
+  fastKronError syncError(uint32_t* word);
+  void* syncArea() const { return mergeWs_ ? (char*)mergeWs_ + mergeWsBytes_ : nullptr; }
 
  private:
   fastKronError ensureDevice();
@@ -114,6 +118,7 @@ class Handle {
   bool mergeWsUsed_ = false;
   hipEvent_t mergeWsEvent_ = nullptr;                 // orders a new stream behind the last user of the workspace
   bool planOnly_ = false;
+  bool callWs_ = false;                               // the running call brought its own workspace (touches none of the handle's)
   std::string launchLog_;
 };
 

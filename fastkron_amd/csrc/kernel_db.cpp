@@ -21,7 +21,17 @@ std::string KronProblem::str() const {
   if (mm == MMType::MKM) { o << M << "x" << K() << "*("; facs(); o << ")"; }
   else                   { o << "("; facs(); o << ")*" << K() << "x" << M; }
   o << "_" << (opX == 2 ? "T" : "N") << (opF == 2 ? "T" : "N") << "_" << (dt == DType::F32 ? "f" : "d");
-  if (strided) o << "_stridedBatched_" << batch;
+  if (strided) {
+    o << "_stridedBatched_" << batch;
+    // the stride class: a shared X and shared factors change which kernels and rewritings apply (merging, the
+    // two-part plan), so plans of one class are not looked up for another.  Per-batch operands carry no suffix.
+    if (batch > 1) {
+      if (strideX == 0) o << "_Xs";
+      uint64_t shared = 0;
+      for (uint32_t i = 0; i < N; i++) if (strideF[i] == 0) shared |= 1ull << i;
+      if (shared) o << "_Fs" << std::hex << shared << std::dec;
+    }
+  }
   return o.str();
 }
 
@@ -285,6 +295,22 @@ static bool kmm4x6CanRun(const KernelInfo&, const KronProblem& p, uint32_t lo, u
   if (dev.rulesOfThumb && (uint64_t)(p.M / 8) * p.batch > (uint64_t)dev.cus) return false;
   return dev.ldsPerBlock >= (8 * 64 * 65 + 32) * 4;
 }
+// The two-phase form: M a multiple of 256.  By rule only from 2048 columns on (one column block per XCD), where it
+// is 1.4 times faster than the whole-column kernel; with fewer columns part of the XCDs would work on blocks whose
+// intermediate lives in another XCD's L2.
+static bool kmm4x6TwoPhaseCanRun(const KernelInfo&, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
+                                 const DeviceInfo& dev) {
+  if (p.dt != DType::F32 || p.mm != MMType::KMM || hi - lo + 1 != 6 || p.forward) return false;
+  for (uint32_t i = lo; i <= hi; i++) if (p.P[i] != 4 || p.Q[i] != 4) return false;
+  if (p.colsBefore(hi) != 4096 || p.M % 256) return false;
+  if (first && p.opX == 2) return false;
+  if ((uint64_t)(p.M / 256) * p.batch > 248) return false;          // counters per column block in a 4 KB area
+  if (!dev.xcdRoundRobin) return false;                              // its blocks synchronise through one XCD's L2
+  if (dev.rulesOfThumb && (p.M % 2048 || dev.cus < 256)) return false;
+  return true;
+}
+static hipError_t kmm4x6TwoPhaseLaunch(const KernelInfo&, const StepArgs& a, hipStream_t s) { return launchKmm4x6TwoPhase(a, s); }
+static bool kmm4x6TwoPhaseCheck(const KernelInfo&, const StepArgs& a) { return kmm4x6TwoPhaseSupported(a); }
 static hipError_t kmm4x6Launch(const KernelInfo&, const StepArgs& a, hipStream_t s) { return launchKmm4x6(a, s); }
 static bool kmm4x6Check(const KernelInfo&, const StepArgs& a) { return kmm4x6Supported(a); }
 
@@ -363,6 +389,15 @@ void registerRowKernels(std::vector<KernelInfo>& out) {
     out.push_back(k2);
   }
 
+  {
+    // ahead of the whole-column kernel: chosen first where both apply
+    KernelInfo k6{};
+    k6.name = "kmm_hip_gfx950_256_f_4x4_4x4_6_256x4096_mfma4x4x1_NN_strided_0_3";
+    k6.dt = DType::F32; k6.P = 4; k6.Q = 4; k6.fused = 6; k6.tileM = 256; k6.tileK = 4096; k6.threads = 256; k6.variant = 0;
+    k6.canRun = kmm4x6TwoPhaseCanRun; k6.launch = kmm4x6TwoPhaseLaunch; k6.check = kmm4x6TwoPhaseCheck;
+    k6.usesSync = true;
+    out.push_back(k6);
+  }
   {
     KernelInfo k6{};
     k6.name = "kmm_hip_gfx950_512_f_4x4_4x4_6_8x4096_mfma4x4x1_NN_strided_0_3";
@@ -560,7 +595,7 @@ void KernelDB::storeTuned(const std::string& key, const Plan& plan, float ms, in
 // File format, one problem per line:
 //   <problem string> <ms> [M<merge> S<split> [X<transposeX>]] <nsteps> {<lo> <hi> <kernel name>}...
 // (lines without the M / S fields leave both to the online selection)
-bool KernelDB::loadFile(const std::string& path) {
+bool KernelDB::loadFile(const std::string& path, bool shipped) {
   std::ifstream f(path);
   if (!f) return false;
   std::string line;
@@ -569,7 +604,7 @@ bool KernelDB::loadFile(const std::string& path) {
     std::istringstream is(line);
     std::string key, tok; float ms; size_t n = 0;
     if (!(is >> key >> ms >> tok)) continue;
-    Tuned t; t.ms = ms;
+    Tuned t; t.ms = ms; t.shipped = shipped;
     if (!tok.empty() && tok[0] == 'M') {
       std::string stok, ntok;
       if (!(is >> stok >> ntok) || stok.empty() || stok[0] != 'S') continue;
@@ -604,6 +639,7 @@ bool KernelDB::saveFile(const std::string& path) const {
   if (!f) return false;
   f << "# fastkron gfx950 tuned launch plans: problem ms nsteps {lo hi kernel}\n";
   for (auto& kv : tuned_) {
+    if (kv.second.shipped) continue;       // the library's own records stay in its own file
     f << kv.first << " " << kv.second.ms;
     if (kv.second.merge >= 0) {
       f << " M" << kv.second.merge << " S" << kv.second.split;

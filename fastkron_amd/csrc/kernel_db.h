@@ -25,6 +25,8 @@ struct DeviceInfo {
   // is faster (few rows, small factors ...).  The tuner and the check of a tuned plan switch this off and ask only
   // what a kernel is able to run.
   bool rulesOfThumb = true;
+  // Workgroups i and i + 8 k of a launch run on one XCD and share its L2 (checked once by fastKronInitHIP).
+  bool xcdRoundRobin = false;
 };
 
 struct KernelInfo;
@@ -45,6 +47,7 @@ struct KernelInfo {
   uint32_t threads;
   uint32_t variant;       // kernel-family specific
   bool     tunerOnly;     // a candidate for the tuner, never chosen by the online selection
+  bool     usesSync;      // synchronises its workgroups through the handle's counter area (StepArgs::sync)
   CanRunFn canRun;
   LaunchFn launch;
   CheckFn  check;
@@ -81,7 +84,9 @@ class KernelDB {
                    int* transposeX = nullptr) const;
   void storeTuned(const std::string& key, const Plan& plan, float ms, int merge = -1, uint32_t split = 0,
                   int transposeX = 0);
-  bool loadFile(const std::string& path);
+  // `shipped`: the records come from the file that ships with the library; saveFile leaves those out, so that a
+  // user's file never holds stale copies that would override later versions of them
+  bool loadFile(const std::string& path, bool shipped = false);
   bool saveFile(const std::string& path) const;
   static std::string defaultPath();
   static std::string shippedPath();
@@ -94,6 +99,7 @@ class KernelDB {
     int merge = -1;
     uint32_t split = 0;
     int transposeX = 0;
+    bool shipped = false;
   };
   std::map<std::string, Tuned> tuned_;
 };

@@ -129,6 +129,16 @@ hipError_t launchKmm64F64(const StepArgs& a, hipStream_t stream);
 bool kmm4x6Supported(const StepArgs& a);
 hipError_t launchKmm4x6(const StepArgs& a, hipStream_t stream);
 
+// The same problem in two phases with an intermediate in a temporary of the call: every access a full 256-byte piece.
+bool kmm4x6TwoPhaseSupported(const StepArgs& a);
+hipError_t launchKmm4x6TwoPhase(const StepArgs& a, hipStream_t stream);
+constexpr size_t kSyncAreaBytes = 4096;     // zero-initialised counter area such kernels need (StepArgs::sync)
+// Whether workgroups i and i + 8 k of a launch share an XCD on this device (checked with a small launch and a
+// synchronisation, at set-up); the kernel above is only offered where that holds.
+bool kmm4x6TwoPhasePlacementHolds(uint32_t* scratchWords, hipStream_t stream);
+// Polls after which a waiting workgroup of that kernel runs missing jobs itself (tests set 0).
+void setKmm4x6TwoPhaseHelpAfter(uint32_t polls);
+
 // KMM layout, fp32: three fused 4x4 or two fused 8x8 factors held in registers, lanes along M.
 bool kmmRegSupported(const StepArgs& a);
 hipError_t launchKmmReg(const StepArgs& a, hipStream_t stream);

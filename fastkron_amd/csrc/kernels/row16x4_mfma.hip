@@ -49,14 +49,8 @@ typedef float f4 __attribute__((ext_vector_type(4)));
 #define MFMA4(a, b, c) __builtin_amdgcn_mfma_f32_4x4x1f32((a), (b), (c), 0, 0, 0)
 
 constexpr int kRowLen = 65536;
-#ifndef ROW16_WIN
-#define ROW16_WIN 6
-#endif
-#ifndef ROW16_CARRY
-#define ROW16_CARRY 2
-#endif
-constexpr int kWin = ROW16_WIN;            // slices in flight per wave while it works on slices (registers: 64 accumulators + 4*kWin + operands)
-constexpr int kCarry = ROW16_CARRY;        // slices of the next row in flight during the exchange (<= kWin)
+constexpr int kWin = 6;            // slices in flight per wave while it works on slices (registers: 64 accumulators + 4*kWin + operands)
+constexpr int kCarry = 2;        // slices of the next row in flight during the exchange (<= kWin)
 constexpr uint32_t kStaggerGroups = 5;     // measured: 5 groups 2.5 us apart or 3 groups 4 us apart; 2 or 4 groups lose to no stagger
 constexpr uint32_t kStaggerTicks = 250;    // of the 100 MHz wall clock
 constexpr int kQuarterWords = 16384;       // 64 KB: 16 rows k1 of 1024 columns (four values of q2)

@@ -108,16 +108,6 @@ __global__ __launch_bounds__(256, 2) void kron_step_mfma_kernel(const StepArgs a
     const uint32_t m = t / tilesPerRow;
     const uint64_t s0 = (uint64_t)(t % tilesPerRow) * 16;
     const uint64_t s = (s0 + lo < S) ? s0 + lo : s0;
-#ifdef STEP_HACK_COALESCED      // timing experiment only: the lanes of an instruction read consecutive 16 bytes (results are wrong)
-    const T* xq = inB + (size_t)m * a.in_ldm + s0 * P + l * VE;
-#pragma unroll
-    for (int c = 0; c < PC; c += VE) {
-      const VT v = *(const VT*)(xq + (c / VE) * 64 * VE);
-#pragma unroll
-      for (int e = 0; e < VE; e++) x[c + e] = v[e];
-    }
-    return;
-#endif
     const T* xp = inB + (size_t)m * a.in_ldm + s * P + PC * hi;
 #pragma unroll
     for (int c = 0; c < PC; c += VE) {
@@ -187,11 +177,7 @@ __global__ __launch_bounds__(256, 2) void kron_step_mfma_kernel(const StepArgs a
           const uint64_t col = (uint64_t)(q0 + 16 * ib + M16::row(r, hi)) * qStride;
           T v = acc[ib][r] * scale;
           if (HAS_Y) v += beta * yv[ib][r];
-  #ifdef STEP_HACK_STORE          // timing experiment only: every store instruction writes 256 contiguous bytes (results are wrong)
-        outB[(size_t)(t / tilesPerRow) * a.out_ldm + ((size_t)(t % tilesPerRow) * QS + qpart) * (16 * NB * 16) + (ib * 4 + r) * 64 + l] = v;
-#else
-        out[col] = v;
-#endif
+          out[col] = v;
         }
     };
     if (waveId >= totalTiles) return;

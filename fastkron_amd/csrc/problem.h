@@ -80,6 +80,12 @@ struct StepArgs {
   // a launch of this call / the output is large and no launch of this call reads it back (or it is larger than
   // the memory-side cache anyway).  Such data gains nothing from being kept in the caches.
   uint32_t stream_in, stream_out;
+  // A temporary of the call that this launch neither reads nor writes (null when there is none), for kernels that
+  // pass an intermediate through memory inside one launch, and a small zero-initialised counter area of the handle
+  // (null for calls that must not touch the handle's device memory).
+  void*    scratch;
+  uint64_t scratch_elems;
+  void*    sync;
 };
 
 // Merging of adjacent small factors into their Kronecker product (kernels/merge_factors.hip).

@@ -56,6 +56,18 @@ fastKronError sgemkmStaticScratch(fastKronHandle handle, fastKronBackend backend
                                   const float* const Fs[], fastKronOp opFs, float* Z, float alpha, float beta,
                                   const float* Y);
 
+/*
+ * Kernels whose workgroups wait for each other inside one launch (the two-phase 4x4^6 GeKMM kernel) keep their counters
+ * in device memory of the handle and bound every wait; a wait that runs out sets an error word there and the results
+ * of that launch are not valid.  fastKronGetSyncError synchronises the handle's stream, copies the word to *word
+ * (0: no wait ever ran out) and clears it.  fastKronSetSyncHelpAfter sets, for every handle of the process, after how
+ * many polls a waiting workgroup runs the missing work of others itself (default 100000, far beyond what a launch
+ * needs when all its workgroups run; 0 makes every workgroup do so at once, which tests use to cover that path).
+ * Neither has a counterpart in the reference, whose kernels never synchronise across workgroups.
+ */
+fastKronError fastKronGetSyncError(fastKronHandle handle, uint32_t* word);
+fastKronError fastKronSetSyncHelpAfter(uint32_t polls);
+
 #ifdef __cplusplus
 }
 #endif

@@ -625,6 +625,70 @@ def test_kmm_six_4x4_factors_in_one_launch(fk, M):
     assert len(fk.last_plan()) == (1 if M * 40 // 8 <= 256 else 2), fk.last_plan()
 
 
+TWO_PHASE_4X6 = "kmm_hip_gfx950_256_f_4x4_4x4_6_256x4096_mfma4x4x1_NN_strided_0_3"
+
+
+def test_kmm_six_4x4_factors_in_two_phases_of_one_launch(fk):
+    """sgekmm with 4x4^6 from 2048 columns on: one launch whose workgroups pass an intermediate through a temporary of
+    the call and wait for each other per block of 256 columns.  With and without Y, transposed factors, one temporary
+    only, a batch (16 column blocks: more workgroups than are resident at once)."""
+    Ps = [4] * 6
+    check(fk, ko.KMM, 2048, Ps, Ps, np.float32, alpha=1.5, beta=0.5, seed=291)
+    assert [k for _, _, k in fk.last_plan()] == [TWO_PHASE_4X6], fk.last_plan()
+    check(fk, ko.KMM, 2048, Ps, Ps, np.float32, alpha=1.0, beta=0.0, seed=292, opFs=ko.OP_T)
+    check(fk, ko.KMM, 2048, Ps, Ps, np.float32, alpha=2.0, beta=0.0, seed=293, integer=True, use_temp2=False)
+    assert [k for _, _, k in fk.last_plan()] == [TWO_PHASE_4X6], fk.last_plan()
+    check(fk, ko.KMM, 2048, Ps, Ps, np.float32, alpha=1.0, beta=1.0, seed=294, batch=2)
+    assert [k for _, _, k in fk.last_plan()] == [TWO_PHASE_4X6], fk.last_plan()
+    check(fk, ko.KMM, 4096, Ps, Ps, np.float32, alpha=-1.0, beta=0.25, seed=295)
+    assert [k for _, _, k in fk.last_plan()] == [TWO_PHASE_4X6], fk.last_plan()
+    # the same call again and again: every launch leaves the counters as it found them
+    for i in range(5):
+        check(fk, ko.KMM, 2048, Ps, Ps, np.float32, alpha=1.5, beta=0.5, seed=296 + i)
+    assert fk.sync_error() == 0
+
+
+def test_two_phase_4x4_kernel_when_workgroups_run_the_jobs_of_others(fk):
+    """A workgroup of the two-phase kernel that waits too long for the others runs their missing jobs itself (what keeps
+    the launch from deadlocking when not all workgroups are resident).  With the threshold at 0 every workgroup does so
+    at once: jobs then run twice, with the same values, and the result must not change."""
+    from fastkron_amd import capi
+    Ps = [4] * 6
+    lib = capi.load()
+    try:
+        assert lib.fastKronSetSyncHelpAfter(0) == 0
+        check(fk, ko.KMM, 2048, Ps, Ps, np.float32, alpha=1.5, beta=0.5, seed=391)
+        assert [k for _, _, k in fk.last_plan()] == [TWO_PHASE_4X6], fk.last_plan()
+        check(fk, ko.KMM, 2048, Ps, Ps, np.float32, alpha=1.0, beta=0.0, seed=392, batch=2)
+        check(fk, ko.KMM, 2048, Ps, Ps, np.float32, alpha=1.0, beta=1.0, seed=393)
+    finally:
+        lib.fastKronSetSyncHelpAfter(100000)
+    check(fk, ko.KMM, 2048, Ps, Ps, np.float32, alpha=1.5, beta=0.5, seed=394)
+    assert fk.sync_error() == 0
+
+
+def test_two_phase_4x4_kernel_on_column_counts_it_is_not_chosen_for(tmp_path):
+    """Any multiple of 256 columns runs on the two-phase kernel when a tuned plan names it: fewer column blocks than
+    XCDs (workgroups without a block leave at once), blocks of different batch entries, shared factors."""
+    import fastkron_amd
+    db = tmp_path / "plans.txt"
+    db.write_text("".join(f"{prob} 0.1 M0 S0 1 0 5 {TWO_PHASE_4X6}\n" for prob in
+                          ["(4x4^6)*4096x256_NN_f", "(4x4^6)*4096x768_NN_f", "(4x4^6)*4096x512_NN_f_stridedBatched_3",
+                           "(4x4^6)*4096x256_NN_f_stridedBatched_5_Fs3f", "(4x4^6)*4096x1280_NT_f"]))
+    h = fastkron_amd.FastKron()
+    h.set_tuned_db(str(db))
+    try:
+        Ps = [4] * 6
+        for M, kw in [(256, dict(alpha=1.5, beta=0.5)), (768, dict(alpha=1.0, beta=0.0)),
+                      (512, dict(alpha=1.0, beta=1.0, batch=3)), (256, dict(alpha=2.0, beta=0.5, batch=5, share_f=True)),
+                      (1280, dict(alpha=1.0, beta=-1.0, opFs=ko.OP_T))]:
+            check(h, ko.KMM, M, Ps, Ps, np.float32, seed=301 + M, **kw)
+            assert [k for _, _, k in h.last_plan()] == [TWO_PHASE_4X6], h.last_plan()
+        assert h.sync_error() == 0
+    finally:
+        h.close()
+
+
 @pytest.mark.parametrize("mm,M,Ps,dt,launches", [
     (ko.MKM, 96, [4] * 8, np.float32, 1),         # -> 16x16^4: one whole-block launch
     (ko.MKM, 4, [4] * 8, np.float32, 2),          # the same with few rows: three factors per 4096-block + one across
