@@ -20,7 +20,7 @@ def fk():
 
 
 def check(fk, mm, M, Ps, Qs, dt, alpha=1.0, beta=0.0, seed=0, **kw):
-    run_kw = {k: kw.pop(k) for k in ("use_temp2", "strided") if k in kw}
+    run_kw = {k: kw.pop(k) for k in ("use_temp2", "strided", "y_is_z") if k in kw}
     integer = kw.get("integer", False)
     X, Fs, Y = make_case(mm, M, Ps, Qs, dt, seed=seed, with_y=(beta != 0), **kw)
     kw.pop("integer", None)
@@ -951,3 +951,72 @@ def test_kmm_three_fused_8x8_factors(fk, mm, M, Ps, launches):
     check(fk, mm, M, Ps, Ps, np.float32, alpha=1.0, beta=1.0, seed=223, batch=3)
     check(fk, mm, M, Ps, Ps, np.float32, alpha=2.0, beta=0.0, seed=224, batch=2, share_f=True)
     check(fk, mm, M, Ps, Ps, np.float32, alpha=1.0, beta=0.0, seed=225, integer=True, use_temp2=False)
+
+
+# ---- Z == Y: the epilogue reads Y and writes Z through one buffer (allowed with two temporaries, reference
+# include/fastkron.h:274-277, src/handle/handle.cpp:120-122).  Every kernel family that has a Y epilogue: each reads
+# Y and writes Z from registers laid out its own way, and must read an element before it writes it. ----
+IN_PLACE = [
+    # kernel family, mm, M, Ps, Qs, dtype, extra
+    ("whole-column 4x4^6", ko.KMM, 512, [4] * 6, [4] * 6, np.float32, {}),
+    ("4x4x3 register kernel, two launches", ko.KMM, 100, [4] * 6, [4] * 6, np.float32, {}),
+    ("32x16^3 row kernel, batched", ko.MKM, 8, [32] * 3, [16] * 3, np.float32, dict(batch=3)),
+    ("16x16^4 row kernel", ko.MKM, 6, [16] * 4, [16] * 4, np.float32, {}),
+    ("8x8^5 row kernel", ko.MKM, 5, [8] * 5, [8] * 5, np.float32, {}),
+    ("32x32^3 row kernel", ko.MKM, 3, [32] * 3, [32] * 3, np.float32, {}),
+    ("16x16^3 wave-per-block fp64", ko.MKM, 8, [16] * 3, [16] * 3, np.float64, {}),
+    ("16x16^3 wave-per-block fp32", ko.MKM, 8, [16] * 3, [16] * 3, np.float32, {}),
+    ("64x64 pair fp64", ko.MKM, 600, [64] * 2, [64] * 2, np.float64, {}),
+    ("64x64 pair fp32", ko.MKM, 600, [64] * 2, [64] * 2, np.float32, {}),
+    ("32x32 pair fp64", ko.MKM, 40, [32] * 2, [32] * 2, np.float64, {}),
+    ("padded 24x24 pair", ko.MKM, 16, [24] * 2, [24] * 2, np.float32, {}),
+    ("two-part plan fp32", ko.MKM, 4, [16] * 5, [16] * 5, np.float32, {}),
+    ("two-part plan fp64, KMM-layout 64x64 step", ko.MKM, 2, [64] * 3, [64] * 3, np.float64, {}),
+    ("two-part plan 8x8^7", ko.MKM, 2, [8] * 7, [8] * 7, np.float32, {}),
+    ("GeKMM as GeMKM + transposition", ko.KMM, 64, [8] * 5, [8] * 5, np.float32, dict(opX=ko.OP_T)),
+    ("GeKMM as GeMKM + transposition fp64", ko.KMM, 64, [16] * 3, [16] * 3, np.float64, dict(opX=ko.OP_T, opFs=ko.OP_T)),
+    ("transposed copy of X first", ko.MKM, 64, [8] * 5, [8] * 5, np.float32, dict(opX=ko.OP_T)),
+    ("8x8^3 KMM kernel", ko.KMM, 128, [8] * 3, [8] * 3, np.float32, {}),
+    ("16x16^2 KMM kernel", ko.KMM, 96, [16] * 2, [16] * 2, np.float32, {}),
+    ("16x16^2 KMM kernel fp64", ko.KMM, 96, [16] * 2, [16] * 2, np.float64, {}),
+    ("64x64 KMM step fp64", ko.KMM, 128, [64], [64], np.float64, {}),
+    ("wide step 128x128", ko.MKM, 64, [128] * 2, [128] * 2, np.float32, {}),
+    ("wide step KMM 64x64", ko.KMM, 256, [64] * 2, [64] * 2, np.float32, {}),
+    ("streaming step 16x16", ko.MKM, 33, [16], [16], np.float32, {}),
+    ("padded step 31x63", ko.MKM, 16, [31] * 2, [63] * 2, np.float32, {}),
+    ("padded step 50x50 fp64 KMM", ko.KMM, 48, [50] * 2, [50] * 2, np.float64, {}),
+    ("LDS-fused small factors", ko.MKM, 16, [3] * 7, [3] * 7, np.float32, {}),
+    ("LDS-fused small factors KMM", ko.KMM, 64, [5] * 4, [5] * 4, np.float64, {}),
+    ("LDS-fused rectangular", ko.MKM, 16, [2] * 5, [4] * 5, np.float32, {}),
+    ("merged 4x4^8", ko.MKM, 8, [4] * 8, [4] * 8, np.float32, {}),
+    ("generic", ko.MKM, 7, [297], [127], np.float32, {}),
+    ("generic KMM", ko.KMM, 20, [5, 1, 7], [1, 6, 2], np.float64, {}),
+]
+
+
+@pytest.mark.parametrize("family,mm,M,Ps,Qs,dt,extra", IN_PLACE, ids=[c[0] for c in IN_PLACE])
+def test_z_is_y(fk, family, mm, M, Ps, Qs, dt, extra):
+    check(fk, mm, M, Ps, Qs, dt, alpha=1.5, beta=0.5, seed=501, y_is_z=True, **extra)
+    check(fk, mm, M, Ps, Qs, dt, alpha=-1.0, beta=2.0, seed=502, y_is_z=True, integer=True, **extra)
+
+
+def test_z_is_y_needs_the_second_temporary(fk):
+    """reference src/handle/handle.cpp:120-122"""
+    import torch
+    Ps = [8] * 3
+    X = torch.zeros(4 * 512, device="cuda:0")
+    Fs = [torch.zeros(64, device="cuda:0") for _ in Ps]
+    Z = torch.zeros(4 * 512, device="cuda:0")
+    t1 = torch.zeros(4 * 512, device="cuda:0")
+    assert fk.xgemkm(4, Ps, Ps, X, Fs, Z, 1.0, 1.0, Z, t1, None) == 4
+
+
+def test_z_is_y_at_full_size_on_the_two_phase_4x4_kernel(fk):
+    from tests.gpu_util import sampled_check
+    err_rows, err_sum = sampled_check(fk, ko.KMM, 2048, [4] * 6, [4] * 6, np.float32, alpha=1.5, beta=0.5, y_is_z=True)
+    assert [k for _, _, k in fk.last_plan()] == [TWO_PHASE_4X6], fk.last_plan()
+    assert err_rows <= 1e-5 and err_sum <= 1e-5, (err_rows, err_sum)
+    err_rows, err_sum = sampled_check(fk, ko.MKM, 1024, [16] * 4, [16] * 4, np.float32, alpha=2.0, beta=-0.5, y_is_z=True)
+    assert err_rows <= 1e-5 and err_sum <= 1e-5, (err_rows, err_sum)
+    err_rows, err_sum = sampled_check(fk, ko.MKM, 256, [64] * 3, [64] * 3, np.float64, alpha=1.0, beta=1.0, y_is_z=True)
+    assert err_rows <= 1e-12 and err_sum <= 1e-12, (err_rows, err_sum)

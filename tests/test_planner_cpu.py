@@ -292,6 +292,45 @@ def test_transposed_x_is_read_in_place_when_a_copy_does_not_pay_or_does_not_fit(
     assert int(launches[0]["in"], 16) == BASE + 3 * GAP
 
 
+def test_copy_into_the_only_temporary_is_decided_on_every_calls_own_buffers(online_planner):
+    """Without a second temporary the transposed copy of X sits in temp1, so the launches behind it must be one launch.
+    How many they are depends on the buffers of the call at hand: a second call of the same shape whose temp1 (or Z) is
+    off the alignment of the whole-row kernel gets several launches and must then read the transposed X in place;
+    no launch may ever read and write the same buffer."""
+    for dt, M, P, N in [("s", 1024, 16, 4), ("s", 1024, 64, 2), ("d", 1024, 32, 2)]:
+        e, names, launches = plan(online_planner, "mkm", dt, M, [P] * N, [P] * N, opX=capi.OP_T, temp2=False)
+        assert e == capi.SUCCESS and names[0].startswith("transpose_") and len(names) == 2, (dt, P, names)
+        for offs in ({"t1": 4}, {"z": 4}, {"t1": 4, "z": 4}):
+            e, names, launches = plan(online_planner, "mkm", dt, M, [P] * N, [P] * N, opX=capi.OP_T, temp2=False, offs=offs)
+            assert e == capi.SUCCESS, (dt, P, offs)
+            for rec in launches:
+                assert rec["in"] != rec["out"], (dt, P, offs, names, rec)
+            if any(n.startswith("transpose_") for n in names):
+                assert len(names) == 2, (dt, P, offs, names)
+        # and the aligned call still gets the copy afterwards
+        e, names, _ = plan(online_planner, "mkm", dt, M, [P] * N, [P] * N, opX=capi.OP_T, temp2=False)
+        assert e == capi.SUCCESS and names[0].startswith("transpose_") and len(names) == 2, (dt, P, names)
+
+
+def test_leaving_plan_only_mode_drops_its_stand_in_workspace():
+    """Plan-only mode on a handle without a device uses a stand-in address for the merged-factor workspace; once the
+    mode is left, a call must not plan on it (it would be handed to kernels): without a device and a workspace the
+    chain is then not merged, and fastKronInitHIP allocates the real one."""
+    lib = capi.load()
+    h = ctypes.c_void_p()
+    assert lib.fastKronInit(ctypes.byref(h), capi.BACKEND_HIP) == capi.SUCCESS
+    try:
+        assert lib.fastKronSetPlanOnly(h, 1) == capi.SUCCESS
+        e, names, _ = plan((lib, h), "mkm", "s", 1024, [4] * 8, [4] * 8)
+        assert e == capi.SUCCESS and len(names) == 1 and "16x16" in names[0], names       # merged into 16x16^4
+        assert lib.fastKronSetPlanOnly(h, 0) == capi.SUCCESS
+        assert lib.fastKronSetPlanOnly(h, 1) == capi.SUCCESS
+        e, names, _ = plan((lib, h), "mkm", "s", 1024, [4] * 8, [4] * 8)
+        assert e == capi.SUCCESS and len(names) == 1 and "16x16" in names[0], names       # the stand-in is back, as before
+    finally:
+        lib.fastKronDestroy(h)
+
+
 def test_transposition_rules_that_came_from_tuned_plans(online_planner):
     planner = online_planner
     copied = lambda names: names[0].startswith("transpose_")
