@@ -9,7 +9,9 @@ configuration the headline metric is quoted on: sgemkm, X 1024 x 65536, four 16x
 Prints ONE JSON line: GFLOP/s with FastKron's FLOP count (2*M*sum_i Kin_i*Q_i), the roofline of the
 dominant kernel measured with HIP events on the library's stream, a CPU baseline (the oracle's
 vectorised OpenMP port) timed on the host cores in the same run, and under "configs" the same GPU figures
-(ms, GFLOP/s, roofline fraction, launches, kernels) for the other four configurations, timed the same way.
+(ms, GFLOP/s, roofline fraction, launches, kernels) for the other four configurations, timed the same way, under
+"cpu_baselines" the CPU figure of each of those, and under "published_shapes" the fp32 GeMKM shapes of the reference's
+published table (plus c1 / c2 transposed and as sgekmm) timed through the same handle.
 """
 import argparse
 import ctypes
@@ -249,6 +251,33 @@ def shape_table(fk):
                     torch.cuda.empty_cache()
 
 
+def published_shapes(fk, budget_s):
+    """The 15 fp32 GeMKM shapes of the reference's published table (documents/performance.md:9-23), plus c1 and c2's
+    shapes with both operands transposed and as sgekmm (the rows nearest to them there: :29-31, :89-91), through the
+    same handle, operands rotated so that the memory-side cache holds none, wall clock around batches of calls with
+    a device synchronisation on both sides.  Stops adding shapes once `budget_s` seconds are spent."""
+    import torch
+    from fastkron_amd.capi import OP_N, OP_T
+    from fastkron_amd.tune import _Case
+    todo = [("mkm", M, P, N, OP_N, "NN") for M, P, N in PUBLISHED_GPU_SHAPES]
+    todo += [("mkm", 1024, 8, 5, OP_T, "TT"), ("mkm", 1024, 16, 4, OP_T, "TT"),
+             ("kmm", 1024, 8, 5, OP_N, "NN"), ("kmm", 1024, 16, 4, OP_N, "NN")]
+    out, t_start = {}, time.perf_counter()
+    for mm, M, P, N, op, on in todo:
+        if time.perf_counter() - t_start > budget_s:
+            break
+        try:
+            case = _Case(fk, mm, M, [P] * N, [P] * N, torch.float32)
+        except torch.cuda.OutOfMemoryError:
+            continue
+        ms = case.time(fk, op, op, runs=10, samples=3)
+        out[f"s{'gemkm' if mm == 'mkm' else 'gekmm'}_{M}_{P}x{P}^{N}_{on}"] = {
+            "ms": round(ms, 5), "gflops": round(case.gflops(ms), 1), "launches": len(fk.last_plan())}
+        del case
+        torch.cuda.empty_cache()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -261,7 +290,10 @@ def main():
     ap.add_argument("--only", action="store_true", help="time the --config workload alone (profiling runs)")
     ap.add_argument("--tune", action="store_true", help="time candidate launch plans first (excluded from timing)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--cpu-seconds", type=float, default=10.0)
+    ap.add_argument("--cpu-seconds", type=float, default=10.0,
+                    help="CPU work spent on the headline workload's baseline (the other four get 3 s each)")
+    ap.add_argument("--published-seconds", type=float, default=45.0,
+                    help="time budget of the published-shapes leg (0 skips it)")
     ap.add_argument("--sets", type=int, default=3,
                     help="least number of operand sets rotated between steps; raised per workload until the sets add up "
                          "to 640 MB, so that the 256 MB Infinity Cache serves none of the traffic")
@@ -311,10 +343,22 @@ def main():
                             "roofline": {k: rf[k] for k in ("bound", "achieved", "peak", "unit", "frac")},
                             "launches": rf["launches_per_step"], "kernel": rf["kernel"]}
         out["configs"] = others
+        if args.published_seconds > 0:
+            out["published_shapes"] = published_shapes(fk, args.published_seconds)
     if not args.no_cpu:
         M, Ps, Qs, alpha, beta, batch = head["dims"]
         dt = np.float32 if head["dtype"] == "f32" else np.float64
         out["cpu_baseline"] = cpu_baseline(M, Ps, Qs, dt, alpha, beta, batch, args.cpu_seconds)
+        # the same port on the other configurations (c1 is the one the reference's own x86 case is stated on), so
+        # that every GPU figure of this line has its CPU figure from the same host beside it
+        if not args.only:
+            out["cpu_baselines"] = {}
+            for name in sorted(CONFIGS):
+                if name == args.config:
+                    continue
+                _, M, Ps, Qs, dts, alpha, beta, batch, _ = CONFIGS[name]
+                out["cpu_baselines"][name] = cpu_baseline(M, Ps, Qs, np.float32 if dts == "f32" else np.float64, alpha, beta,
+                                                          batch, 6.0 if name == "c1" else 3.0)
     print(json.dumps(out))
 
 

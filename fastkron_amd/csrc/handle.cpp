@@ -23,6 +23,7 @@ Handle::Handle(uint32_t backends) : backends_(backends) {
   // the plans that ship with the library first, then the user's own file on top of them
   const std::string shipped = KernelDB::shippedPath();
   if (!shipped.empty()) db_.loadFile(shipped, true);
+  if (const char* e = getenv("FASTKRON_CHUNK_MB")) chunkMB_ = atol(e);          // read when the handle is created
   dbPath_ = KernelDB::defaultPath();
   if (!dbPath_.empty()) db_.loadFile(dbPath_);
 }
@@ -643,6 +644,39 @@ fastKronError Handle::runSplit(const KronProblem& p, uint32_t g, const KronProbl
     lastPlan_ += ";" + std::to_string(g + s.lo) + "-" + std::to_string(g + s.hi) + ":" + db_.kernels()[s.kernel].name;
   for (auto& s : plan2)
     lastPlan_ += ";" + std::to_string(s.lo) + "-" + std::to_string(s.hi) + ":" + db_.kernels()[s.kernel].name;
+  // Rows are independent, and the intermediate between the two parts is written once and read once.  With
+  // FASTKRON_CHUNK_MB set, the rows go through the two parts in chunks whose intermediate has that size, every chunk
+  // through the same stretch of temp1, so that the second part reads what the first wrote from the 256 MB memory-side
+  // cache and the stretch is overwritten before most of it has to go out to HBM.  Off by default: measured on an
+  // MI355X it loses (dgemkm 256 x 64^3: 496 us unchunked, 548 / 569 / 601 us with chunks of 192 / 128 / 64 MB; sgemkm
+  // 1024 x 16^5: 2.98 ms against 3.33 ms at 128 MB; 1024 x 8^6, 1024 x 32^4, dgemkm 1024 x 16^4, sgemkm 16 x 16^6 likewise):
+  // each chunk's launches start and drain on their own, which costs more than the cache returns.
+  // (reference src/kmm/kmmalgo.cpp:72-115 plans whole-problem intermediates.)
+  const uint32_t chunkRows = chunkRowsForCache(p, q2);
+  auto forChunks = [&](bool dry) -> fastKronError {
+    const size_t es = dtypeSize(p.dt);
+    const uint64_t K = q2.strideX;                              // elements of one row of the problem
+    const uint64_t KA = q1.M / p.M;                             // blocks of a row
+    for (uint32_t m0 = 0; m0 < p.M; m0 += chunkRows) {
+      const uint32_t rows = p.M - m0 < chunkRows ? p.M - m0 : chunkRows;
+      KronProblem c1 = q1, c2 = q2;
+      c1.M = (uint32_t)(rows * KA);
+      c1.X = (const char*)q1.X + (size_t)m0 * K * es;
+      c2.batch = rows;
+      c2.Z = (char*)q2.Z + (size_t)m0 * K * es;
+      if (q2.Y) c2.Y = (const char*)q2.Y + (size_t)m0 * K * es;
+      fastKronError e = execute(c1, plan1, nullptr, nullptr, dry);
+      if (e != fastKronSuccess) return e;
+      e = execute(c2, plan2, temp2, nullptr, dry);
+      if (e != fastKronSuccess) return e;
+    }
+    return fastKronSuccess;
+  };
+  if (chunkRows < p.M) {
+    if (planOnly_) { launchLog_.clear(); return forChunks(true); }
+    if (forChunks(true) != fastKronSuccess) return fastKronKernelNotFound;      // every chunk's buffers checked first
+    return forChunks(false);
+  }
   if (planOnly_) {
     launchLog_.clear();
     (void)execute(q1, plan1, nullptr, nullptr, true);
@@ -651,6 +685,17 @@ fastKronError Handle::runSplit(const KronProblem& p, uint32_t g, const KronProbl
   fastKronError e = execute(q1, plan1, nullptr, nullptr);
   if (e != fastKronSuccess) return e;
   return execute(q2, plan2, temp2, nullptr);
+}
+
+// Rows per chunk of a two-part plan (p.M: no chunking, the default).  FASTKRON_CHUNK_MB=<n> sets the size of a
+// chunk's intermediate.
+uint32_t Handle::chunkRowsForCache(const KronProblem& p, const KronProblem& q2) const {
+  const long forcedMB = chunkMB_;
+  if (forcedMB <= 0 || p.batch != 1 || p.M < 2 || p.forward) return p.M;
+  const uint64_t rowBytes = q2.strideX * dtypeSize(p.dt);
+  uint64_t rows = ((uint64_t)forcedMB << 20) / rowBytes;
+  if (rows < 1) rows = 1;
+  return rows >= p.M ? p.M : (uint32_t)rows;
 }
 
 // The online rule for the two-part plan: how many trailing factors one whole-block kernel takes.

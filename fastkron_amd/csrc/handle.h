@@ -70,6 +70,7 @@ class Handle {
   bool buildSplit(const KronProblem& p, uint32_t g, void* temp1, void* temp2, KronProblem* q1, KronProblem* q2) const;
   fastKronError runSplit(const KronProblem& p, uint32_t g, const KronProblem& q1, const Plan& plan1,
                          const KronProblem& q2, const Plan& plan2, void* temp2);
+  uint32_t chunkRowsForCache(const KronProblem& p, const KronProblem& q2) const;
   // MKM chains longer than a whole-row kernel can take: trailing factors by the row kernel on
   // M * prod(leading P) virtual rows, leading factors as a batched KMM over the row blocks.
   // Returns fastKronKernelNotFound when the problem does not have that form.
@@ -118,6 +119,7 @@ class Handle {
   bool mergeWsUsed_ = false;
   hipEvent_t mergeWsEvent_ = nullptr;                 // orders a new stream behind the last user of the workspace
   bool planOnly_ = false;
+  long chunkMB_ = 0;                                  // FASTKRON_CHUNK_MB: two-part plans run in row chunks of this size (0: whole)
   bool callWs_ = false;                               // the running call brought its own workspace (touches none of the handle's)
   std::string launchLog_;
 };

@@ -1020,3 +1020,20 @@ def test_z_is_y_at_full_size_on_the_two_phase_4x4_kernel(fk):
     assert err_rows <= 1e-5 and err_sum <= 1e-5, (err_rows, err_sum)
     err_rows, err_sum = sampled_check(fk, ko.MKM, 256, [64] * 3, [64] * 3, np.float64, alpha=1.0, beta=1.0, y_is_z=True)
     assert err_rows <= 1e-12 and err_sum <= 1e-12, (err_rows, err_sum)
+
+
+def test_two_part_plan_in_row_chunks(monkeypatch):
+    """FASTKRON_CHUNK_MB: the rows of a two-part plan go through its two parts in chunks that share one stretch of
+    temp1 (off by default).  Chunks of 1 MB: 16 rows of 16^4 fp32 at a time, the last chunk ragged; with Y, Z == Y."""
+    import fastkron_amd
+    monkeypatch.setenv("FASTKRON_CHUNK_MB", "1")
+    h = fastkron_amd.FastKron()
+    monkeypatch.delenv("FASTKRON_CHUNK_MB")
+    try:
+        check(h, ko.MKM, 5, [16] * 5, [16] * 5, np.float32, alpha=1.5, beta=0.5, seed=601)       # 4 MB per row: row by row
+        assert len(h.last_plan()) == 2, h.last_plan()
+        check(h, ko.MKM, 37, [8] * 6, [8] * 6, np.float32, alpha=1.0, beta=0.0, seed=602)        # 1 MB per row
+        check(h, ko.MKM, 70, [16] * 4, [16] * 4, np.float64, alpha=2.0, beta=1.0, seed=603, y_is_z=True)   # 2 rows per chunk
+        check(h, ko.MKM, 3, [64] * 3, [64] * 3, np.float64, alpha=1.0, beta=0.0, seed=604)
+    finally:
+        h.close()
