@@ -251,6 +251,53 @@ def shape_table(fk):
                     torch.cuda.empty_cache()
 
 
+def pattern_ceilings(fk, steps, warmup, ev, stream):
+    """c4's bytes (X, Y read, Z written, 4096 x 2048 fp32 each) moved by copy kernels that have the access pattern of a
+    4x4^6 GeKMM kernel and none of its arithmetic (include/fastkron_ext.h, fastKronProbeCopyPattern), timed like the
+    configurations: 7 operand sets rotated (672 MB per rotation), hipEvents on the library's stream."""
+    import torch
+    from fastkron_amd import capi
+    M, n = 2048, 4096 * 2048
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(0xFA57C0DE)
+    sets = [tuple(torch.rand(n, generator=gen, device=dev) * 2 - 1 for _ in range(2)) + (torch.empty(n, device=dev),)
+            for _ in range(7)]
+    T = torch.empty(n, device=dev)
+    names = {0: "contiguous 16-byte accesses", 1: "32-byte strips of 8 columns x 4096 rows per workgroup",
+             2: "256-byte pieces, two phases, intermediate through the L2"}
+    out = {}
+    for pattern, label in names.items():
+        def step(i):
+            X, Y, Z = sets[i % len(sets)]
+            e = fk.lib.fastKronProbeCopyPattern(fk.h, pattern, X.data_ptr(), Y.data_ptr(), Z.data_ptr(), T.data_ptr(), M)
+            if e != capi.SUCCESS:
+                raise RuntimeError(f"fastKronProbeCopyPattern failed with fastKronError {e}")
+        t_ramp = time.perf_counter()
+        while time.perf_counter() - t_ramp < 0.25:
+            for i in range(20):
+                step(i)
+            torch.cuda.synchronize()
+        for i in range(max(warmup, 1)):
+            step(i)
+        torch.cuda.synchronize()
+        e0, e1 = ev.create(), ev.create()
+        ev.record(e0, stream)
+        for i in range(steps):
+            step(i)
+        ev.record(e1, stream)
+        torch.cuda.synchronize()
+        ms = ev.elapsed_ms(e0, e1) / steps
+        X, Y, Z = sets[(steps - 1) % len(sets)]
+        # (the strips are read in the order of the kernel's first phase and written in that of its second: a permuted copy)
+        ok = bool(torch.allclose(Z, 1.5 * X + 0.5 * Y, rtol=0, atol=1e-5)) if pattern != 1 else None
+        gbs = 3 * n * 4 / (ms * 1e-3) / 1e9
+        out[str(pattern)] = {"pattern": label, "ms": round(ms, 5), "gbs": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
+                             "copy_is_exact": ok}
+    out["sync_error"] = fk.sync_error()
+    return out
+
+
 def published_shapes(fk, budget_s):
     """The 15 fp32 GeMKM shapes of the reference's published table (documents/performance.md:9-23), plus c1 and c2's
     shapes with both operands transposed and as sgekmm (the rows nearest to them there: :29-31, :89-91), through the
@@ -301,6 +348,9 @@ def main():
                     help="instead of the benchmark line: time the shapes of the reference's published GPU table "
                          "(reference documents/performance.md:5-137: M_PxP^N for MKM and KMM, float and double, operands "
                          "untransposed and transposed) with cold operands and print one JSON line per shape")
+    ap.add_argument("--pattern-ceilings", action="store_true",
+                    help="instead of the benchmark line: time copy kernels with the access patterns of the 4x4^6 GeKMM "
+                         "kernels on c4's operands (what the memory system gives each pattern) and print one JSON line")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run 4 plain device copies of 256 MiB (a known-size kernel for scaling rocprof counters)")
     args = ap.parse_args()
@@ -319,6 +369,12 @@ def main():
 
     if args.shape_table:
         shape_table(fk)
+        return
+    if args.pattern_ceilings:
+        out = pattern_ceilings(fk, args.steps, args.warmup, ev, sp)
+        out["c4"] = {k: v for k, v in measure(fk, "c4", args.steps, args.warmup, args.ramp_seconds, args.sets, ev, sp).items()
+                     if k in ("gpu_ms_per_step", "roofline")}
+        print(json.dumps(out))
         return
     head = measure(fk, args.config, args.steps, args.warmup, args.ramp_seconds, args.sets, ev, sp, args.calibrate_copy)
     out = {

@@ -29,7 +29,8 @@ EXPORTS = [
 ]
 
 EXT_EXPORTS = ["fastKronGetLastPlan", "fastKronSetTunedDB", "fastKronSetPlanOnly", "fastKronGetLastLaunches",
-               "sgemkmStaticScratch", "fastKronGetSyncError", "fastKronSetSyncHelpAfter"]     # include/fastkron_ext.h
+               "sgemkmStaticScratch", "fastKronGetSyncError", "fastKronSetSyncHelpAfter",
+               "fastKronProbeCopyPattern"]     # include/fastkron_ext.h
 
 _lib = None
 
@@ -94,6 +95,7 @@ def load():
     lib.sgemkmStaticScratch.restype = cint
     lib.fastKronGetSyncError.argtypes = [vp, u32p]
     lib.fastKronSetSyncHelpAfter.argtypes = [u32]
+    lib.fastKronProbeCopyPattern.argtypes = [vp, cint, vp, vp, vp, vp, u32]
     lib.fastKronSetPlanOnly.argtypes = [vp, cint]
     lib.fastKronGetLastLaunches.argtypes = [vp, ctypes.c_char_p, ctypes.c_size_t]
     lib.fastKronGetLastLaunches.restype = ctypes.c_size_t

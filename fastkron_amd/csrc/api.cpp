@@ -105,6 +105,13 @@ fastKronError fastKronGetSyncError(fastKronHandle handle, uint32_t* word) {
   return H(handle)->syncError(word);
 }
 
+fastKronError fastKronProbeCopyPattern(fastKronHandle handle, int pattern, const float* X, const float* Y, float* Z,
+                                       float* T, uint32_t M) {
+  if (!handle) return fastKronInvalidArgument;
+  return fk::launchPatternProbe(pattern, X, Y, Z, T, H(handle)->syncArea(), M, H(handle)->stream()) == hipSuccess
+             ? fastKronSuccess : fastKronInvalidArgument;
+}
+
 fastKronError fastKronSetSyncHelpAfter(uint32_t polls) {
   fk::setKmm4x6TwoPhaseHelpAfter(polls);
   return fastKronSuccess;

@@ -25,7 +25,7 @@
 // Each workgroup of four waves works on the block's two halves of 128 columns (units A and B) one behind the other:
 // X of both is requested at the start; as A arrives it is contracted and stored to T, Y of A is requested (it is not
 // needed before the end, but the memory system must not run dry meanwhile), then the same for B; then T of A and B
-// is read back, contracted and Z stored.  Loads and stores of a wave complete in issue order, so "T is stored" is
+// are read back, contracted and Z stored, unit A before unit B is waited for.  Loads and stores of a wave complete in issue order, so "T is stored" is
 // known when at most as many younger operations are outstanding as were issued behind the stores.
 //
 // Synchronisation without assuming that all workgroups are resident at once.  Per block and unit a bit mask of the
@@ -231,11 +231,6 @@ __global__ __launch_bounds__(256) void kron_kmm4x6_twophase_kernel(const StepArg
       markDone(job, 1);
     }
   }
-  // (a full mask of unit A means that every job has at least started its unit B, which nothing holds up: only wait)
-  for (uint32_t spins = 0; tid == 0 && t6L2Load(words + 1, zero) != ~0u; spins++) {
-    if (spins >= kT6SpinLimit) { (void)__hip_atomic_fetch_or(sync + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); break; }
-    __builtin_amdgcn_s_sleep(4);
-  }
   auto loadT = [&](int unit, float (&x)[64]) __attribute__((always_inline)) {
     const uint32_t off = (uint32_t)(unit * (64 * 64 * 128) + s * (64 * 128)) * 4;
 #pragma unroll
@@ -253,15 +248,21 @@ __global__ __launch_bounds__(256) void kron_kmm4x6_twophase_kernel(const StepArg
       __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), zRes, lane4, off + (r * 64) * ldo, 2);
     }
   };
+  // Unit A is finished before unit B is waited for (measured: 29.2 us against 31.0 with the intermediates of both
+  // units read back first).
+  loadT(0, xa);
+  storeZ(0, xa, ya);
+  // (a full mask of unit A means that every job has at least started its unit B, which nothing holds up: only wait)
+  for (uint32_t spins = 0; tid == 0 && t6L2Load(words + 1, zero) != ~0u; spins++) {
+    if (spins >= kT6SpinLimit) { (void)__hip_atomic_fetch_or(sync + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); break; }
+    __builtin_amdgcn_s_sleep(4);
+  }
   // this workgroup is through with the block's words: said now, the answer (am I the last?) is looked at at the end
   uint32_t through = 0;
   if (tid == 0) through = t6L2Add(words + 2, 1u);
   __syncthreads();
   __builtin_amdgcn_sched_barrier(0);
-  loadT(0, xa);
   loadT(1, xb);
-  __builtin_amdgcn_sched_barrier(0);
-  storeZ(0, xa, ya);
   storeZ(1, xb, yb);
   // the last of the block's workgroups to be through zeroes the words for the next launch (the same L2 serves it)
   if (tid == 0 && through + 1 == (uint32_t)kT6Jobs) {

@@ -139,6 +139,11 @@ bool kmm4x6TwoPhasePlacementHolds(uint32_t* scratchWords, hipStream_t stream);
 // Polls after which a waiting workgroup of that kernel runs missing jobs itself (tests set 0).
 void setKmm4x6TwoPhaseHelpAfter(uint32_t polls);
 
+// Copy kernels with the access patterns of the two kernels above (0 contiguous, 1 strips, 2 two phases): Z = 1.5 X + 0.5 Y
+// on 4096 x M fp32.  Measurement only (bench.py --pattern-ceilings).
+hipError_t launchPatternProbe(int pattern, const float* X, const float* Y, float* Z, float* T, void* sync, uint32_t M,
+                              hipStream_t stream);
+
 // KMM layout, fp32: three fused 4x4 or two fused 8x8 factors held in registers, lanes along M.
 bool kmmRegSupported(const StepArgs& a);
 hipError_t launchKmmReg(const StepArgs& a, hipStream_t stream);

@@ -68,6 +68,16 @@ fastKronError sgemkmStaticScratch(fastKronHandle handle, fastKronBackend backend
 fastKronError fastKronGetSyncError(fastKronHandle handle, uint32_t* word);
 fastKronError fastKronSetSyncHelpAfter(uint32_t polls);
 
+/*
+ * Measurement aid, no counterpart in the reference: launches on the handle's stream a copy kernel Z = 1.5 X + 0.5 Y over
+ * 4096 x M fp32 matrices (M a multiple of 2048, at most 16384) that touches memory the way one of the 4x4^6 GeKMM kernels
+ * does and computes nothing else.  pattern 0: contiguous 16-byte accesses; 1: 32-byte strips of 8 columns, all 4096
+ * rows per workgroup; 2: 256-byte pieces in two phases with an intermediate T (4096 x M floats) passed through the
+ * L2 and workgroups waiting for each other.  `python bench.py --pattern-ceilings` times them beside the kernels.
+ */
+fastKronError fastKronProbeCopyPattern(fastKronHandle handle, int pattern, const float* X, const float* Y, float* Z,
+                                       float* T, uint32_t M);
+
 #ifdef __cplusplus
 }
 #endif
