@@ -141,7 +141,7 @@ static bool row16CanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, 
   return dev.ldsPerBlock >= 131072 && k.dt == p.dt;
 }
 static hipError_t row16Launch(const KernelInfo& k, const StepArgs& a, hipStream_t s) {
-  return k.threads == 512 ? launchRow16x4W8(a, s) : launchRow16x4(a, s);
+  return k.threads == 512 ? launchRow16x4W8(a, s) : launchRow16x4(a, s, k.variant == 0);
 }
 static bool row16Check(const KernelInfo& k, const StepArgs& a) {
   return k.threads == 512 ? row16x4W8Supported(a) : row16x4Supported(a);
@@ -159,7 +159,7 @@ static bool row8CanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, u
   if (first && p.opX == 2) return false;
   return dev.ldsPerBlock >= 67000 && k.dt == p.dt;
 }
-static hipError_t row8Launch(const KernelInfo&, const StepArgs& a, hipStream_t s) { return launchRow8x5(a, s); }
+static hipError_t row8Launch(const KernelInfo& k, const StepArgs& a, hipStream_t s) { return launchRow8x5(a, s, (int)k.variant); }
 static bool row8Check(const KernelInfo&, const StepArgs& a) { return row8x5Supported(a); }
 
 // ---- wave-per-block kernel for two or three fused PxP factors, 9 <= P <= 16 ----
@@ -212,7 +212,7 @@ static bool row32x3Check(const KernelInfo&, const StepArgs& a) { return row32x3S
 // ---- single-factor fp32 step for 64x64 and 128x128, whole-line accesses through LDS (variant 3: MKM, 4: KMM) ----
 static bool stepWideCanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
                            const DeviceInfo&) {
-  const MMType mm = (k.variant == 4) ? MMType::KMM : MMType::MKM;
+  const MMType mm = ((k.variant & 255) == 4) ? MMType::KMM : MMType::MKM;
   if (p.dt != k.dt || p.mm != mm || lo != hi) return false;
   if (p.P[lo] != k.P || p.Q[lo] != k.Q) return false;
   if (first && p.opX == 2) return false;
@@ -220,7 +220,7 @@ static bool stepWideCanRun(const KernelInfo& k, const KronProblem& p, uint32_t l
   const uint64_t TS = 16384 / dtypeSize(k.dt) / k.P;
   return mm == MMType::KMM ? p.M % TS == 0 : (p.colsBefore(hi) / k.P) % TS == 0;
 }
-static hipError_t stepWideLaunch(const KernelInfo& k, const StepArgs& a, hipStream_t s) { return launchStepWide(a, k.dt, s); }
+static hipError_t stepWideLaunch(const KernelInfo& k, const StepArgs& a, hipStream_t s) { return launchStepWide(a, k.dt, s, (int)(k.variant >> 8)); }
 static bool stepWideCheck(const KernelInfo& k, const StepArgs& a) { return stepWideSupported(a, k.dt); }
 
 // ---- single-factor MFMA step (fp64 and fp32) ----
@@ -293,6 +293,9 @@ static bool kmm4x6CanRun(const KernelInfo&, const KronProblem& p, uint32_t lo, u
   // together and their 32-byte pieces meet in its L2.  With more tiles than CUs that order is lost and the
   // two-launch plan, which reads 256 bytes per row and wave, is faster (measured from M = 4096 on).
   if (dev.rulesOfThumb && (uint64_t)(p.M / 8) * p.batch > (uint64_t)dev.cus) return false;
+  // With fewer than 128 tiles half of the CUs or more stand idle and the two-launch plan is ahead (tuned: 512 columns
+  // 20.0 against 17.1 us; 1024 columns 23.4 against 23.3).
+  if (dev.rulesOfThumb && (uint64_t)(p.M / 8) * p.batch < 128) return false;
   return dev.ldsPerBlock >= (8 * 64 * 65 + 32) * 4;
 }
 // The two-phase form: M a multiple of 256.  By rule only from 2048 columns on (one column block per XCD), where it
@@ -360,6 +363,13 @@ void registerRowKernels(std::vector<KernelInfo>& out) {
     k.dt = DType::F32; k.P = 16; k.Q = 16; k.fused = 4; k.tileM = 1; k.tileK = 65536; k.threads = threads; k.variant = 0;
     k.canRun = row16CanRun; k.launch = row16Launch; k.check = row16Check;
     out.push_back(k);
+    if (threads == 1024) {
+      // for the tuner: all workgroups started at once ("ns" in the tile field) instead of in groups
+      KernelInfo v = k;
+      v.name = "mkm_hip_gfx950_1024_f_16x16_16x16_4_1x65536ns_mfma16x16x4_NN_strided_0_3";
+      v.variant = 1; v.tunerOnly = true;
+      out.push_back(v);
+    }
   }
 
   KernelInfo k8{};
@@ -367,6 +377,14 @@ void registerRowKernels(std::vector<KernelInfo>& out) {
   k8.dt = DType::F32; k8.P = 8; k8.Q = 8; k8.fused = 5; k8.tileM = 1; k8.tileK = 32768; k8.threads = 512; k8.variant = 0;
   k8.canRun = row8CanRun; k8.launch = row8Launch; k8.check = row8Check;
   out.push_back(k8);
+  // the same kernel under other schedules, for the tuner: one workgroup per CU ("wg1"), two without the start delay
+  // of the later one ("wg2nd"); the tile field of the name carries the schedule
+  for (uint32_t schedule : {1u, 2u}) {
+    KernelInfo v = k8;
+    v.name = std::string("mkm_hip_gfx950_512_f_8x8_8x8_5_1x32768") + (schedule == 1 ? "wg1" : "wg2nd") + "_mfma4x4x1_NN_strided_0_3";
+    v.variant = schedule; v.tunerOnly = true;
+    out.push_back(v);
+  }
 
   KernelInfo k32{};
   k32.name = "mkm_hip_gfx950_512_f_32x16_32x16_3_1x32768_mfma16x16x4_NN_strided_0_3";
@@ -465,6 +483,14 @@ void registerRowKernels(std::vector<KernelInfo>& out) {
     kw.tileK = variant == 4 ? P : E; kw.threads = 256; kw.variant = variant;
     kw.canRun = stepWideCanRun; kw.launch = stepWideLaunch; kw.check = stepWideCheck;
     out.push_back(kw);
+    // for the tuner: the same kernel with at most one / two persistent workgroups per CU ("wg1", "wg2" in the tile field)
+    for (uint32_t cap : {1u, 2u}) {
+      KernelInfo v = kw;
+      const size_t at = v.name.find("_mfma16x16x4lds");
+      v.name.insert(at, "wg" + std::to_string(cap));
+      v.variant = variant | (cap << 8); v.tunerOnly = true;
+      out.push_back(v);
+    }
   }
 
   // variant 1 = the same kernel on the KMM layout (tiles of 16 consecutive m)

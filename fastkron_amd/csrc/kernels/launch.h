@@ -76,7 +76,7 @@ hipError_t launchGenericStep(const StepArgs& a, DType dt, hipStream_t stream);
 
 // Four fused 16x16 fp32 factors on rows of exactly 16^4 columns, one workgroup per row.
 bool row16x4Supported(const StepArgs& a);
-hipError_t launchRow16x4(const StepArgs& a, hipStream_t stream);
+hipError_t launchRow16x4(const StepArgs& a, hipStream_t stream, bool staggered = true);
 
 // The same with 8 waves of 128 values per lane and the whole next block prefetched.
 bool row16x4W8Supported(const StepArgs& a);
@@ -84,7 +84,7 @@ hipError_t launchRow16x4W8(const StepArgs& a, hipStream_t stream);
 
 // Five fused 8x8 fp32 factors on rows of exactly 8^5 columns, one workgroup per row, two per CU.
 bool row8x5Supported(const StepArgs& a);
-hipError_t launchRow8x5(const StepArgs& a, hipStream_t stream);
+hipError_t launchRow8x5(const StepArgs& a, hipStream_t stream, int schedule = 0);
 
 // Three fused 32x16 fp32 factors on rows of exactly 32^3 columns, one workgroup per row, two per CU.
 bool row32x16x3Supported(const StepArgs& a);
@@ -102,7 +102,7 @@ hipError_t launchKmm8x3(const StepArgs& a, hipStream_t stream);
 
 // One step with a 64x64 or 128x128 factor, either type and layout, tiles of 16 KB passed through LDS.
 bool stepWideSupported(const StepArgs& a, DType dt);
-hipError_t launchStepWide(const StepArgs& a, DType dt, hipStream_t stream);
+hipError_t launchStepWide(const StepArgs& a, DType dt, hipStream_t stream, int maxWorkgroupsPerCU = 0);
 
 // One step with a 16x16 ... 128x128 factor on the matrix cores, fp64 or fp32, MKM or KMM layout.
 bool stepMfmaSupported(const StepArgs& a, DType dt);

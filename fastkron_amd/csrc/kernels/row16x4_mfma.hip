@@ -288,7 +288,8 @@ bool row16x4Supported(const StepArgs& a) {
   return a.batch <= 65535;
 }
 
-hipError_t launchRow16x4(const StepArgs& a, hipStream_t stream) {
+// stagger: start the workgroups in groups some microseconds apart (the online choice) or all at once (a tuner candidate)
+hipError_t launchRow16x4(const StepArgs& a, hipStream_t stream, bool staggered) {
   if (!row16x4Supported(a)) return hipErrorInvalidValue;
   static PerDeviceOnce attrOnce;
   const int devIdx = launchDeviceIndex();
@@ -311,7 +312,7 @@ hipError_t launchRow16x4(const StepArgs& a, hipStream_t stream) {
   if (total >= (1ull << 32) - 65536) return hipErrorInvalidValue;      // item + gridDim.x stays a 32-bit number
   // persistent workgroups, one per CU
   const uint32_t wgs = total < (uint64_t)cus ? (uint32_t)total : (uint32_t)cus;
-  const uint32_t stagger = total >= 2ull * wgs ? kStaggerTicks : 0;
+  const uint32_t stagger = (staggered && total >= 2ull * wgs) ? kStaggerTicks : 0;
   dim3 grid(wgs), block(1024);
   hipLaunchKernelGGL(kernels[(a.y && a.epilogue) ? 1 : 0][streamMode(a)], grid, block, ldsBytes, stream, a, blocksPerBatch,
                      (uint32_t)total, stagger);

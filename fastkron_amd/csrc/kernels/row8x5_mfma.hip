@@ -237,11 +237,14 @@ bool row8x5Supported(const StepArgs& a) {
   return a.batch <= 65535;
 }
 
-hipError_t launchRow8x5(const StepArgs& a, hipStream_t stream) {
+// schedule: 0 = two workgroups per CU, the later one of a CU started kRow8SlotDelayTicks behind (the online choice);
+// 1 = one workgroup per CU (the launch asks for more LDS than two workgroups can have); 2 = two per CU without the delay.
+hipError_t launchRow8x5(const StepArgs& a, hipStream_t stream, int schedule) {
   if (!row8x5Supported(a)) return hipErrorInvalidValue;
   static PerDeviceOnce attrOnce;
   const int devIdx = launchDeviceIndex();
-  const size_t ldsBytes = kRow8LdsWords * sizeof(float);
+  const size_t ldsMax = 96 * 1024;
+  const size_t ldsBytes = schedule == 1 ? ldsMax : kRow8LdsWords * sizeof(float);
   using Kernel = void (*)(const StepArgs, const uint32_t, const uint32_t);
   static const Kernel kernels[2][3] = {
       {kron_row8x5_kernel<false, 0>, kron_row8x5_kernel<false, 1>, kron_row8x5_kernel<false, 2>},
@@ -249,7 +252,7 @@ hipError_t launchRow8x5(const StepArgs& a, hipStream_t stream) {
   if (!attrOnce.done(devIdx)) {
     for (int y = 0; y < 2; y++)
       for (int nt = 0; nt < 3; nt++) {
-        hipError_t e = hipFuncSetAttribute((const void*)kernels[y][nt], hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes);
+        hipError_t e = hipFuncSetAttribute((const void*)kernels[y][nt], hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsMax);
         if (e != hipSuccess) return e;
       }
     attrOnce.mark(devIdx);
@@ -257,7 +260,7 @@ hipError_t launchRow8x5(const StepArgs& a, hipStream_t stream) {
   dim3 grid(a.M / row8Rows(a), a.batch), block(512);
   const uint32_t firstRound = 2u * (uint32_t)deviceCUs();
   hipLaunchKernelGGL(kernels[(a.y && a.epilogue) ? 1 : 0][streamMode(a)], grid, block, ldsBytes, stream, a, firstRound,
-                     kRow8SlotDelayTicks);
+                     schedule == 0 ? kRow8SlotDelayTicks : 0u);
   return hipGetLastError();
 }
 

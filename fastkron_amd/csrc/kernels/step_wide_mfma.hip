@@ -253,7 +253,7 @@ bool stepWideSupported(const StepArgs& a, DType dt) {
 }
 
 template <typename T, int P, bool KMM>
-static hipError_t launchStepWideT(const StepArgs& a, hipStream_t stream) {
+static hipError_t launchStepWideT(const StepArgs& a, hipStream_t stream, int maxPerCU) {
   const uint32_t E = kSwTileBytes / sizeof(T), TS = E / P;
   const uint32_t tilesPerLine = KMM ? a.M / TS : (uint32_t)(a.Kin / E);
   const uint32_t totalTiles = KMM ? (uint32_t)(a.Kin / P) * tilesPerLine : tilesPerLine * a.M;
@@ -267,6 +267,7 @@ static hipError_t launchStepWideT(const StepArgs& a, hipStream_t stream) {
     if (occ > 4) occ = 4;
     occCache[devIdx].store(occ, std::memory_order_relaxed);
   }
+  if (maxPerCU > 0 && occ > maxPerCU) occ = maxPerCU;          // (a tuner candidate: fewer, longer-running workgroups)
   uint32_t wgs = (uint32_t)occ * (uint32_t)deviceCUs();
   if (a.batch > 1) wgs = (wgs + a.batch - 1) / a.batch;
   if (wgs > totalTiles) wgs = totalTiles;
@@ -285,18 +286,18 @@ static hipError_t launchStepWideT(const StepArgs& a, hipStream_t stream) {
 }
 
 template <typename T>
-static hipError_t launchStepWideD(const StepArgs& a, hipStream_t stream) {
+static hipError_t launchStepWideD(const StepArgs& a, hipStream_t stream, int maxPerCU) {
   const uint32_t P = a.p[0];
   if (stepWideIsKmm(a))
-    return P == 128 ? launchStepWideT<T, 128, true>(a, stream) : P == 64 ? launchStepWideT<T, 64, true>(a, stream)
-                                                                         : launchStepWideT<T, 32, true>(a, stream);
-  return P == 128 ? launchStepWideT<T, 128, false>(a, stream) : P == 64 ? launchStepWideT<T, 64, false>(a, stream)
-                                                                        : launchStepWideT<T, 32, false>(a, stream);
+    return P == 128 ? launchStepWideT<T, 128, true>(a, stream, maxPerCU) : P == 64 ? launchStepWideT<T, 64, true>(a, stream, maxPerCU)
+                                                                         : launchStepWideT<T, 32, true>(a, stream, maxPerCU);
+  return P == 128 ? launchStepWideT<T, 128, false>(a, stream, maxPerCU) : P == 64 ? launchStepWideT<T, 64, false>(a, stream, maxPerCU)
+                                                                        : launchStepWideT<T, 32, false>(a, stream, maxPerCU);
 }
 
-hipError_t launchStepWide(const StepArgs& a, DType dt, hipStream_t stream) {
+hipError_t launchStepWide(const StepArgs& a, DType dt, hipStream_t stream, int maxWorkgroupsPerCU) {
   if (!stepWideSupported(a, dt)) return hipErrorInvalidValue;
-  return dt == DType::F32 ? launchStepWideD<float>(a, stream) : launchStepWideD<double>(a, stream);
+  return dt == DType::F32 ? launchStepWideD<float>(a, stream, maxWorkgroupsPerCU) : launchStepWideD<double>(a, stream, maxWorkgroupsPerCU);
 }
 
 }  // namespace fk

@@ -606,23 +606,47 @@ def test_two_part_plan_with_three_leading_launches(fk, dt):
     assert len(plan) == launches and plan[0][2].startswith("mkm_") and all(k.startswith("kmm_") for _, _, k in plan[1:]), plan
 
 
-@pytest.mark.parametrize("M", [8, 72, 512])
+WHOLE_COLUMN_4X6 = "kmm_hip_gfx950_512_f_4x4_4x4_6_8x4096_mfma4x4x1_NN_strided_0_3"
+
+
+@pytest.mark.parametrize("M", [1024, 1096, 1536])
 def test_kmm_six_4x4_factors_in_one_launch(fk, M):
-    """sgekmm with 4x4^6: one launch, every workgroup owns 8 columns and all 4096 rows of them."""
+    """sgekmm with 4x4^6 between 1024 and 2048 columns (and no multiple of 256 x 8): one launch, every workgroup owns 8
+    columns and all 4096 rows of them."""
     Ps = [4] * 6
     check(fk, ko.KMM, M, Ps, Ps, np.float32, alpha=1.5, beta=0.5, seed=191)
-    plan = fk.last_plan()
-    assert len(plan) == 1 and "_6_8x4096_" in plan[0][2], plan
+    assert [k for _, _, k in fk.last_plan()] == [WHOLE_COLUMN_4X6], fk.last_plan()
     check(fk, ko.KMM, M, Ps, Ps, np.float32, alpha=1.0, beta=0.0, seed=192, opFs=ko.OP_T)
-    check(fk, ko.KMM, M, Ps, Ps, np.float32, alpha=1.0, beta=1.0, seed=193, batch=3)
-    assert len(fk.last_plan()) == 1, fk.last_plan()
-    check(fk, ko.KMM, M, Ps, Ps, np.float32, alpha=2.0, beta=0.0, seed=194, batch=2, share_f=True)
     check(fk, ko.KMM, M, Ps, Ps, np.float32, alpha=1.0, beta=0.0, seed=195, integer=True, use_temp2=False)
-    # column counts that are not a multiple of 8, or more column tiles than CUs, keep the two-launch plan
+    assert [k for _, _, k in fk.last_plan()] == [WHOLE_COLUMN_4X6], fk.last_plan()
+    # column counts that are not a multiple of 8, fewer than 128 column tiles or more than there are CUs: two launches
     check(fk, ko.KMM, M + 12, Ps, Ps, np.float32, alpha=1.5, beta=0.5, seed=196)
     assert len(fk.last_plan()) == 2, fk.last_plan()
-    check(fk, ko.KMM, M, Ps, Ps, np.float32, alpha=1.0, beta=1.0, seed=197, batch=40)
-    assert len(fk.last_plan()) == (1 if M * 40 // 8 <= 256 else 2), fk.last_plan()
+    check(fk, ko.KMM, M // 4, Ps, Ps, np.float32, alpha=1.5, beta=0.5, seed=198)
+    assert len(fk.last_plan()) == 2, fk.last_plan()
+    check(fk, ko.KMM, M // 2, Ps, Ps, np.float32, alpha=1.0, beta=1.0, seed=197, batch=5)
+    assert len(fk.last_plan()) == 2, fk.last_plan()
+
+
+def test_whole_column_4x4_kernel_on_few_columns_and_batches(tmp_path):
+    """The whole-column kernel where the online rules prefer two launches (fewer than 128 column tiles), as a tuned plan
+    may name it: 8, 72 and 512 columns, batches with per-batch and shared factors."""
+    import fastkron_amd
+    db = tmp_path / "plans.txt"
+    keys = ["(4x4^6)*4096x8_NN_f", "(4x4^6)*4096x72_NN_f", "(4x4^6)*4096x512_NN_f", "(4x4^6)*4096x72_NN_f_stridedBatched_3",
+            "(4x4^6)*4096x8_NN_f_stridedBatched_2_Fs3f", "(4x4^6)*4096x72_NT_f"]
+    db.write_text("".join(f"{k} 0.1 M0 S0 1 0 5 {WHOLE_COLUMN_4X6}\n" for k in keys))
+    h = fastkron_amd.FastKron()
+    h.set_tuned_db(str(db))
+    try:
+        Ps = [4] * 6
+        for M, kw in [(8, dict(alpha=1.5, beta=0.5)), (72, dict(alpha=1.0, beta=0.0)), (512, dict(alpha=2.0, beta=1.0)),
+                      (72, dict(alpha=1.0, beta=1.0, batch=3)), (8, dict(alpha=2.0, beta=0.0, batch=2, share_f=True)),
+                      (72, dict(alpha=1.0, beta=0.0, opFs=ko.OP_T))]:
+            check(h, ko.KMM, M, Ps, Ps, np.float32, seed=199 + M, **kw)
+            assert [k for _, _, k in h.last_plan()] == [WHOLE_COLUMN_4X6], h.last_plan()
+    finally:
+        h.close()
 
 
 TWO_PHASE_4X6 = "kmm_hip_gfx950_256_f_4x4_4x4_6_256x4096_mfma4x4x1_NN_strided_0_3"
@@ -958,7 +982,7 @@ def test_kmm_three_fused_8x8_factors(fk, mm, M, Ps, launches):
 # Y and writes Z from registers laid out its own way, and must read an element before it writes it. ----
 IN_PLACE = [
     # kernel family, mm, M, Ps, Qs, dtype, extra
-    ("whole-column 4x4^6", ko.KMM, 512, [4] * 6, [4] * 6, np.float32, {}),
+    ("whole-column 4x4^6", ko.KMM, 1032, [4] * 6, [4] * 6, np.float32, {}),
     ("4x4x3 register kernel, two launches", ko.KMM, 100, [4] * 6, [4] * 6, np.float32, {}),
     ("32x16^3 row kernel, batched", ko.MKM, 8, [32] * 3, [16] * 3, np.float32, dict(batch=3)),
     ("16x16^4 row kernel", ko.MKM, 6, [16] * 4, [16] * 4, np.float32, {}),

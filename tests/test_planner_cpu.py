@@ -126,7 +126,8 @@ VECTOR_CASES = [
     ("kmm64d", "kmm", "d", 64, [64], [64], 8, 0.5, "kmm_hip_gfx950_256_d_64x64_64x64_1_64x64"),
     ("row8x5", "mkm", "s", 64, [8] * 5, [8] * 5, None, 0.5, "_8x8_8x8_5_1x32768"),
     ("row32x16", "mkm", "s", 64, [32] * 3, [16] * 3, None, 0.5, "_32x16_32x16_3_1x32768"),
-    ("kmm4x6", "kmm", "s", 64, [4] * 6, [4] * 6, None, 0.5, "_4x4_4x4_6_8x4096"),
+    ("kmm4x6", "kmm", "s", 1032, [4] * 6, [4] * 6, None, 0.5, "_4x4_4x4_6_8x4096"),
+    ("kmm4x6 two-phase", "kmm", "s", 2048, [4] * 6, [4] * 6, None, 0.5, "_4x4_4x4_6_256x4096"),
     ("wide128", "mkm", "s", 8, [128] * 2, [128] * 2, None, 0.5, "_128x128_128x128_1_1x4096_mfma16x16x4lds"),
     ("wide64k", "kmm", "s", 64, [64] * 2, [64] * 2, None, 0.5, "_64x64_64x64_1_64x64_mfma16x16x4lds"),
 ]

@@ -127,3 +127,37 @@ def test_shapes_with_a_shipped_plan_match_the_oracle(mm, M, Ps, dt, opX, opF):
         assert normwise(got, want) <= TOL[dt], h.last_plan()
     finally:
         h.close()
+
+
+VARIANTS = [
+    # problem string, factor range, kernel variant, (mm, M, Ps, dtype, kwargs)
+    ("64x32768*(8x8^5)_NN_f", 4, "mkm_hip_gfx950_512_f_8x8_8x8_5_1x32768wg1_mfma4x4x1_NN_strided_0_3", (ko.MKM, 64, [8] * 5, np.float32)),
+    ("64x32768*(8x8^5)_NN_f", 4, "mkm_hip_gfx950_512_f_8x8_8x8_5_1x32768wg2nd_mfma4x4x1_NN_strided_0_3", (ko.MKM, 64, [8] * 5, np.float32)),
+    ("600x65536*(16x16^4)_NN_f", 3, "mkm_hip_gfx950_1024_f_16x16_16x16_4_1x65536ns_mfma16x16x4_NN_strided_0_3", (ko.MKM, 600, [16] * 4, np.float32)),
+    ("96x16384*(128x128^2)_NN_f", -2, "mkm_hip_gfx950_256_f_128x128_128x128_1_1x4096wg1_mfma16x16x4lds_NN_strided_0_3", (ko.MKM, 96, [128] * 2, np.float32)),
+    ("128x4096*(64x64^2)_NN_d", -2, "mkm_hip_gfx950_256_d_64x64_64x64_1_1x2048wg2_mfma16x16x4lds_NN_strided_0_3", (ko.MKM, 128, [64] * 2, np.float64)),
+    ("(32x32^1)*32x256_NN_f", 0, "kmm_hip_gfx950_256_f_32x32_32x32_1_128x32wg1_mfma16x16x4lds_NN_strided_0_3", (ko.KMM, 256, [32], np.float32)),
+    ("(4x4^6)*4096x512_NN_f", 5, "kmm_hip_gfx950_256_f_4x4_4x4_6_256x4096_mfma4x4x1_NN_strided_0_3", (ko.KMM, 512, [4] * 6, np.float32)),
+]
+
+
+@pytest.mark.parametrize("key,hi,kernel,case", VARIANTS, ids=[v[2].split("_NN_")[0][16:] for v in VARIANTS])
+def test_tile_and_schedule_variants_that_only_the_tuner_chooses(tmp_path, key, hi, kernel, case):
+    """Kernels registered for the tuner alone (another tile, workgroups per CU or start schedule than the online rules
+    take; the variant is named in the tile field of the kernel string): a tuned-plan file naming one makes a handle run
+    it, and the result is the oracle's.  Counterpart of the tile sizes the reference's generator enumerates
+    (reference src/gen_tuner_kernels.py:396-469)."""
+    import fastkron_amd
+    mm, M, Ps, dt = case
+    db = tmp_path / "plans.txt"
+    # hi >= 0: one launch on factors 0..hi; hi = -n: n launches of one factor each
+    steps = [(0, hi, kernel)] if hi >= 0 else [(i, i, kernel) for i in range(-hi - 1, -1, -1)]
+    db.write_text(f"{key} 0.1 M0 S0 {len(steps)} " + " ".join(f"{lo} {h_} {k}" for lo, h_, k in steps) + "\n")
+    h = fastkron_amd.FastKron()
+    h.set_tuned_db(str(db))
+    try:
+        for alpha, beta, seed in [(1.5, 0.5, 701), (1.0, 0.0, 702)]:
+            run_and_check(h, mm, M, Ps, dt, alpha, beta, seed=seed)
+            assert h.last_plan() == steps, h.last_plan()
+    finally:
+        h.close()
