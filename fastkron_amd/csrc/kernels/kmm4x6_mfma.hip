@@ -90,12 +90,9 @@ __global__ __launch_bounds__(512) void kron_kmm4x6_kernel(const StepArgs a, cons
     for (int p = 0; p < 4; p++) fa[j][p] = F[(int64_t)p * a.f_sp[j] + (int64_t)(l & 3) * a.f_sq[j]];
   }
 
-  // Where Y is requested: 0 = right behind X, 1 = behind the first contraction, 2 = behind the exchange barrier.
-  // Measured with operands from HBM (no cache holding them): 36.6 / 37.7 / 40.4 us.  Holding Y back lets X arrive
-  // sooner, but the more requests are in flight the better this access pattern is served.
-#ifndef K6_YPOS
-#define K6_YPOS 0
-#endif
+  // Y is requested right behind X.  Measured with operands from HBM (no cache holding them) against requesting it
+  // behind the first contraction or behind the exchange barrier: 36.6 / 37.7 / 40.4 us.  Holding Y back lets X
+  // arrive sooner, but the more requests are in flight the better this access pattern is served.
   float yv[HAS_Y ? 64 : 1];
   auto loadY = [&]() {
     if (HAS_Y) {
@@ -110,22 +107,18 @@ __global__ __launch_bounds__(512) void kron_kmm4x6_kernel(const StepArgs a, cons
 #pragma unroll
     for (int r = 0; r < 64; r++) x[r] = in[(uint64_t)k6RegRowA(r) * ldi];
   }
-  if (K6_YPOS == 0) loadY();
+  loadY();
   {
     // register stride 1 = digit 2, stride 4 = digit 0, stride 16 = digit 1
     const float fA[3][4] = {{fa[2][0], fa[2][1], fa[2][2], fa[2][3]}, {fa[0][0], fa[0][1], fa[0][2], fa[0][3]},
                             {fa[1][0], fa[1][1], fa[1][2], fa[1][3]}};
     k6Contract3(x, fA);                     // registers: (q4,q5,q6) in the same arrangement
   }
-  // Y: requested here, behind the arrival of X, for the rows this lane stores (phase B arrangement)
-  __builtin_amdgcn_sched_barrier(0);
-  if (K6_YPOS == 1) loadY();
   __builtin_amdgcn_sched_barrier(0);
   float* col = lds + m8 * kK6MStride + k6Spread(m8);
 #pragma unroll
   for (int r = 0; r < 64; r++) col[coord * 65 + k6RegRowA(r)] = x[r];
   __syncthreads();
-  if (K6_YPOS == 2) { loadY(); __builtin_amdgcn_sched_barrier(0); }
 #pragma unroll
   for (int r = 0; r < 64; r++) x[r] = col[r * 65 + coord];  // registers: row bits 6-11 = (k1,k2,k3), k3 fastest
   {
