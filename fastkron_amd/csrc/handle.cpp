@@ -517,6 +517,16 @@ bool Handle::mergeSmallFactors(const KronProblem& p, KronProblem* out, const Cal
   // 16x16 ones; chains of 2x2 and 4x4 factors alone run faster as 16x16 products (a quarter of the multiplications,
   // and the wave-per-block kernel for three 16x16 factors: dgemkm 1024x4^8 0.57 -> 0.47 ms, 1024x4^6 60 -> 20 us).
   uint32_t target = 16;
+  // fp64 rows of five 8x8 factors have a whole-row kernel of their own (one launch, one pass, an eighth of the
+  // multiplications of 64x64 products): the chain stays as it is where that kernel is the online choice
+  if (p.dt == DType::F64 && p.mm == MMType::MKM && p.N == 5) {
+    bool all8 = true;
+    for (uint32_t i = 0; i < p.N; i++) all8 = all8 && p.P[i] == 8 && p.Q[i] == 8;
+    if (all8) {
+      const Plan whole = db_.selectOnline(p, dev_, true);
+      if (whole.size() == 1 && whole[0].lo == 0 && whole[0].hi == 4) return false;
+    }
+  }
   if (p.dt == DType::F64) {
     for (uint32_t i = 0; i < p.N; i++)
       if (p.P[i] == p.Q[i] && (p.P[i] == 8 || p.P[i] == 32)) target = 64;

@@ -162,6 +162,22 @@ static bool row8CanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, u
 static hipError_t row8Launch(const KernelInfo& k, const StepArgs& a, hipStream_t s) { return launchRow8x5(a, s, (int)k.variant); }
 static bool row8Check(const KernelInfo&, const StepArgs& a) { return row8x5Supported(a); }
 
+// ---- whole-row kernel for five fused 8x8 fp64 factors ----
+// A row is one workgroup's work for about 25 us and one workgroup fills a CU: below this many rows the merged
+// 64x64 factors on the pair kernel (a wave per 4096-column block) spread the work over more of the device.
+constexpr uint64_t kRow8dMinRows = 128;
+static bool row8dCanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
+                        const DeviceInfo& dev) {
+  if (p.dt != DType::F64 || p.mm != MMType::MKM || hi - lo + 1 != 5 || p.forward) return false;
+  for (uint32_t i = lo; i <= hi; i++) if (p.P[i] != 8 || p.Q[i] != 8) return false;
+  if (p.colsBefore(hi) != 32768) return false;
+  if (first && p.opX == 2) return false;
+  if (dev.rulesOfThumb && (uint64_t)p.M * p.batch < kRow8dMinRows) return false;
+  return dev.ldsPerBlock >= 133120 && k.dt == p.dt;
+}
+static hipError_t row8dLaunch(const KernelInfo&, const StepArgs& a, hipStream_t s) { return launchRow8x5F64(a, s); }
+static bool row8dCheck(const KernelInfo&, const StepArgs& a) { return row8x5F64Supported(a); }
+
 // ---- wave-per-block kernel for two or three fused PxP factors, 9 <= P <= 16 ----
 static bool row16x3CanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
                           const DeviceInfo&) {
@@ -385,6 +401,12 @@ void registerRowKernels(std::vector<KernelInfo>& out) {
     v.variant = schedule; v.tunerOnly = true;
     out.push_back(v);
   }
+
+  KernelInfo k8d{};
+  k8d.name = "mkm_hip_gfx950_512_d_8x8_8x8_5_1x32768_valu_NN_strided_0_3";
+  k8d.dt = DType::F64; k8d.P = 8; k8d.Q = 8; k8d.fused = 5; k8d.tileM = 1; k8d.tileK = 32768; k8d.threads = 512; k8d.variant = 0;
+  k8d.canRun = row8dCanRun; k8d.launch = row8dLaunch; k8d.check = row8dCheck;
+  out.push_back(k8d);
 
   KernelInfo k32{};
   k32.name = "mkm_hip_gfx950_512_f_32x16_32x16_3_1x32768_mfma16x16x4_NN_strided_0_3";

@@ -82,6 +82,10 @@ hipError_t launchRow16x4(const StepArgs& a, hipStream_t stream, bool staggered =
 bool row16x4W8Supported(const StepArgs& a);
 hipError_t launchRow16x4W8(const StepArgs& a, hipStream_t stream);
 
+// Five fused 8x8 fp64 factors on rows of exactly 8^5 columns, one workgroup per row and CU, on the vector ALU.
+bool row8x5F64Supported(const StepArgs& a);
+hipError_t launchRow8x5F64(const StepArgs& a, hipStream_t stream);
+
 // Five fused 8x8 fp32 factors on rows of exactly 8^5 columns, one workgroup per row, two per CU.
 bool row8x5Supported(const StepArgs& a);
 hipError_t launchRow8x5(const StepArgs& a, hipStream_t stream, int schedule = 0);

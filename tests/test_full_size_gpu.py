@@ -31,6 +31,7 @@ FULL = [
     ("c3", ko.MKM, 256, [64] * 3, [64] * 3, np.float64, 1.0, 0.0, 1),
     ("c4", ko.KMM, 2048, [4] * 6, [4] * 6, np.float32, 1.5, 0.5, 1),
     ("c5", ko.MKM, 512, [32] * 3, [16] * 3, np.float32, 1.0, 1.0, 8),
+    ("dgemkm 1024 x 8^5 (fp64 row kernel)", ko.MKM, 1024, [8] * 5, [8] * 5, np.float64, 1.5, 0.5, 1),
     # sizes at which three more kernels stream their results (system-scope 16-byte stores)
     ("16x16^3 on 8192 rows", ko.MKM, 8192, [16] * 3, [16] * 3, np.float32, 1.5, 0.5, 1),
     ("32x32^3 on 2048 rows", ko.MKM, 2048, [32] * 3, [32] * 3, np.float32, 1.0, 0.0, 1),
