@@ -163,9 +163,10 @@ static hipError_t row8Launch(const KernelInfo& k, const StepArgs& a, hipStream_t
 static bool row8Check(const KernelInfo&, const StepArgs& a) { return row8x5Supported(a); }
 
 // ---- whole-row kernel for five fused 8x8 fp64 factors ----
-// A row is one workgroup's work for about 25 us and one workgroup fills a CU: below this many rows the merged
-// 64x64 factors on the pair kernel (a wave per 4096-column block) spread the work over more of the device.
-constexpr uint64_t kRow8dMinRows = 128;
+// A row is one workgroup's work for about 25 us whatever the number of rows (one workgroup fills a CU); tuned against
+// the merged 64x64 products on kernels that spread a row over many CUs it still wins at 32 rows (26.7 us), the
+// smallest count measured.
+constexpr uint64_t kRow8dMinRows = 32;
 static bool row8dCanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
                         const DeviceInfo& dev) {
   if (p.dt != DType::F64 || p.mm != MMType::MKM || hi - lo + 1 != 5 || p.forward) return false;

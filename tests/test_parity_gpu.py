@@ -255,22 +255,22 @@ ROW_8X5_F64 = "mkm_hip_gfx950_512_d_8x8_8x8_5_1x32768_valu_NN_strided_0_3"
 
 def test_whole_row_kernel_for_five_8x8_fp64_factors(fk):
     """8x8^5 fp64 rows run as ONE launch of the register-resident row kernel (vector-ALU FMAs with the factor in scalar
-    registers) from 128 rows on; below that the chain is merged into 64x64 products as before."""
+    registers) from 32 rows on; below that the chain is merged into 64x64 products as before."""
     check(fk, ko.MKM, 130, [8] * 5, [8] * 5, np.float64, alpha=1.0, beta=0.0, seed=41)
     assert [k for _, _, k in fk.last_plan()] == [ROW_8X5_F64], fk.last_plan()
     check(fk, ko.MKM, 128, [8] * 5, [8] * 5, np.float64, alpha=-1.5, beta=0.75, seed=42)
     assert [k for _, _, k in fk.last_plan()] == [ROW_8X5_F64], fk.last_plan()
     check(fk, ko.MKM, 128, [8] * 5, [8] * 5, np.float64, alpha=2.0, beta=1.0, seed=43, opFs=ko.OP_T)      # factors stored the other way round
     assert [k for _, _, k in fk.last_plan()] == [ROW_8X5_F64], fk.last_plan()
-    check(fk, ko.MKM, 48, [8] * 5, [8] * 5, np.float64, alpha=2.0, beta=1.0, seed=44, batch=3)            # factors per batch entry
+    check(fk, ko.MKM, 11, [8] * 5, [8] * 5, np.float64, alpha=2.0, beta=1.0, seed=44, batch=3)            # factors per batch entry
     assert [k for _, _, k in fk.last_plan()] == [ROW_8X5_F64], fk.last_plan()
-    check(fk, ko.MKM, 64, [8] * 5, [8] * 5, np.float64, alpha=1.0, beta=0.5, seed=45, batch=2, share_f=True, share_y=True)
+    check(fk, ko.MKM, 33, [8] * 5, [8] * 5, np.float64, alpha=1.0, beta=0.5, seed=45, batch=2, share_f=True, share_y=True)
     assert [k for _, _, k in fk.last_plan()] == [ROW_8X5_F64], fk.last_plan()
     check(fk, ko.MKM, 128, [8] * 5, [8] * 5, np.float64, alpha=1.0, beta=0.0, seed=46, integer=True)
     check(fk, ko.MKM, 128, [8] * 5, [8] * 5, np.float64, alpha=1.0, beta=0.0, seed=47, use_temp2=False)
     check(fk, ko.MKM, 129, [8] * 5, [8] * 5, np.float64, alpha=0.5, beta=-1.0, seed=48, opX=ko.OP_T)      # X copied transposed first
     assert fk.last_plan()[-1][2] == ROW_8X5_F64, fk.last_plan()
-    check(fk, ko.MKM, 127, [8] * 5, [8] * 5, np.float64, alpha=1.0, beta=1.0, seed=49)
+    check(fk, ko.MKM, 31, [8] * 5, [8] * 5, np.float64, alpha=1.0, beta=1.0, seed=49)
     assert ROW_8X5_F64 not in [k for _, _, k in fk.last_plan()], fk.last_plan()
 
 
@@ -745,7 +745,7 @@ def test_two_phase_4x4_kernel_on_column_counts_it_is_not_chosen_for(tmp_path):
     (ko.MKM, 3, [4] * 7, np.float32, None),       # same, but 12 virtual rows are no whole block: shorter launches
     (ko.MKM, 5, [2, 4, 2, 4, 8, 2], np.float32, None),
     (ko.MKM, 8, [4] * 6, np.float64, 1),          # -> 16x16^3: chains of 2x2 / 4x4 alone become 16x16 in fp64 too
-    (ko.MKM, 64, [8] * 5, np.float64, None),      # -> 8, 64x64^2 (8x8 factors: 64x64 products; from 128 rows on 8x8^5 has a row kernel)
+    (ko.MKM, 24, [8] * 5, np.float64, None),      # -> 8, 64x64^2 (8x8 factors: 64x64 products; from 32 rows on 8x8^5 has a row kernel)
     (ko.MKM, 2048, [8] * 4, np.float64, 1),       # -> 64x64^2: one launch of the pair kernel
     (ko.MKM, 3, [2] * 9, np.float64, None),       # -> 2, 16, 16
     (ko.MKM, 16, [2] * 9, np.float64, 2),         # the same with whole blocks of rows: two 16x16 in one launch + the 2x2

@@ -113,6 +113,24 @@ def test_two_part_plan_reads_leading_factors_with_stride_zero(planner):
     assert e == capi.SUCCESS and int(launches[-1]["batch"]) == 16 and launches[-1]["f_batch"] == [0]
 
 
+def test_fp64_rows_of_five_8x8_factors_get_the_whole_row_kernel(online_planner):
+    """dgemkm 8x8^5 from 32 rows on: one launch of the fp64 row kernel on the chain as given (no 64x64 products); with
+    fewer rows, with a sixth factor or in the KMM layout the chain is merged as before."""
+    row = "mkm_hip_gfx950_512_d_8x8_8x8_5_1x32768_valu_NN_strided_0_3"
+    for M, opF in [(1024, capi.OP_N), (32, capi.OP_T)]:
+        e, names, launches = plan(online_planner, "mkm", "d", M, [8] * 5, [8] * 5, opF=opF, beta=0.5, with_y=True)
+        assert e == capi.SUCCESS and names == [row], names
+    e, names, _ = plan(online_planner, "mkm", "d", 31, [8] * 5, [8] * 5)
+    assert e == capi.SUCCESS and row not in names and any("64x64" in n for n in names), names
+    e, names, _ = plan(online_planner, "mkm", "d", 1024, [8] * 6, [8] * 6)
+    assert e == capi.SUCCESS and row not in names, names
+    e, names, _ = plan(online_planner, "kmm", "d", 1024, [8] * 5, [8] * 5)
+    assert e == capi.SUCCESS and row not in names, names
+    # per-batch factors: every batch entry reads its own five factors
+    e, names, launches = plan(online_planner, "mkm", "d", 16, [8] * 5, [8] * 5, batch=4)
+    assert e == capi.SUCCESS and names == [row] and launches[0]["f_batch"] == [64] * 5, (names, launches)
+
+
 # ---- kernels with 16-byte global accesses are only chosen for buffers that allow them ----
 VECTOR_CASES = [
     # (label, mm, dt, M, Ps, Qs, batch, beta, substring of the kernel expected on aligned buffers)
