@@ -603,15 +603,22 @@ bool Handle::buildSplit(const KronProblem& p, uint32_t g, void* temp1, void* tem
   if (p.mm != MMType::MKM || p.forward || p.opX != fastKronOp_N) return false;
   if (!temp1 || !temp2 || p.N < 3 || g == 0 || g >= p.N) return false;
   const uint32_t nT = p.N - g;
-  for (uint32_t i = 0; i < p.N; i++) if (p.P[i] != p.Q[i]) return false;            // square: K and L agree throughout
-  uint64_t KA = 1, T = 1;
-  for (uint32_t i = 0; i < g; i++) KA *= p.P[i];
-  for (uint32_t i = g; i < p.N; i++) T *= p.P[i];
-  const uint64_t K = KA * T;
-  if (T >= (1ull << 32)) return false;
+  // KA x Tin columns come in; the trailing factors make Tout of every Tin, the leading ones LA of the KA blocks
+  uint64_t KA = 1, LA = 1, Tin = 1, Tout = 1;
+  for (uint32_t i = 0; i < g; i++) { KA *= p.P[i]; LA *= p.Q[i]; }
+  for (uint32_t i = g; i < p.N; i++) { Tin *= p.P[i]; Tout *= p.Q[i]; }
+  const uint64_t K = KA * Tin, L = LA * Tout, mid = KA * Tout;
+  if (Tin >= (1ull << 32) || Tout >= (1ull << 32)) return false;
+  {
+    // the intermediate (M x KA x Tout) is one of the step outputs the temporaries are sized for; the second part uses
+    // temp2 for the outputs of all but its last launch, each at most as wide as the widest step of the call
+    size_t yElems = 0, tmpElems = 0;
+    if (const_cast<Handle*>(this)->sizes(p.M, p.N, p.P, p.Q, &yElems, &tmpElems) != fastKronSuccess) return false;
+    if ((uint64_t)p.M * mid > tmpElems) return false;
+  }
   if (p.batch > 1) {
-    if (p.strideX != (uint64_t)p.M * K || p.strideZ != (uint64_t)p.M * K) return false;
-    if (p.Y && p.beta != 0.0 && p.strideY != (uint64_t)p.M * K) return false;
+    if (p.strideX != (uint64_t)p.M * K || p.strideZ != (uint64_t)p.M * L) return false;
+    if (p.Y && p.beta != 0.0 && p.strideY != (uint64_t)p.M * L) return false;
   }
   // the leading factors are read by a problem whose batch entries are the rows of this one: shared factors only
   for (uint32_t i = 0; i < g; i++) if (p.strideF[i] != 0) return false;
@@ -623,18 +630,18 @@ bool Handle::buildSplit(const KronProblem& p, uint32_t g, void* temp1, void* tem
   for (uint32_t i = 0; i < nT; i++) {
     q1.P[i] = p.P[g + i]; q1.Q[i] = p.Q[g + i]; q1.F[i] = p.F[g + i]; q1.strideF[i] = p.strideF[g + i];
   }
-  q1.Z = temp1; q1.strideZ = (uint64_t)p.M * K;
+  q1.Z = temp1; q1.strideZ = (uint64_t)p.M * mid;
   q1.Y = nullptr; q1.strideY = 0; q1.alpha = 1.0; q1.beta = 0.0;
   q1.zReadNext = true;
 
   // part 2: leading factors as a KMM over every row block; P x Q storage is the transpose of KMM's Q x P
   KronProblem q2 = p;
-  q2.mm = MMType::KMM; q2.M = (uint32_t)T; q2.N = g;
+  q2.mm = MMType::KMM; q2.M = (uint32_t)Tout; q2.N = g;
   q2.opF = (p.opF == fastKronOp_N) ? fastKronOp_T : fastKronOp_N;
   q2.opX = fastKronOp_N;
-  q2.X = temp1; q2.strideX = K;
+  q2.X = temp1; q2.strideX = mid;
   q2.xJustWritten = true;
-  q2.strideZ = K; q2.strideY = K;
+  q2.strideZ = L; q2.strideY = L;
   q2.batch = p.batch * p.M; q2.strided = true;
   for (uint32_t i = 0; i < g; i++) q2.strideF[i] = 0;
   *q1out = q1; *q2out = q2;
@@ -701,7 +708,7 @@ fastKronError Handle::runSplit(const KronProblem& p, uint32_t g, const KronProbl
 // chunk's intermediate.
 uint32_t Handle::chunkRowsForCache(const KronProblem& p, const KronProblem& q2) const {
   const long forcedMB = chunkMB_;
-  if (forcedMB <= 0 || p.batch != 1 || p.M < 2 || p.forward) return p.M;
+  if (forcedMB <= 0 || p.batch != 1 || p.M < 2 || p.forward || p.K() != p.L()) return p.M;
   const uint64_t rowBytes = q2.strideX * dtypeSize(p.dt);
   uint64_t rows = ((uint64_t)forcedMB << 20) / rowBytes;
   if (rows < 1) rows = 1;
@@ -715,8 +722,19 @@ fastKronError Handle::trySplitLeadingTrailing(const KronProblem& p, void* temp1,
   // trailing run of identical square factors that one whole-row kernel fuses:
   // fp32 8x8 (five), 16x16 (four), 32x32 (three), 64x64 (two); fp64 16x16 (three), 32x32 or 64x64 (two);
   // 9x9 ... 15x15 (three, either type)
-  const uint32_t tp = p.P[p.N - 1];
-  if (p.Q[p.N - 1] != tp) return fastKronKernelNotFound;
+  const uint32_t tp = p.P[p.N - 1], tq = p.Q[p.N - 1];
+  if (tq != tp) {
+    // two trailing rectangular factors of a shape the pair kernel has exact tiles for (32x64, 64x32)
+    if (p.P[p.N - 2] != tp || p.Q[p.N - 2] != tq) return fastKronKernelNotFound;
+    const uint32_t g2 = p.N - 2;
+    KronProblem r1, r2;
+    if (!buildSplit(p, g2, temp1, temp2, &r1, &r2)) return fastKronKernelNotFound;
+    Plan rp1 = db_.selectOnline(r1, dev_, true);
+    if (rp1.size() != 1 || db_.kernels()[rp1[0].kernel].fused != 2 || db_.kernels()[rp1[0].kernel].P == 0)
+      return fastKronKernelNotFound;
+    Plan rp2 = db_.selectOnline(r2, dev_, true);
+    return runSplit(p, g2, r1, rp1, r2, rp2, temp2);
+  }
   uint32_t maxT = 0;
   if (tp == 32 && p.dt == DType::F32) maxT = 3;      // three 32x32 fp32 factors fused per 32768-column block
   else if (tp == 32 || tp == 64)      maxT = 2;

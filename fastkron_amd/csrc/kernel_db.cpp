@@ -258,6 +258,12 @@ static bool stepF64Check(const KernelInfo& k, const StepArgs& a) { return stepMf
 static bool pairCanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
                        const DeviceInfo& dev) {
   if (p.dt != k.dt || p.mm != MMType::MKM || hi - lo + 1 != 2 || p.forward) return false;
+  if (k.P != k.Q) {
+    // two rectangular factors of exactly the kernel's shape (32x64, 64x32): rows of P*P elements become Q*Q
+    for (uint32_t i = lo; i <= hi; i++) if (p.P[i] != k.P || p.Q[i] != k.Q) return false;
+    if (p.colsBefore(hi) != (uint64_t)k.P * k.P) return false;
+    return !(first && p.opX == 2) && dev.ldsPerBlock >= (int)(2 * k.P * k.Q * 8);
+  }
   // the 32x32 kernel also takes factors of 17x17 ... 31x31, zero-padded to its tile
   const uint32_t P = p.P[hi];
   if (!(P == k.P || (k.P == 32 && P >= 17 && P < 32))) return false;
@@ -481,6 +487,20 @@ void registerRowKernels(std::vector<KernelInfo>& out) {
               ps + "x" + ps + "_2_1x" + std::to_string(P * P) + (f64 && P == 64 ? "_mfma4x4x4" : "_mfma16x16x4") +
               "_NN_strided_0_3";
     kp.dt = dt; kp.P = P; kp.Q = P; kp.fused = 2; kp.tileM = 1; kp.tileK = P * P; kp.threads = (f64 && P == 64) ? 512 : 256;
+    kp.variant = 0;
+    kp.canRun = pairCanRun; kp.launch = pairLaunch; kp.check = pairCheck;
+    out.push_back(kp);
+  }
+
+  // rectangular pairs on exact tiles (fp64 only 32x64: see pair_mfma.hip)
+  for (DType dt : {DType::F32, DType::F64})
+  for (auto pq : {std::pair<uint32_t, uint32_t>{32, 64}, {64, 32}}) {
+    if (dt == DType::F64 && pq.first == 64) continue;
+    KernelInfo kp{};
+    const std::string ps = std::to_string(pq.first) + "x" + std::to_string(pq.second);
+    kp.name = std::string("mkm_hip_gfx950_256") + (dt == DType::F64 ? "_d_" : "_f_") + ps + "_" + ps + "_2_1x" +
+              std::to_string(pq.first * pq.first) + "_mfma16x16x4_NN_strided_0_3";
+    kp.dt = dt; kp.P = pq.first; kp.Q = pq.second; kp.fused = 2; kp.tileM = 1; kp.tileK = pq.first * pq.first; kp.threads = 256;
     kp.variant = 0;
     kp.canRun = pairCanRun; kp.launch = pairLaunch; kp.check = pairCheck;
     out.push_back(kp);

@@ -69,17 +69,21 @@ template <> struct PairMfma<float> {
 // EXACT = false: factors of R x R with 16 < R < P, operands zero-padded to the P x P tile: a row is R*R contiguous
 // elements, loaded and stored element by element with indices >= R masked (what the padded lanes and registers
 // compute is exact zeros and is never stored).
-template <typename T, int P, bool HAS_Y, bool EXACT = true>
+// Q != P: two factors of P x Q each (32 x 64, 64 x 32): the row is a P x P tile, the first product leaves P x Q, the
+// result is a Q x Q tile; exact sizes only.
+template <typename T, int P, bool HAS_Y, bool EXACT = true, int Q = P>
 __global__ __launch_bounds__(256, 2) void kron_pair_kernel(const StepArgs a) {
+  static_assert(EXACT || P == Q, "the zero-padded form is square");
   using MF = PairMfma<T>;
   using Acc = typename MF::Acc;
-  constexpr int PB = P / 16;             // 16-wide blocks per digit
+  constexpr int PB = P / 16;             // 16-wide blocks of an input digit
+  constexpr int QB = Q / 16;             // 16-wide blocks of an output digit
   constexpr int PC = P / 4;              // products per block of product 1, elements per lane and row
   constexpr int VE = 16 / sizeof(T);     // elements per 128-bit load
   typedef T VT __attribute__((ext_vector_type(VE)));
   extern __shared__ double pairLdsRaw[];
-  T* fA = (T*)pairLdsRaw;                // F_a[k_a][q_a], row-major P x P
-  T* fB = fA + P * P;                    // F_b[k_b][q_b]
+  T* fA = (T*)pairLdsRaw;                // F_a[k_a][q_a], row-major P x Q
+  T* fB = fA + P * Q;                    // F_b[k_b][q_b]
   const int tid = threadIdx.x;
   const int l0 = tid & 63;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -91,22 +95,23 @@ __global__ __launch_bounds__(256, 2) void kron_pair_kernel(const StepArgs a) {
   // multiplying by 1 is exact: launches that do not write Z need no branch around the scaling
   const T alpha = a.epilogue ? (T)a.alpha : (T)1, beta = (T)a.beta;
   const int R = EXACT ? P : (int)a.p[0];            // the factors' real size; the row is R * R elements
+  const int RO = EXACT ? Q : R;                     // pitch of the result tile
 
   {
     const T* Fa = (const T*)a.f[0] + (size_t)bt * a.f_batch[0];
     const T* Fb = (const T*)a.f[1] + (size_t)bt * a.f_batch[1];
     // all loads of a thread go out before the first LDS write waits for one (a loop of load, wait, write puts one
     // memory round trip per iteration in front of the first product)
-    T va[P * P / 256], vb[P * P / 256];
+    T va[P * Q / 256], vb[P * Q / 256];
 #pragma unroll
-    for (int k = 0; k < P * P / 256; k++) {
-      const int i = tid + 256 * k, p = i / P, q = i % P;
+    for (int k = 0; k < P * Q / 256; k++) {
+      const int i = tid + 256 * k, p = i / Q, q = i % Q;
       const bool in = EXACT || (p < R && q < R);
       va[k] = in ? Fa[(int64_t)p * a.f_sp[0] + (int64_t)q * a.f_sq[0]] : (T)0;
       vb[k] = in ? Fb[(int64_t)p * a.f_sp[1] + (int64_t)q * a.f_sq[1]] : (T)0;
     }
 #pragma unroll
-    for (int k = 0; k < P * P / 256; k++) { fA[tid + 256 * k] = va[k]; fB[tid + 256 * k] = vb[k]; }
+    for (int k = 0; k < P * Q / 256; k++) { fA[tid + 256 * k] = va[k]; fB[tid + 256 * k] = vb[k]; }
   }
   __syncthreads();
 
@@ -142,7 +147,7 @@ __global__ __launch_bounds__(256, 2) void kron_pair_kernel(const StepArgs a) {
     const T* Y = HAS_Y ? YB + (size_t)row * a.y_ldm : nullptr;
 
 #pragma unroll 1
-    for (int jb = 0; jb < PB; jb++) {
+    for (int jb = 0; jb < QB; jb++) {
       int ofs = 16 * jb + lo;
       asm volatile("" : "+v"(ofs));
       Acc d1[PB];
@@ -150,14 +155,14 @@ __global__ __launch_bounds__(256, 2) void kron_pair_kernel(const StepArgs a) {
       for (int g = 0; g < PB; g++) d1[g] = (Acc){0, 0, 0, 0};
 #pragma unroll
       for (int c = 0; c < PC; c++) {
-        const T b = fA[(PC * hi + c) * P + ofs];
+        const T b = fA[(PC * hi + c) * Q + ofs];
 #pragma unroll
         for (int g = 0; g < PB; g++) d1[g] = MF::mma(x[g][c], b, d1[g]);
       }
       // register r of d1[g] holds the rows k_b = 16g + row(r, hi): the B operand of product 2 for them;
       // two independent accumulator chains at a time
 #pragma unroll
-      for (int jb2 = 0; jb2 < PB; jb2 += 2) {
+      for (int jb2 = 0; jb2 < QB; jb2 += 2) {
         Acc acc[2] = {(Acc){0, 0, 0, 0}, (Acc){0, 0, 0, 0}};
 #pragma unroll
         for (int g = 0; g < PB; g++)
@@ -165,7 +170,7 @@ __global__ __launch_bounds__(256, 2) void kron_pair_kernel(const StepArgs a) {
           for (int r = 0; r < 4; r++)
 #pragma unroll
             for (int u = 0; u < 2; u++) {
-              const T fa = fB[(16 * g + MF::row(r, hi)) * P + 16 * (jb2 + u) + lo];
+              const T fa = fB[(16 * g + MF::row(r, hi)) * Q + 16 * (jb2 + u) + lo];
               acc[u] = MF::mma(fa, d1[g][r], acc[u]);
             }
         T yv[2][4];
@@ -175,7 +180,7 @@ __global__ __launch_bounds__(256, 2) void kron_pair_kernel(const StepArgs a) {
 #pragma unroll
             for (int r = 0; r < 4; r++)
               yv[u][r] = (EXACT || (16 * (jb2 + u) + MF::row(r, hi) < R && ofs < R))
-                             ? Y[(16 * (jb2 + u) + MF::row(r, hi)) * R + ofs] : (T)0;
+                             ? Y[(16 * (jb2 + u) + MF::row(r, hi)) * RO + ofs] : (T)0;
         }
 #pragma unroll
         for (int u = 0; u < 2; u++)
@@ -184,7 +189,7 @@ __global__ __launch_bounds__(256, 2) void kron_pair_kernel(const StepArgs a) {
             T v = acc[u][r] * alpha;
             if (HAS_Y) v += beta * yv[u][r];
             if (EXACT || (16 * (jb2 + u) + MF::row(r, hi) < R && ofs < R))
-              out[(16 * (jb2 + u) + MF::row(r, hi)) * R + ofs] = v;
+              out[(16 * (jb2 + u) + MF::row(r, hi)) * RO + ofs] = v;
           }
       }
     }
@@ -396,27 +401,36 @@ __global__ __launch_bounds__(512, 2) void kron_pair64_f64_kernel(const StepArgs 
   for (row += stride; row < a.M; row += stride) computeRow(row, nextOf(row));
 }
 
+// Rectangular pairs with exact tiles: 32x64 and 64x32 in fp32, 32x64 in fp64 (a 64 x 64 tile of doubles, twice over
+// for the row in flight, would not leave this kernel's waves enough registers).
+static bool pairRectShape(uint32_t P, uint32_t Q, DType dt) {
+  return (P == 32 && Q == 64) || (P == 64 && Q == 32 && dt == DType::F32);
+}
+
 bool pairMfmaSupported(const StepArgs& a, DType dt) {
   if (a.nf != 2) return false;
-  const uint32_t P = a.p[0];
-  if ((P != 64 && (P < 17 || P > 32)) || a.q[0] != P || a.p[1] != P || a.q[1] != P) return false;
-  if (a.Kin != (uint64_t)P * P || a.Kout != a.Kin) return false;
+  const uint32_t P = a.p[0], Q = a.q[0];
+  if (a.p[1] != P || a.q[1] != Q) return false;
+  if (P != Q) {
+    if (!pairRectShape(P, Q, dt)) return false;
+  } else if (P != 64 && (P < 17 || P > 32)) return false;
+  if (a.Kin != (uint64_t)P * P || a.Kout != (uint64_t)Q * Q) return false;
   if (a.in_ldc != 1 || a.out_ldc != 1 || (a.y && a.y_ldc != 1)) return false;
   if (P < 32) return a.batch <= 65535;                                                // padded form: element-wise accesses
   const uint64_t vmask = 16 / dtypeSize(dt) - 1;                                      // 128-bit loads
   if (((uintptr_t)a.in & 15) || ((uint64_t)a.in_ldm & vmask) || (a.in_batch & vmask)) return false;
-  if (dt == DType::F64 && P == 64) {                                                  // and 128-bit stores / Y loads
+  if (dt == DType::F64 && P == 64 && Q == 64) {                                       // and 128-bit stores / Y loads
     if (((uintptr_t)a.out & 15) || ((uint64_t)a.out_ldm & 1) || (a.out_batch & 1)) return false;
     if (a.y && (((uintptr_t)a.y & 15) || ((uint64_t)a.y_ldm & 1) || (a.y_batch & 1))) return false;
   }
   return a.batch <= 65535;
 }
 
-template <typename T, int P, bool EXACT = true>
+template <typename T, int P, bool EXACT = true, int Q = P>
 static hipError_t launchPairT(const StepArgs& a, hipStream_t stream) {
   const int cus = deviceCUs();
-  const size_t ldsBytes = 2 * P * P * sizeof(T);
-  uint32_t wgs = (uint32_t)cus * (P == 32 ? 4 : 2);   // persistent; the 32x32 kernels need few registers
+  const size_t ldsBytes = 2 * P * Q * sizeof(T);
+  uint32_t wgs = (uint32_t)cus * (P == 32 && Q == 32 ? 4 : 2);   // persistent; the 32x32 kernels need few registers
   if (a.batch > 1) wgs = (wgs + a.batch - 1) / a.batch;
   const uint32_t need = (a.M + kPairWaves - 1) / kPairWaves;
   if (wgs > need) wgs = need;
@@ -426,15 +440,15 @@ static hipError_t launchPairT(const StepArgs& a, hipStream_t stream) {
   const int devIdx = launchDeviceIndex();
   const bool y = a.y && a.epilogue;
   if (!attrOnce[y].done(devIdx)) {
-    hipError_t e = y ? hipFuncSetAttribute((const void*)kron_pair_kernel<T, P, true, EXACT>,
+    hipError_t e = y ? hipFuncSetAttribute((const void*)kron_pair_kernel<T, P, true, EXACT, Q>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes)
-                     : hipFuncSetAttribute((const void*)kron_pair_kernel<T, P, false, EXACT>,
+                     : hipFuncSetAttribute((const void*)kron_pair_kernel<T, P, false, EXACT, Q>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes);
     if (e != hipSuccess) return e;
     attrOnce[y].mark(devIdx);
   }
-  if (y) hipLaunchKernelGGL((kron_pair_kernel<T, P, true, EXACT>), grid, block, ldsBytes, stream, a);
-  else   hipLaunchKernelGGL((kron_pair_kernel<T, P, false, EXACT>), grid, block, ldsBytes, stream, a);
+  if (y) hipLaunchKernelGGL((kron_pair_kernel<T, P, true, EXACT, Q>), grid, block, ldsBytes, stream, a);
+  else   hipLaunchKernelGGL((kron_pair_kernel<T, P, false, EXACT, Q>), grid, block, ldsBytes, stream, a);
   return hipGetLastError();
 }
 
@@ -467,6 +481,10 @@ static hipError_t launchPair64(const StepArgs& a, hipStream_t stream) {
 
 hipError_t launchPairMfma(const StepArgs& a, DType dt, hipStream_t stream) {
   if (!pairMfmaSupported(a, dt)) return hipErrorInvalidValue;
+  if (a.p[0] != a.q[0]) {
+    if (dt == DType::F64) return launchPairT<double, 32, true, 64>(a, stream);
+    return a.p[0] == 32 ? launchPairT<float, 32, true, 64>(a, stream) : launchPairT<float, 64, true, 32>(a, stream);
+  }
   if (a.p[0] < 32) return dt == DType::F64 ? launchPairT<double, 32, false>(a, stream) : launchPairT<float, 32, false>(a, stream);
   if (dt == DType::F64) return a.p[0] == 64 ? launchPair64(a, stream) : launchPairT<double, 32>(a, stream);
   return a.p[0] == 64 ? launchPairT<float, 64>(a, stream) : launchPairT<float, 32>(a, stream);

@@ -274,6 +274,41 @@ def test_whole_row_kernel_for_five_8x8_fp64_factors(fk):
     assert ROW_8X5_F64 not in [k for _, _, k in fk.last_plan()], fk.last_plan()
 
 
+RECT_PAIRS = [
+    # P, Q, dtype: the shapes the pair kernel has exact rectangular tiles for
+    (32, 64, np.float32), (64, 32, np.float32), (32, 64, np.float64),
+]
+
+
+@pytest.mark.parametrize("P,Q,dt", RECT_PAIRS)
+def test_pair_kernel_for_two_rectangular_factors(fk, P, Q, dt):
+    """Two factors of 32x64 / 64x32 (reference tests/src/general-tests-NN.cpp:94-100 runs 32x64 chains): one launch of
+    the pair kernel on exact tiles (a P x P row in, a Q x Q row out), and for three factors the two-part plan with the
+    pair on the blocks of a row and the leading factor across them."""
+    t = "d" if dt == np.float64 else "f"
+    name = f"mkm_hip_gfx950_256_{t}_{P}x{Q}_{P}x{Q}_2_1x{P * P}_mfma16x16x4_NN_strided_0_3"
+    check(fk, ko.MKM, 37, [P] * 2, [Q] * 2, dt, alpha=1.0, beta=0.0, seed=61)
+    assert [k for _, _, k in fk.last_plan()] == [name], fk.last_plan()
+    check(fk, ko.MKM, 5, [P] * 2, [Q] * 2, dt, alpha=-1.5, beta=0.75, seed=62)
+    check(fk, ko.MKM, 9, [P] * 2, [Q] * 2, dt, alpha=2.0, beta=1.0, seed=63, opFs=ko.OP_T)
+    check(fk, ko.MKM, 6, [P] * 2, [Q] * 2, dt, alpha=1.0, beta=1.0, seed=64, batch=3)
+    check(fk, ko.MKM, 6, [P] * 2, [Q] * 2, dt, alpha=1.0, beta=0.5, seed=65, batch=2, share_f=True, share_y=True)
+    check(fk, ko.MKM, 4, [P] * 2, [Q] * 2, dt, alpha=1.0, beta=0.0, seed=66, integer=True)
+    if P <= Q:
+        check(fk, ko.MKM, 7, [P] * 2, [Q] * 2, dt, alpha=1.5, beta=0.5, seed=67, y_is_z=True)
+    # three factors: the pair runs on the M * P blocks of P*P columns, the leading factor across the blocks
+    check(fk, ko.MKM, 3, [P] * 3, [Q] * 3, dt, alpha=1.5, beta=0.5, seed=68)
+    plan = fk.last_plan()
+    assert len(plan) == 2 and plan[0][2] == name and plan[0][:2] == (1, 2), plan
+    check(fk, ko.MKM, 3, [P] * 3, [Q] * 3, dt, alpha=1.0, beta=1.0, seed=69, batch=2, share_f=True)    # reference: batched, X shared
+    assert len(fk.last_plan()) == 2, fk.last_plan()
+    check(fk, ko.MKM, 3, [P] * 3, [Q] * 3, dt, alpha=1.0, beta=1.0, seed=70, batch=2)                  # factors per batch entry: no two-part plan
+    check(fk, ko.MKM, 2, [16, P, P], [8, Q, Q], dt, alpha=1.0, beta=0.0, seed=71)                      # another leading factor
+    assert fk.last_plan()[0][2] == name, fk.last_plan()
+    if P <= Q:        # (with shrinking factors Z is smaller than the temporary, and the second temporary is mandatory)
+        check(fk, ko.MKM, 2, [P] * 3, [Q] * 3, dt, alpha=1.0, beta=0.0, seed=72, use_temp2=False)      # one temporary: no two-part plan
+
+
 def test_whole_row_kernel_for_three_32x16_factors(fk):
     """32x16^3 fp32 rows (non-square, which the reference never fuses) run as ONE launch."""
     check(fk, ko.MKM, 5, [32] * 3, [16] * 3, np.float32, alpha=1.0, beta=0.0, seed=31)

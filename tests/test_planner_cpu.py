@@ -131,6 +131,26 @@ def test_fp64_rows_of_five_8x8_factors_get_the_whole_row_kernel(online_planner):
     assert e == capi.SUCCESS and names == [row] and launches[0]["f_batch"] == [64] * 5, (names, launches)
 
 
+def test_rectangular_pairs_get_the_pair_kernel_and_the_two_part_plan(online_planner):
+    """Two 32x64 / 64x32 factors: one launch on exact tiles; three: the pair on the blocks of a row (M * P virtual rows of
+    P*P columns, Q*Q out) and the leading factor across the blocks as a KMM problem with one batch entry per row."""
+    for dt, P, Q in [("s", 32, 64), ("s", 64, 32), ("d", 32, 64)]:
+        name = f"mkm_hip_gfx950_256_{'f' if dt == 's' else 'd'}_{P}x{Q}_{P}x{Q}_2_1x{P * P}_mfma16x16x4_NN_strided_0_3"
+        e, names, launches = plan(online_planner, "mkm", dt, 40, [P] * 2, [Q] * 2, beta=0.5, with_y=True)
+        assert e == capi.SUCCESS and names == [name], names
+        e, names, launches = plan(online_planner, "mkm", dt, 3, [P] * 3, [Q] * 3, beta=0.5, with_y=True)
+        assert e == capi.SUCCESS and len(names) == 2 and names[0] == name, names
+        assert int(launches[0]["M"]) == 3 * P and int(launches[0]["out"], 16) == BASE + 3 * GAP, launches      # into temp1
+        assert int(launches[1]["M"]) == Q * Q and int(launches[1]["batch"]) == 3, launches
+        assert int(launches[1]["in"], 16) == BASE + 3 * GAP and int(launches[1]["out"], 16) == BASE + 1 * GAP, launches
+    # fp64 64x32 has no such kernel (a 64 x 64 tile of doubles per row in flight): one launch per factor
+    e, names, _ = plan(online_planner, "mkm", "d", 40, [64] * 2, [32] * 2)
+    assert e == capi.SUCCESS and len(names) == 2 and all("_2_1x" not in n for n in names), names
+    # the leading factors of a two-part plan are shared between the rows: per-batch factors rule it out
+    e, names, _ = plan(online_planner, "mkm", "s", 3, [32] * 3, [64] * 3, batch=2)
+    assert e == capi.SUCCESS and len(names) == 3, names
+
+
 # ---- kernels with 16-byte global accesses are only chosen for buffers that allow them ----
 VECTOR_CASES = [
     # (label, mm, dt, M, Ps, Qs, batch, beta, substring of the kernel expected on aligned buffers)
