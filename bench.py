@@ -300,25 +300,29 @@ def pattern_ceilings(fk, steps, warmup, ev, stream):
 
 def published_shapes(fk, budget_s):
     """The 15 fp32 GeMKM shapes of the reference's published table (documents/performance.md:9-23), plus c1 and c2's
-    shapes with both operands transposed and as sgekmm (the rows nearest to them there: :29-31, :89-91), through the
+    shapes with both operands transposed, as sgekmm (the rows nearest to them there: :29-31, :89-91) and in fp64, through the
     same handle, operands rotated so that the memory-side cache holds none, wall clock around batches of calls with
     a device synchronisation on both sides.  Stops adding shapes once `budget_s` seconds are spent."""
     import torch
     from fastkron_amd.capi import OP_N, OP_T
     from fastkron_amd.tune import _Case
-    todo = [("mkm", M, P, N, OP_N, "NN") for M, P, N in PUBLISHED_GPU_SHAPES]
-    todo += [("mkm", 1024, 8, 5, OP_T, "TT"), ("mkm", 1024, 16, 4, OP_T, "TT"),
-             ("kmm", 1024, 8, 5, OP_N, "NN"), ("kmm", 1024, 16, 4, OP_N, "NN")]
+    # (the four extra fp32 rows and the two fp64 rows come first: they are the ones this leg is for, and the largest of
+    # the 15 table shapes use most of the budget)
+    f32, f64 = torch.float32, torch.float64
+    todo = [("mkm", 1024, 8, 5, OP_T, "TT", f32), ("mkm", 1024, 16, 4, OP_T, "TT", f32),
+            ("kmm", 1024, 8, 5, OP_N, "NN", f32), ("kmm", 1024, 16, 4, OP_N, "NN", f32),
+            ("mkm", 1024, 8, 5, OP_N, "NN", f64), ("mkm", 1024, 16, 4, OP_N, "NN", f64)]     # reference :49-51 (double)
+    todo += [("mkm", M, P, N, OP_N, "NN", f32) for M, P, N in PUBLISHED_GPU_SHAPES]
     out, t_start = {}, time.perf_counter()
-    for mm, M, P, N, op, on in todo:
+    for mm, M, P, N, op, on, dt in todo:
         if time.perf_counter() - t_start > budget_s:
             break
         try:
-            case = _Case(fk, mm, M, [P] * N, [P] * N, torch.float32)
+            case = _Case(fk, mm, M, [P] * N, [P] * N, dt)
         except torch.cuda.OutOfMemoryError:
             continue
         ms = case.time(fk, op, op, runs=10, samples=3)
-        out[f"s{'gemkm' if mm == 'mkm' else 'gekmm'}_{M}_{P}x{P}^{N}_{on}"] = {
+        out[f"{'s' if dt == f32 else 'd'}{'gemkm' if mm == 'mkm' else 'gekmm'}_{M}_{P}x{P}^{N}_{on}"] = {
             "ms": round(ms, 5), "gflops": round(case.gflops(ms), 1), "launches": len(fk.last_plan())}
         del case
         torch.cuda.empty_cache()
