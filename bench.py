@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the Kronecker-matrix multiplication hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c1|c2|c3|c4|c5] [--only] [--tune] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c1|c2|c3|c4|c5|c1d] [--only] [--tune] [--no-cpu]
 
 One "step" is one call of the C-ABI entry point (sgemkm / dgemkm / sgekmm / sgemkmStridedBatched) on a
 synthetic problem whose operands are already resident in HBM.  The default workload is c2, the
@@ -36,6 +36,8 @@ CONFIGS = {
     "c3": ("dgemkm", 256, [64] * 3, [64] * 3, "f64", 1.0, 0.0, 1, "mfma"),
     "c4": ("sgekmm", 2048, [4] * 6, [4] * 6, "f32", 1.5, 0.5, 1, "hbm"),
     "c5": ("sgemkmStridedBatched", 512, [32] * 3, [16] * 3, "f32", 1.0, 1.0, 8, "hbm"),
+    # c1's shape in fp64 (reference documents/performance.md:49, the double GeMKM row of 1024 x 8^5): the fp64 whole-row kernel
+    "c1d": ("dgemkm", 1024, [8] * 5, [8] * 5, "f64", 1.0, 0.0, 1, "hbm"),
 }
 
 
