@@ -37,6 +37,11 @@ typedef double d2 __attribute__((ext_vector_type(2)));
 typedef const double __attribute__((address_space(4))) * FactorPtr;
 
 constexpr int kRow8dLen = 32768;
+// Start groups of the first round of workgroups (measured on dgemkm 1024 / 2048 x 8^5: no stagger 125 / 242 us; three
+// groups 6 us apart 121 / 228, 7 us apart 119 / 232, 8 to 10 us apart 131-135 / 247; two, four, five, six or eight
+// groups at spacings from 2 to 14 us 124-137 / 237-252).
+constexpr uint32_t kRow8dStaggerGroups = 3;
+constexpr uint32_t kRow8dStaggerTicks = 650;      // of the 100 MHz wall clock
 constexpr int kRow8dWaveRegion = 32 * 65;                       // doubles per wave in exchange 2
 constexpr int kRow8dLdsDoubles = 8 * kRow8dWaveRegion;          // 133 120 bytes; exchange 1 needs 131 072
 
@@ -131,12 +136,24 @@ __device__ __forceinline__ void contractSecond(double (&x)[8][8], const Factor8&
 
 // PMAJOR: the factors are stored with q fastest (element (p,q) at 8p + q), otherwise with p fastest (the other op)
 template <bool HAS_Y, int NT, bool PMAJOR>
-__global__ __launch_bounds__(512) void kron_row8x5_f64_kernel(const StepArgs a) {
+__global__ __launch_bounds__(512) void kron_row8x5_f64_kernel(const StepArgs a, const uint32_t firstRound,
+                                                              const uint32_t staggerGroups, const uint32_t staggerTicks) {
   extern __shared__ __align__(16) double ldsd[];
   const int tid = threadIdx.x;
   const int l = tid & 63;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const uint32_t m = blockIdx.x, bt = blockIdx.y;
+  // The workgroups that the device starts together (one per CU) would load, compute and store in lockstep, all of
+  // them waiting for HBM in one phase and none using it in the next: they start in groups, staggerTicks of the 100 MHz
+  // clock apart; later workgroups start whenever a predecessor ends and keep that spread.
+  if (staggerTicks) {
+    const uint32_t idx = blockIdx.x + gridDim.x * blockIdx.y;
+    const uint32_t grp = (idx >> 3) % staggerGroups;              // idx % 8 is the XCD
+    if (idx < firstRound && grp) {
+      const unsigned long long t0 = __builtin_amdgcn_s_memrealtime();
+      while (__builtin_amdgcn_s_memrealtime() - t0 < (unsigned long long)grp * staggerTicks) __builtin_amdgcn_s_sleep(16);
+    }
+  }
 
   const double* X = (const double*)a.in + (size_t)bt * a.in_batch + (size_t)m * kRow8dLen;
   double* Z = (double*)a.out + (size_t)bt * a.out_batch + (size_t)m * kRow8dLen;
@@ -270,7 +287,7 @@ hipError_t launchRow8x5F64(const StepArgs& a, hipStream_t stream) {
   static PerDeviceOnce attrOnce;
   const int devIdx = launchDeviceIndex();
   const size_t ldsBytes = kRow8dLdsDoubles * sizeof(double);
-  using Kernel = void (*)(const StepArgs);
+  using Kernel = void (*)(const StepArgs, const uint32_t, const uint32_t, const uint32_t);
   static const Kernel kernels[2][2][3] = {
       {{kron_row8x5_f64_kernel<false, 0, false>, kron_row8x5_f64_kernel<false, 1, false>, kron_row8x5_f64_kernel<false, 2, false>},
        {kron_row8x5_f64_kernel<true, 0, false>, kron_row8x5_f64_kernel<true, 1, false>, kron_row8x5_f64_kernel<true, 2, false>}},
@@ -286,7 +303,10 @@ hipError_t launchRow8x5F64(const StepArgs& a, hipStream_t stream) {
     attrOnce.mark(devIdx);
   }
   dim3 grid(a.M, a.batch), block(512);
-  hipLaunchKernelGGL(kernels[row8dPMajor(a) ? 1 : 0][(a.y && a.epilogue) ? 1 : 0][streamMode(a)], grid, block, ldsBytes, stream, a);
+  const uint32_t cus = (uint32_t)deviceCUs();
+  const bool stagger = (uint64_t)a.M * a.batch >= 2ull * cus;     // with one row per CU there is nothing to interleave
+  hipLaunchKernelGGL(kernels[row8dPMajor(a) ? 1 : 0][(a.y && a.epilogue) ? 1 : 0][streamMode(a)], grid, block, ldsBytes, stream, a,
+                     cus, kRow8dStaggerGroups, stagger ? kRow8dStaggerTicks : 0u);
   return hipGetLastError();
 }
 
