@@ -533,13 +533,24 @@ bool Handle::mergeSmallFactors(const KronProblem& p, KronProblem* out, const Cal
   }
   // groups of adjacent square power-of-two factors, formed from the last factor towards the first, each as
   // large as fits the target size
+  // fp64 chains of six or seven 8x8 factors: the trailing five stay as they are, for the whole-row kernel on the
+  // blocks of 32768 columns (a two-part plan), and only the leading ones are merged (tuned: dgemkm 1024 x 8^6 1.95 ->
+  // 1.79 ms, 256 x 8^6 0.52 -> 0.45 ms; with eight factors the merged chain takes as many launches and stays)
+  int keepFrom = (int)p.N;
+  if (p.dt == DType::F64 && p.mm == MMType::MKM && (p.N == 6 || p.N == 7) && p.opX == fastKronOp_N && dev_.rulesOfThumb) {
+    bool all8 = true;
+    for (uint32_t i = 0; i < p.N; i++) all8 = all8 && p.P[i] == 8 && p.Q[i] == 8;
+    // (from 32 blocks on, as the kernel's own rule has it)
+    const uint64_t blocks = (uint64_t)p.M * (p.N == 6 ? 8 : 64) * p.batch;
+    if (all8 && blocks >= 32) keepFrom = (int)p.N - 5;
+  }
   struct Grp { uint32_t lo, hi, size; };
   Grp grp[kMaxFactors];
   uint32_t ng = 0, mergedGroups = 0;
   for (int hi = (int)p.N - 1; hi >= 0;) {
     uint32_t size = p.P[hi];
     int lo = hi;
-    const bool small = p.P[hi] == p.Q[hi] && isPow2(p.P[hi]) && p.P[hi] < target;
+    const bool small = p.P[hi] == p.Q[hi] && isPow2(p.P[hi]) && p.P[hi] < target && hi < keepFrom;
     if (small)
       while (lo > 0 && p.P[lo - 1] == p.Q[lo - 1] && isPow2(p.P[lo - 1]) && size * p.P[lo - 1] <= target &&
              (uint32_t)(hi - lo + 1) < kMaxMergeSources) {
@@ -740,6 +751,7 @@ fastKronError Handle::trySplitLeadingTrailing(const KronProblem& p, void* temp1,
   else if (tp == 32 || tp == 64)      maxT = 2;
   else if (p.dt == DType::F32) maxT = (tp == 8) ? 5 : (tp == 16) ? 4 : 0;
   else if (tp == 16)           maxT = 3;
+  else if (tp == 8)            maxT = 5;              // fp64: the whole-row kernel for five 8x8 factors
   // (few rows of 32^3, fp32: the pair kernel spreads them over more CUs than one workgroup per row does)
   if (p.dt == DType::F32 && tp == 32 && (uint64_t)p.M * (p.K() / 32768) * p.batch < 96) maxT = 2;
   // (few blocks of 16^4: the wave-per-block kernel for three factors spreads them over more CUs)
@@ -750,6 +762,7 @@ fastKronError Handle::trySplitLeadingTrailing(const KronProblem& p, void* temp1,
   uint32_t nT = 0;
   while (nT < maxT && nT < p.N && p.P[p.N - 1 - nT] == tp && p.Q[p.N - 1 - nT] == tp) nT++;
   if (nT < 2 || nT == p.N) return fastKronKernelNotFound;         // a chain of nT factors alone is a whole-row problem
+  if (p.dt == DType::F64 && tp == 8 && nT != 5) return fastKronKernelNotFound;   // (that kernel takes exactly five)
   const uint32_t g = p.N - nT;
   KronProblem q1, q2;
   if (!buildSplit(p, g, temp1, temp2, &q1, &q2)) return fastKronKernelNotFound;

@@ -272,6 +272,15 @@ def test_whole_row_kernel_for_five_8x8_fp64_factors(fk):
     assert fk.last_plan()[-1][2] == ROW_8X5_F64, fk.last_plan()
     check(fk, ko.MKM, 31, [8] * 5, [8] * 5, np.float64, alpha=1.0, beta=1.0, seed=49)
     assert ROW_8X5_F64 not in [k for _, _, k in fk.last_plan()], fk.last_plan()
+    # six and seven factors: the row kernel on the blocks of 32768 columns, the leading factor(s) across them
+    check(fk, ko.MKM, 5, [8] * 6, [8] * 6, np.float64, alpha=1.5, beta=0.5, seed=50)
+    plan = fk.last_plan()
+    assert len(plan) == 2 and plan[0] == (1, 5, ROW_8X5_F64), plan
+    check(fk, ko.MKM, 4, [8] * 6, [8] * 6, np.float64, alpha=1.0, beta=1.0, seed=51, opFs=ko.OP_T, y_is_z=True)
+    check(fk, ko.MKM, 2, [8] * 6, [8] * 6, np.float64, alpha=1.0, beta=0.0, seed=52, batch=2, share_f=True)
+    check(fk, ko.MKM, 1, [8] * 7, [8] * 7, np.float64, alpha=-1.0, beta=0.5, seed=53)
+    plan = fk.last_plan()
+    assert len(plan) == 2 and plan[0][2] == ROW_8X5_F64 and "64x64" in plan[1][2], plan
 
 
 RECT_PAIRS = [

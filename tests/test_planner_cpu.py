@@ -115,14 +115,21 @@ def test_two_part_plan_reads_leading_factors_with_stride_zero(planner):
 
 def test_fp64_rows_of_five_8x8_factors_get_the_whole_row_kernel(online_planner):
     """dgemkm 8x8^5 from 32 rows on: one launch of the fp64 row kernel on the chain as given (no 64x64 products); with
-    fewer rows, with a sixth factor or in the KMM layout the chain is merged as before."""
+    fewer rows, with eight factors or in the KMM layout the chain is merged as before."""
     row = "mkm_hip_gfx950_512_d_8x8_8x8_5_1x32768_valu_NN_strided_0_3"
     for M, opF in [(1024, capi.OP_N), (32, capi.OP_T)]:
         e, names, launches = plan(online_planner, "mkm", "d", M, [8] * 5, [8] * 5, opF=opF, beta=0.5, with_y=True)
         assert e == capi.SUCCESS and names == [row], names
     e, names, _ = plan(online_planner, "mkm", "d", 31, [8] * 5, [8] * 5)
     assert e == capi.SUCCESS and row not in names and any("64x64" in n for n in names), names
-    e, names, _ = plan(online_planner, "mkm", "d", 1024, [8] * 6, [8] * 6)
+    # six or seven factors: the row kernel on the blocks of 32768 columns, the leading factor(s) across the blocks
+    e, names, launches = plan(online_planner, "mkm", "d", 1024, [8] * 6, [8] * 6)
+    assert e == capi.SUCCESS and len(names) == 2 and names[0] == row and int(launches[0]["M"]) == 8192, (names, launches)
+    e, names, launches = plan(online_planner, "mkm", "d", 16, [8] * 7, [8] * 7)
+    assert e == capi.SUCCESS and len(names) == 2 and names[0] == row and "64x64" in names[1], names
+    e, names, _ = plan(online_planner, "mkm", "d", 3, [8] * 6, [8] * 6)           # 24 blocks: merged as before
+    assert e == capi.SUCCESS and row not in names and any("64x64" in n for n in names), names
+    e, names, _ = plan(online_planner, "mkm", "d", 16, [8] * 8, [8] * 8)
     assert e == capi.SUCCESS and row not in names, names
     e, names, _ = plan(online_planner, "kmm", "d", 1024, [8] * 5, [8] * 5)
     assert e == capi.SUCCESS and row not in names, names
