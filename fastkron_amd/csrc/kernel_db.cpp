@@ -221,10 +221,15 @@ static bool row32x3CanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo
   // a row is one workgroup's work for about 17 us: with few rows the pair kernel (a wave per 1024-column block) plus
   // one step across the blocks finishes sooner (measured crossover between 64 and 128 rows)
   if (dev.rulesOfThumb && (uint64_t)p.M * p.batch < kRow32MinRows) return false;
+  // the persistent form (four quarter buffers in LDS) from three rows per CU on; with fewer the two workgroups of a CU
+  // that start together are faster (768 rows 57.8 against 59.6 us, 512 rows 44.0 against 39.2)
+  if (k.threads == 1024 && (dev.ldsPerBlock < 143360 || (dev.rulesOfThumb && (uint64_t)p.M * p.batch < 3ull * dev.cus))) return false;
   return k.dt == p.dt;
 }
-static hipError_t row32x3Launch(const KernelInfo&, const StepArgs& a, hipStream_t s) { return launchRow32x3(a, s); }
-static bool row32x3Check(const KernelInfo&, const StepArgs& a) { return row32x3Supported(a); }
+static hipError_t row32x3Launch(const KernelInfo& k, const StepArgs& a, hipStream_t s) {
+  return k.threads == 1024 ? launchRow32x3p(a, s) : launchRow32x3(a, s);
+}
+static bool row32x3Check(const KernelInfo& k, const StepArgs& a) { return k.threads == 1024 ? row32x3pSupported(a) : row32x3Supported(a); }
 
 // ---- single-factor fp32 step for 64x64 and 128x128, whole-line accesses through LDS (variant 3: MKM, 4: KMM) ----
 static bool stepWideCanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, uint32_t hi, bool first, bool,
@@ -421,6 +426,14 @@ void registerRowKernels(std::vector<KernelInfo>& out) {
   k32.variant = 0; k32.canRun = row32CanRun; k32.launch = row32Launch; k32.check = row32Check;
   out.push_back(k32);
 
+  {
+    // ahead of the kernel with two workgroups of 8 waves per CU: chosen first where both apply
+    KernelInfo kp{};
+    kp.name = "mkm_hip_gfx950_1024_f_32x32_32x32_3_1x32768_mfma16x16x4_NN_strided_0_3";
+    kp.dt = DType::F32; kp.P = 32; kp.Q = 32; kp.fused = 3; kp.tileM = 1; kp.tileK = 32768; kp.threads = 1024;
+    kp.variant = 0; kp.canRun = row32x3CanRun; kp.launch = row32x3Launch; kp.check = row32x3Check;
+    out.push_back(kp);
+  }
   KernelInfo k323{};
   k323.name = "mkm_hip_gfx950_512_f_32x32_32x32_3_1x32768_mfma16x16x4_NN_strided_0_3";
   k323.dt = DType::F32; k323.P = 32; k323.Q = 32; k323.fused = 3; k323.tileM = 1; k323.tileK = 32768; k323.threads = 512;

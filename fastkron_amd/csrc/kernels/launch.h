@@ -95,6 +95,9 @@ bool row32x16x3Supported(const StepArgs& a);
 hipError_t launchRow32x16x3(const StepArgs& a, hipStream_t stream);
 bool row32x3Supported(const StepArgs& a);
 hipError_t launchRow32x3(const StepArgs& a, hipStream_t stream);
+// The same as one persistent workgroup of 16 waves per CU with the next row's loads in flight.
+bool row32x3pSupported(const StepArgs& a);
+hipError_t launchRow32x3p(const StepArgs& a, hipStream_t stream);
 
 // Two fused 32x32 or 64x64 factors (fp64 or fp32) on rows of exactly P*P columns (MKM layout), one wave per row.
 bool pairMfmaSupported(const StepArgs& a, DType dt);

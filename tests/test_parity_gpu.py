@@ -283,6 +283,28 @@ def test_whole_row_kernel_for_five_8x8_fp64_factors(fk):
     assert len(plan) == 2 and plan[0][2] == ROW_8X5_F64 and "64x64" in plan[1][2], plan
 
 
+ROW_32X3_PERSISTENT = "mkm_hip_gfx950_1024_f_32x32_32x32_3_1x32768_mfma16x16x4_NN_strided_0_3"
+
+
+def test_persistent_whole_row_kernel_for_three_32x32_factors(fk):
+    """32x32^3 fp32 from three rows per CU on: one persistent workgroup of 16 waves per CU that goes from row to row with
+    the next row's loads in flight (three block slots per lane, rotating with a period of three rows).  Row counts that
+    give the workgroups 3 or 4 rows each, batches whose factors are restaged between rows, Z == Y."""
+    check(fk, ko.MKM, 770, [32] * 3, [32] * 3, np.float32, alpha=1.5, beta=0.5, seed=81)
+    assert [k for _, _, k in fk.last_plan()] == [ROW_32X3_PERSISTENT], fk.last_plan()
+    check(fk, ko.MKM, 1030, [32] * 3, [32] * 3, np.float32, alpha=1.0, beta=0.0, seed=82, opFs=ko.OP_T)
+    assert [k for _, _, k in fk.last_plan()] == [ROW_32X3_PERSISTENT], fk.last_plan()
+    check(fk, ko.MKM, 97, [32] * 3, [32] * 3, np.float32, alpha=2.0, beta=1.0, seed=83, batch=8)          # factors per batch entry
+    assert [k for _, _, k in fk.last_plan()] == [ROW_32X3_PERSISTENT], fk.last_plan()
+    check(fk, ko.MKM, 390, [32] * 3, [32] * 3, np.float32, alpha=1.0, beta=-1.0, seed=84, batch=2, share_f=True, share_y=True)
+    check(fk, ko.MKM, 768, [32] * 3, [32] * 3, np.float32, alpha=-0.5, beta=2.0, seed=85, y_is_z=True)
+    check(fk, ko.MKM, 767, [32] * 3, [32] * 3, np.float32, alpha=1.0, beta=0.0, seed=86)                  # below: two workgroups per CU
+    assert ROW_32X3_PERSISTENT not in [k for _, _, k in fk.last_plan()], fk.last_plan()
+    # four factors: the kernel on the 32 blocks of every row, the leading factor across them
+    check(fk, ko.MKM, 25, [32] * 4, [32] * 4, np.float32, alpha=1.0, beta=0.5, seed=87)
+    assert fk.last_plan()[0][2] == ROW_32X3_PERSISTENT, fk.last_plan()
+
+
 RECT_PAIRS = [
     # P, Q, dtype: the shapes the pair kernel has exact rectangular tiles for
     (32, 64, np.float32), (64, 32, np.float32), (32, 64, np.float64),
