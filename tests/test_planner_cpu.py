@@ -138,6 +138,26 @@ def test_fp64_rows_of_five_8x8_factors_get_the_whole_row_kernel(online_planner):
     assert e == capi.SUCCESS and names == [row] and launches[0]["f_batch"] == [64] * 5, (names, launches)
 
 
+def test_rows_of_three_32x32_factors_choose_the_kernel_by_row_count(online_planner):
+    """sgemkm 32x32^3: from three rows per CU on the persistent kernel (one workgroup of 16 waves per CU), from 96 rows on
+    the kernel with two workgroups of 8 waves per CU, below that the pair kernel and a step; the same on the blocks of
+    a longer chain."""
+    pers = "mkm_hip_gfx950_1024_f_32x32_32x32_3_1x32768_mfma16x16x4_NN_strided_0_3"
+    two = "mkm_hip_gfx950_512_f_32x32_32x32_3_1x32768_mfma16x16x4_NN_strided_0_3"
+    for M, want in [(1024, [pers]), (768, [pers]), (767, [two]), (96, [two])]:
+        e, names, _ = plan(online_planner, "mkm", "s", M, [32] * 3, [32] * 3, beta=0.5, with_y=True)
+        assert e == capi.SUCCESS and names == want, (M, names)
+    e, names, _ = plan(online_planner, "mkm", "s", 95, [32] * 3, [32] * 3)
+    assert e == capi.SUCCESS and pers not in names and two not in names and len(names) == 2, names
+    e, names, launches = plan(online_planner, "mkm", "s", 24, [32] * 4, [32] * 4)          # 768 blocks
+    assert e == capi.SUCCESS and names[0] == pers and int(launches[0]["M"]) == 768, (names, launches)
+    e, names, _ = plan(online_planner, "mkm", "s", 96, [32] * 3, [32] * 3, batch=8)         # 768 rows in all
+    assert e == capi.SUCCESS and names == [pers], names
+    # a misaligned operand sends both away (16-byte accesses)
+    e, names, _ = plan(online_planner, "mkm", "s", 1024, [32] * 3, [32] * 3, offs={"x": 4})
+    assert e == capi.SUCCESS and pers not in names and two not in names, names
+
+
 def test_rectangular_pairs_get_the_pair_kernel_and_the_two_part_plan(online_planner):
     """Two 32x64 / 64x32 factors: one launch on exact tiles; three: the pair on the blocks of a row (M * P virtual rows of
     P*P columns, Q*Q out) and the leading factor across the blocks as a KMM problem with one batch entry per row."""
