@@ -71,8 +71,12 @@ template <> struct PairMfma<float> {
 // compute is exact zeros and is never stored).
 // Q != P: two factors of P x Q each (32 x 64, 64 x 32): the row is a P x P tile, the first product leaves P x Q, the
 // result is a Q x Q tile; exact sizes only.
-template <typename T, int P, bool HAS_Y, bool EXACT = true, int Q = P>
-__global__ __launch_bounds__(256, 2) void kron_pair_kernel(const StepArgs a) {
+// SPLIT: a row is shared by 2^splitArg waves, each of which loads the whole row and produces Q / 16 / 2^splitArg of
+// the 16-wide blocks of output columns q_a (few rows: more waves than rows, and the products of a block are one
+// dependent chain).
+template <typename T, int P, bool HAS_Y, bool EXACT = true, int Q = P, bool SPLIT = false>
+__global__ __launch_bounds__(256, 2) void kron_pair_kernel(const StepArgs a, const uint32_t splitArg) {
+  const uint32_t splitShift = SPLIT ? splitArg : 0;   // a constant in the kernels of whole rows
   static_assert(EXACT || P == Q, "the zero-padded form is square");
   using MF = PairMfma<T>;
   using Acc = typename MF::Acc;
@@ -116,7 +120,10 @@ __global__ __launch_bounds__(256, 2) void kron_pair_kernel(const StepArgs a) {
   __syncthreads();
 
   const uint32_t stride = gridDim.x * kPairWaves;
-  auto loadRow = [&](uint32_t row, T (&x)[PB][PC]) {
+  const uint32_t items = a.M << splitShift;         // an item: one row, one share of its q_a blocks
+  const int jbPer = QB >> splitShift;
+  auto loadRow = [&](uint32_t item, T (&x)[PB][PC]) {
+    const uint32_t row = item >> splitShift;
     const int lo = l0 & 15, hi = l0 >> 4;
     const T* xp = inB + (size_t)row * a.in_ldm + lo * R + PC * hi;
     if (!EXACT) {
@@ -137,17 +144,19 @@ __global__ __launch_bounds__(256, 2) void kron_pair_kernel(const StepArgs a) {
       }
   };
 
-  auto computeRow = [&](uint32_t row, const T (&x)[PB][PC]) {
+  auto computeRow = [&](uint32_t item, const T (&x)[PB][PC]) {
     // the lane id is made opaque once per row so that the LDS reads below (the same for every row) are
     // not hoisted out of the loop into registers
     int l = l0;
     asm volatile("" : "+v"(l));
     const int lo = l & 15, hi = l >> 4;
+    const uint32_t row = item >> splitShift;
+    const int jb0 = SPLIT ? (int)(item & ((1u << splitShift) - 1)) * jbPer : 0;
     T* out = outB + (size_t)row * a.out_ldm;
     const T* Y = HAS_Y ? YB + (size_t)row * a.y_ldm : nullptr;
 
 #pragma unroll 1
-    for (int jb = 0; jb < QB; jb++) {
+    for (int jb = jb0; jb < jb0 + jbPer; jb++) {
       int ofs = 16 * jb + lo;
       asm volatile("" : "+v"(ofs));
       Acc d1[PB];
@@ -199,19 +208,19 @@ __global__ __launch_bounds__(256, 2) void kron_pair_kernel(const StepArgs a) {
   // (the last row of a wave requests itself again rather than branching around the loads: a register that
   // keeps its old value on one path would stay live on every path)
   uint32_t row = blockIdx.x * kPairWaves + w;
-  if (row >= a.M) return;
-  auto nextOf = [&](uint32_t r) { return r + stride < a.M ? r + stride : r; };
+  if (row >= items) return;
+  auto nextOf = [&](uint32_t r) { return r + stride < items ? r + stride : r; };
   T xa[PB][PC], xb[PB][PC];
   loadRow(row, xa);
   while (true) {
     loadRow(nextOf(row), xb);
     computeRow(row, xa);
     row += stride;
-    if (row >= a.M) break;
+    if (row >= items) break;
     loadRow(nextOf(row), xa);
     computeRow(row, xb);
     row += stride;
-    if (row >= a.M) break;
+    if (row >= items) break;
   }
 }
 
@@ -432,7 +441,13 @@ static hipError_t launchPairT(const StepArgs& a, hipStream_t stream) {
   const size_t ldsBytes = 2 * P * Q * sizeof(T);
   uint32_t wgs = (uint32_t)cus * (P == 32 && Q == 32 ? 4 : 2);   // persistent; the 32x32 kernels need few registers
   if (a.batch > 1) wgs = (wgs + a.batch - 1) / a.batch;
-  const uint32_t need = (a.M + kPairWaves - 1) / kPairWaves;
+  // fewer rows than the waves of one workgroup per CU: the rows are shared out by blocks of output columns (a second
+  // workgroup of a CU starts microseconds behind the first, which costs more than the shorter chains gain)
+  uint32_t splitShift = 0;
+  while ((Q / 16) >> (splitShift + 1) >= 1 &&
+         ((uint64_t)a.M << (splitShift + 1)) * a.batch <= (uint64_t)cus * kPairWaves)
+    splitShift++;
+  const uint32_t need = ((a.M << splitShift) + kPairWaves - 1) / kPairWaves;
   if (wgs > need) wgs = need;
   if (wgs == 0) wgs = 1;
   dim3 grid(wgs, a.batch), block(256);
@@ -440,15 +455,22 @@ static hipError_t launchPairT(const StepArgs& a, hipStream_t stream) {
   const int devIdx = launchDeviceIndex();
   const bool y = a.y && a.epilogue;
   if (!attrOnce[y].done(devIdx)) {
-    hipError_t e = y ? hipFuncSetAttribute((const void*)kron_pair_kernel<T, P, true, EXACT, Q>,
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes)
-                     : hipFuncSetAttribute((const void*)kron_pair_kernel<T, P, false, EXACT, Q>,
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes);
-    if (e != hipSuccess) return e;
+    using Kernel = void (*)(const StepArgs, const uint32_t);
+    const Kernel all[4] = {kron_pair_kernel<T, P, false, EXACT, Q, false>, kron_pair_kernel<T, P, false, EXACT, Q, true>,
+                           kron_pair_kernel<T, P, true, EXACT, Q, false>, kron_pair_kernel<T, P, true, EXACT, Q, true>};
+    for (int k = 2 * y; k < 2 * y + 2; k++) {
+      hipError_t e = hipFuncSetAttribute((const void*)all[k], hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes);
+      if (e != hipSuccess) return e;
+    }
     attrOnce[y].mark(devIdx);
   }
-  if (y) hipLaunchKernelGGL((kron_pair_kernel<T, P, true, EXACT, Q>), grid, block, ldsBytes, stream, a);
-  else   hipLaunchKernelGGL((kron_pair_kernel<T, P, false, EXACT, Q>), grid, block, ldsBytes, stream, a);
+  if (y) {
+    if (splitShift) hipLaunchKernelGGL((kron_pair_kernel<T, P, true, EXACT, Q, true>), grid, block, ldsBytes, stream, a, splitShift);
+    else hipLaunchKernelGGL((kron_pair_kernel<T, P, true, EXACT, Q, false>), grid, block, ldsBytes, stream, a, 0u);
+  } else {
+    if (splitShift) hipLaunchKernelGGL((kron_pair_kernel<T, P, false, EXACT, Q, true>), grid, block, ldsBytes, stream, a, splitShift);
+    else hipLaunchKernelGGL((kron_pair_kernel<T, P, false, EXACT, Q, false>), grid, block, ldsBytes, stream, a, 0u);
+  }
   return hipGetLastError();
 }
 

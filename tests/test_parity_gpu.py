@@ -340,6 +340,22 @@ def test_pair_kernel_for_two_rectangular_factors(fk, P, Q, dt):
         check(fk, ko.MKM, 2, [P] * 3, [Q] * 3, dt, alpha=1.0, beta=0.0, seed=72, use_temp2=False)      # one temporary: no two-part plan
 
 
+@pytest.mark.parametrize("P,Q,dt", [(64, 64, np.float32), (32, 32, np.float32), (32, 32, np.float64),
+                                    (24, 24, np.float32), (24, 24, np.float64)] + RECT_PAIRS)
+def test_pair_kernel_rows_shared_between_waves(fk, P, Q, dt):
+    """With few rows the pair kernel hands each row to 2 or 4 waves, one share of the output column blocks each; with
+    more rows than one workgroup per CU holds waves, a wave produces whole rows.  Row counts on both sides of every
+    switch (256 CUs x 4 waves: 4 shares up to 256 rows, 2 up to 512), odd ones included."""
+    for i, M in enumerate((1, 3, 255, 256, 257, 511, 512, 513, 1025)):
+        if P == 64 and Q == 64 and M < 512:
+            continue                                   # (single steps by the rules of thumb)
+        check(fk, ko.MKM, M, [P] * 2, [Q] * 2, dt, alpha=1.0 + i, beta=0.5 * (i % 3), seed=300 + i)
+        plan = fk.last_plan()
+        assert len(plan) == 1 and "_2_1x" in plan[0][2], plan
+    check(fk, ko.MKM, 100, [P] * 2, [Q] * 2, dt, alpha=1.0, beta=1.0, seed=320, batch=3)
+    check(fk, ko.MKM, 200, [P] * 2, [Q] * 2, dt, alpha=1.0, beta=0.0, seed=321, batch=2, share_f=True)
+
+
 def test_whole_row_kernel_for_three_32x16_factors(fk):
     """32x16^3 fp32 rows (non-square, which the reference never fuses) run as ONE launch."""
     check(fk, ko.MKM, 5, [32] * 3, [16] * 3, np.float32, alpha=1.0, beta=0.0, seed=31)
