@@ -277,8 +277,14 @@ static bool pairCanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, u
   if (first && p.opX == 2) return false;
   // one wave per 64x64 block: with few blocks two single-factor launches, whose tiles are 16 times smaller, fill the
   // device better (tuned plans at 256 blocks: 1.4 times faster in fp32, 1.9 times in fp64; at 1024 blocks the pair wins)
-  // (fp64: two single steps on tiles passed through LDS also win at 1024 blocks, 36 against 44 us)
-  if (dev.rulesOfThumb && P == 64 && (uint64_t)p.M * p.batch < (p.dt == DType::F64 ? 2048u : 512u)) return false;
+  // fp64, a block per wave and two waves per SIMD: from 8 blocks per CU on; with up to 4 per CU two or four waves share a
+  // block and the pair wins again (1024 blocks: 25.8 against 31 us, 512: 17.3 against 22.4, 320: 16.2 against 18.1; at
+  // 256 blocks two single steps on tiles passed through LDS take 14.9 us and the pair does not beat them; between 4 and
+  // 8 blocks per CU a wave's chain of one whole block, 35 us, loses to them too)
+  if (dev.rulesOfThumb && P == 64) {
+    const uint64_t blocks = (uint64_t)p.M * p.batch, cus = (uint64_t)dev.cus;
+    if (p.dt == DType::F64 ? (4 * blocks < 5 * cus || (blocks > 4 * cus && blocks < 8 * cus)) : blocks < 2 * cus) return false;
+  }
   return dev.ldsPerBlock >= (int)(2 * k.P * k.P * 8 + 8 * 8192);
 }
 static hipError_t pairLaunch(const KernelInfo& k, const StepArgs& a, hipStream_t s) { return launchPairMfma(a, k.dt, s); }

@@ -230,9 +230,15 @@ constexpr int kPair64Waves = 8;                     // one workgroup of 8 waves 
 constexpr int kPair64XWords = 16 * 64;              // doubles of X staging per wave: 16 rows of the tile
 constexpr size_t kPair64LdsBytes = (2 * kP64 * kP64 + kPair64Waves * kPair64XWords) * sizeof(double);
 
-template <bool HAS_Y, int NT>
+// GN: 16-wide groups of output columns q_a a wave produces.  4: whole rows.  2 / 1: a row is shared by 2 / 4 waves, each
+// of which loads it whole and works on its own columns (for row counts that leave waves without a row: the products
+// of a row in one wave are latency bound, about 35 us whatever else runs).  Columns of group g and lane n: with
+// GN >= 2 the pairs 32*(g/2) + 2n + g%2 (128-bit accesses), with GN = 1 the 16 neighbours 16*g + n.
+template <bool HAS_Y, int NT, int GN = 4>
 __global__ __launch_bounds__(512, 2) void kron_pair64_f64_kernel(const StepArgs a) {
   constexpr int P = kP64;
+  constexpr int HN = GN >= 2 ? GN / 2 : 1;          // 128-bit column pairs (GN = 1: the one column) per lane
+  constexpr uint32_t SHARE = 4 / GN;                // waves per row
   extern __shared__ double pairLds[];
   double* fA = pairLds;                              // F_a[k_a][q_a], row-major
   double* fB = pairLds + P * P;                      // F_b[k_b][q_b] at k_b*64 + (q_b ^ 4*(k_b%4))
@@ -279,19 +285,33 @@ __global__ __launch_bounds__(512, 2) void kron_pair64_f64_kernel(const StepArgs 
     for (int j = 0; j < 8; j++) x[j] = FK_LD(NT, (const pd2*)(xp + j * 128));
   };
 
-  auto computeRow = [&](uint32_t row, uint32_t next) {
+  auto computeRow = [&](uint32_t item, uint32_t next) {
     // the lane id is made opaque once per row: the LDS reads of the factors are the same for every row and
     // must not be hoisted out of the loop into registers
     int l = l0;
     asm volatile("" : "+v"(l));
     const int i4 = l & 3, k4 = l >> 4, n16 = l & 15;  // operand lane = i + 4*blk + 16*k = n + 16*k
+    const uint32_t row = item / SHARE;
+    // first column of this wave's share, and the lane's place in a group
+    const int colB = (int)(item % SHARE) * (GN == 1 ? 16 : 32), colL = GN == 1 ? n16 : 2 * n16;
     double* out = outB + (size_t)row * a.out_ldm;
     const double* Y = HAS_Y ? YB + (size_t)row * a.y_ldm : nullptr;
 
     // staging position of element (r, col) of a 16-row part: r*64 + 16*k + ((c + 4*(r%4) + k) % 16),
     // col = 16*k + c: the 16 addresses (i, k) of one operand read fall into 16 different bank pairs
     const int wr = l >> 5, wk = (l & 31) >> 3, wc = 2 * (l & 7);
-    double d1[16][4];
+    double d1[16][GN];
+    auto loadB = [&](int c, double (&b)[GN]) {
+      if (GN == 1) {
+        b[0] = fA[(16 * k4 + c) * 64 + colB + colL];
+      } else {
+#pragma unroll
+        for (int h = 0; h < HN; h++) {
+          const pd2 v = *(const pd2*)&fA[(16 * k4 + c) * 64 + colB + 32 * h + colL];
+          b[2 * h] = v[0]; b[(2 * h + 1) % GN] = v[1];
+        }
+      }
+    };
 #pragma unroll
     for (int tb = 0; tb < 4; tb++) {
 #pragma unroll
@@ -300,39 +320,33 @@ __global__ __launch_bounds__(512, 2) void kron_pair64_f64_kernel(const StepArgs 
 #pragma unroll
         for (int e = 0; e < 2; e++) xs[r * 64 + 16 * wk + ((wc + e + 4 * (r & 3) + wk) & 15)] = x[j][e];
       }
-      if (tb < 3) loadPart(row, tb + 1); else loadPart(next, 0);
+      if (tb < 3) loadPart(row, tb + 1); else loadPart(next / SHARE, 0);
 #pragma unroll
       for (int tt = 0; tt < 4; tt++)
 #pragma unroll
-        for (int g = 0; g < 4; g++) d1[4 * tb + tt][g] = 0.0;
+        for (int g = 0; g < GN; g++) d1[4 * tb + tt][g] = 0.0;
       // operands of step c+1 are read before the products of step c are issued
-      double an[4], bn[4];
+      double an[4], bn[GN];
 #pragma unroll
       for (int tt = 0; tt < 4; tt++) an[tt] = xs[(4 * tt + i4) * 64 + 16 * k4 + ((4 * i4 + k4) & 15)];
-#pragma unroll
-      for (int h = 0; h < 2; h++) {
-        const pd2 v = *(const pd2*)&fA[(16 * k4) * 64 + 32 * h + 2 * n16];
-        bn[2 * h] = v[0]; bn[2 * h + 1] = v[1];
-      }
+      loadB(0, bn);
 #pragma unroll
       for (int c = 0; c < 16; c++) {
-        double ac[4], bc[4];
+        double ac[4], bc[GN];
 #pragma unroll
-        for (int tt = 0; tt < 4; tt++) { ac[tt] = an[tt]; bc[tt] = bn[tt]; }
+        for (int tt = 0; tt < 4; tt++) ac[tt] = an[tt];
+#pragma unroll
+        for (int g = 0; g < GN; g++) bc[g] = bn[g];
         if (c + 1 < 16) {
 #pragma unroll
           for (int tt = 0; tt < 4; tt++) an[tt] = xs[(4 * tt + i4) * 64 + 16 * k4 + ((c + 1 + 4 * i4 + k4) & 15)];
-#pragma unroll
-          for (int h = 0; h < 2; h++) {
-            const pd2 v = *(const pd2*)&fA[(16 * k4 + c + 1) * 64 + 32 * h + 2 * n16];
-            bn[2 * h] = v[0]; bn[2 * h + 1] = v[1];
-          }
+          loadB(c + 1, bn);
         }
         asm volatile("" ::: "memory");
 #pragma unroll
         for (int tt = 0; tt < 4; tt++)
 #pragma unroll
-          for (int g = 0; g < 4; g++)
+          for (int g = 0; g < GN; g++)
             d1[4 * tb + tt][g] = __builtin_amdgcn_mfma_f64_4x4x4f64(ac[tt], bc[g], d1[4 * tb + tt][g], 0, 0, 0);
       }
     }
@@ -349,11 +363,11 @@ __global__ __launch_bounds__(512, 2) void kron_pair64_f64_kernel(const StepArgs 
         fo[uu] = k4 * 64 + 16 * ub + 4 * (uu ^ k4) + i4;
         asm volatile("" : "+v"(fo[uu]));
       }
-      double acc[4][4];
+      double acc[4][GN];
 #pragma unroll
       for (int uu = 0; uu < 4; uu++)
 #pragma unroll
-        for (int g = 0; g < 4; g++) acc[uu][g] = 0.0;
+        for (int g = 0; g < GN; g++) acc[uu][g] = 0.0;
       double fn[4];
 #pragma unroll
       for (int uu = 0; uu < 4; uu++) fn[uu] = fB[fo[uu]];
@@ -370,44 +384,60 @@ __global__ __launch_bounds__(512, 2) void kron_pair64_f64_kernel(const StepArgs 
 #pragma unroll
         for (int uu = 0; uu < 4; uu++)
 #pragma unroll
-          for (int g = 0; g < 4; g++)
+          for (int g = 0; g < GN; g++)
             acc[uu][g] = __builtin_amdgcn_mfma_f64_4x4x4f64(fc[uu], d1[t][g], acc[uu][g], 0, 0, 0);
       }
       // q_b = 16ub + 4uu + orow; the products g = 2h, 2h+1 hold the neighbouring columns q_a = 32h + 2*ocol, +1
-      const int o0 = (16 * ub + orow) * 64 + 2 * ocol;
+      // (one group: the column 16*share + ocol)
+      const int o0 = (16 * ub + orow) * 64 + colB + (GN == 1 ? ocol : 2 * ocol);
       // Y in two halves, each read before the stores of its half (registers are short with Y)
 #pragma unroll
       for (int uh = 0; uh < 4; uh += 2) {
-        pd2 yv[2][2];
-        if (HAS_Y) {
+        if (GN == 1) {
+          double yv[2];
+          if (HAS_Y) {
+#pragma unroll
+            for (int uu = 0; uu < 2; uu++) yv[uu] = Y[o0 + 4 * (uh + uu) * 64];
+          }
+#pragma unroll
+          for (int uu = 0; uu < 2; uu++) {
+            double v = acc[uh + uu][0] * alpha;
+            if (HAS_Y) v += beta * yv[uu];
+            out[o0 + 4 * (uh + uu) * 64] = v;
+          }
+        } else {
+          pd2 yv[2][HN];
+          if (HAS_Y) {
+#pragma unroll
+            for (int uu = 0; uu < 2; uu++)
+#pragma unroll
+              for (int h = 0; h < HN; h++) yv[uu][h] = *(const pd2*)(Y + o0 + 4 * (uh + uu) * 64 + 32 * h);
+          }
 #pragma unroll
           for (int uu = 0; uu < 2; uu++)
 #pragma unroll
-            for (int h = 0; h < 2; h++) yv[uu][h] = *(const pd2*)(Y + o0 + 4 * (uh + uu) * 64 + 32 * h);
+            for (int h = 0; h < HN; h++) {
+              pd2 v = {acc[uh + uu][2 * h] * alpha, acc[uh + uu][(2 * h + 1) % GN] * alpha};
+              if (HAS_Y) v += beta * yv[uu][h];
+              FK_ST(NT, v, (pd2*)(out + o0 + 4 * (uh + uu) * 64 + 32 * h));
+            }
         }
-#pragma unroll
-        for (int uu = 0; uu < 2; uu++)
-#pragma unroll
-          for (int h = 0; h < 2; h++) {
-            pd2 v = {acc[uh + uu][2 * h] * alpha, acc[uh + uu][2 * h + 1] * alpha};
-            if (HAS_Y) v += beta * yv[uu][h];
-            FK_ST(NT, v, (pd2*)(out + o0 + 4 * (uh + uu) * 64 + 32 * h));
-          }
       }
     }
   };
 
+  const uint32_t items = a.M * SHARE;               // an item: one row, one share of its columns
   uint32_t row = blockIdx.x * kPair64Waves + w;
-  if (row >= a.M) return;
+  if (row >= items) return;
   // the last row of a wave prefetches its own first part again: no branch around memory operations
-  auto nextOf = [&](uint32_t r) { return r + stride < a.M ? r + stride : r; };
-  loadPart(row, 0);
+  auto nextOf = [&](uint32_t r) { return r + stride < items ? r + stride : r; };
+  loadPart(row / SHARE, 0);
   // The first row is peeled off the loop.  Loads and stores retire through one in-order counter and
   // the wait for a prefetched part is counted in younger operations; entering the loop only from a
   // complete row lets that count include the 64 stores issued behind the prefetch, so that the wait
   // at the top of a row does not drain the previous row's stores.
   computeRow(row, nextOf(row));
-  for (row += stride; row < a.M; row += stride) computeRow(row, nextOf(row));
+  for (row += stride; row < items; row += stride) computeRow(row, nextOf(row));
 }
 
 // Rectangular pairs with exact tiles: 32x64 and 64x32 in fp32, 32x64 in fp64 (a 64 x 64 tile of doubles, twice over
@@ -478,26 +508,33 @@ static hipError_t launchPair64(const StepArgs& a, hipStream_t stream) {
   const int cus = deviceCUs();
   uint32_t wgs = (uint32_t)cus;                     // persistent, one workgroup per CU
   if (a.batch > 1) wgs = (wgs + a.batch - 1) / a.batch;
-  const uint32_t need = (a.M + kPair64Waves - 1) / kPair64Waves;
+  // rows for at most half (a quarter) of the waves: two (four) waves per row
+  const uint64_t waves = (uint64_t)wgs * kPair64Waves;
+  const uint32_t share = 4ull * a.M <= waves ? 4 : 2ull * a.M <= waves ? 2 : 1;
+  const uint32_t need = (a.M * share + kPair64Waves - 1) / kPair64Waves;
   if (wgs > need) wgs = need;
   if (wgs == 0) wgs = 1;
   dim3 grid(wgs, a.batch), block(64 * kPair64Waves);
   static PerDeviceOnce attrOnce;
   const int devIdx = launchDeviceIndex();
   using Kernel = void (*)(const StepArgs);
-  static const Kernel kernels[2][3] = {
-      {kron_pair64_f64_kernel<false, 0>, kron_pair64_f64_kernel<false, 1>, kron_pair64_f64_kernel<false, 2>},
-      {kron_pair64_f64_kernel<true, 0>, kron_pair64_f64_kernel<true, 1>, kron_pair64_f64_kernel<true, 2>}};
+  // (the shared forms run on rows that stay in the caches: ordinary loads and stores)
+  static const Kernel kernels[2][5] = {
+      {kron_pair64_f64_kernel<false, 0>, kron_pair64_f64_kernel<false, 1>, kron_pair64_f64_kernel<false, 2>,
+       kron_pair64_f64_kernel<false, 0, 2>, kron_pair64_f64_kernel<false, 0, 1>},
+      {kron_pair64_f64_kernel<true, 0>, kron_pair64_f64_kernel<true, 1>, kron_pair64_f64_kernel<true, 2>,
+       kron_pair64_f64_kernel<true, 0, 2>, kron_pair64_f64_kernel<true, 0, 1>}};
   if (!attrOnce.done(devIdx)) {
     for (int y = 0; y < 2; y++)
-      for (int nt = 0; nt < 3; nt++) {
-        hipError_t e = hipFuncSetAttribute((const void*)kernels[y][nt], hipFuncAttributeMaxDynamicSharedMemorySize,
+      for (int k = 0; k < 5; k++) {
+        hipError_t e = hipFuncSetAttribute((const void*)kernels[y][k], hipFuncAttributeMaxDynamicSharedMemorySize,
                                            (int)kPair64LdsBytes);
         if (e != hipSuccess) return e;
       }
     attrOnce.mark(devIdx);
   }
-  hipLaunchKernelGGL(kernels[(a.y && a.epilogue) ? 1 : 0][streamMode(a)], grid, block, kPair64LdsBytes, stream, a);
+  const int which = share == 4 ? 4 : share == 2 ? 3 : streamMode(a);
+  hipLaunchKernelGGL(kernels[(a.y && a.epilogue) ? 1 : 0][which], grid, block, kPair64LdsBytes, stream, a);
   return hipGetLastError();
 }
 

@@ -356,6 +356,22 @@ def test_pair_kernel_rows_shared_between_waves(fk, P, Q, dt):
     check(fk, ko.MKM, 200, [P] * 2, [Q] * 2, dt, alpha=1.0, beta=0.0, seed=321, batch=2, share_f=True)
 
 
+def test_pair64_fp64_blocks_shared_between_waves(fk):
+    """dgemkm 64x64^2 with few blocks: four waves per block up to 2 blocks per CU, two up to 4 (each wave loads the block
+    whole and produces its own output columns); a block per wave from 8 per CU on."""
+    pair = "mkm_hip_gfx950_512_d_64x64_64x64_2_1x4096_mfma4x4x4_NN_strided_0_3"
+    for i, M in enumerate((320, 511, 512, 513, 1023, 1024, 2049)):
+        check(fk, ko.MKM, M, [64] * 2, [64] * 2, np.float64, alpha=1.0 + i, beta=0.5 * (i % 3), seed=340 + i)
+        assert [k for _, _, k in fk.last_plan()] == [pair], (M, fk.last_plan())
+    check(fk, ko.MKM, 200, [64] * 2, [64] * 2, np.float64, alpha=1.0, beta=1.0, seed=350, batch=3)     # 600 blocks
+    assert [k for _, _, k in fk.last_plan()] == [pair], fk.last_plan()
+    check(fk, ko.MKM, 170, [64] * 2, [64] * 2, np.float64, alpha=-1.0, beta=0.5, seed=351, batch=2, share_f=True, opFs=ko.OP_T)
+    assert [k for _, _, k in fk.last_plan()] == [pair], fk.last_plan()
+    check(fk, ko.MKM, 400, [64] * 2, [64] * 2, np.float64, alpha=1.5, beta=0.5, seed=352, y_is_z=True)
+    check(fk, ko.MKM, 6, [64] * 3, [64] * 3, np.float64, alpha=1.0, beta=0.0, seed=353)                # 384 blocks of a chain
+    assert fk.last_plan()[0][2] == pair, fk.last_plan()
+
+
 def test_whole_row_kernel_for_three_32x16_factors(fk):
     """32x16^3 fp32 rows (non-square, which the reference never fuses) run as ONE launch."""
     check(fk, ko.MKM, 5, [32] * 3, [16] * 3, np.float32, alpha=1.0, beta=0.0, seed=31)
@@ -600,7 +616,9 @@ def test_pair_kernel(fk, M, P, dt):
     """Two fused 64x64 / 32x32 factors (fp64, fp32): chained matrix-core products, one wave per row."""
     check(fk, ko.MKM, M, [P, P], [P, P], dt, alpha=1.5, beta=0.5, seed=121)
     plan = fk.last_plan()
-    if P == 64 and M < (2048 if dt == np.float64 else 512):   # few 64x64 blocks: two single-factor launches fill the device better than a wave per block
+    # few 64x64 blocks: two single-factor launches fill the device better than a wave per block (fp64: except where
+    # two or four waves share a block, 320 to 1024 blocks)
+    if P == 64 and (M < 512 if dt == np.float32 else (M < 320 or 1024 < M < 2048)):
         assert len(plan) == 2 and all("_64x64_64x64_1_" in k for _, _, k in plan), plan
     else:
         assert len(plan) == 1 and f"_2_1x{P * P}_" in plan[0][2], plan

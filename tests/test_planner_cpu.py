@@ -178,6 +178,18 @@ def test_rectangular_pairs_get_the_pair_kernel_and_the_two_part_plan(online_plan
     assert e == capi.SUCCESS and len(names) == 3, names
 
 
+def test_pairs_of_64x64_fp64_factors_by_block_count(online_planner):
+    """dgemkm 64x64^2: the pair kernel from 8 blocks per CU on (a block per wave) and between 1.25 and 4 blocks per CU
+    (a block shared by waves); otherwise two single steps."""
+    pair = "mkm_hip_gfx950_512_d_64x64_64x64_2_1x4096_mfma4x4x4_NN_strided_0_3"
+    for M, fused in [(256, False), (319, False), (320, True), (512, True), (1024, True), (1025, False), (2047, False),
+                     (2048, True), (16384, True)]:
+        e, names, _ = plan(online_planner, "mkm", "d", M, [64] * 2, [64] * 2)
+        assert e == capi.SUCCESS and (names == [pair]) == fused and len(names) == (1 if fused else 2), (M, names)
+    e, names, launches = plan(online_planner, "mkm", "d", 8, [64] * 3, [64] * 3)            # 512 blocks of a longer chain
+    assert e == capi.SUCCESS and names[0] == pair and int(launches[0]["M"]) == 512, (names, launches)
+
+
 # ---- kernels with 16-byte global accesses are only chosen for buffers that allow them ----
 VECTOR_CASES = [
     # (label, mm, dt, M, Ps, Qs, batch, beta, substring of the kernel expected on aligned buffers)
