@@ -267,7 +267,7 @@ static bool pairCanRun(const KernelInfo& k, const KronProblem& p, uint32_t lo, u
     // two rectangular factors of exactly the kernel's shape (32x64, 64x32): rows of P*P elements become Q*Q
     for (uint32_t i = lo; i <= hi; i++) if (p.P[i] != k.P || p.Q[i] != k.Q) return false;
     if (p.colsBefore(hi) != (uint64_t)k.P * k.P) return false;
-    return !(first && p.opX == 2) && dev.ldsPerBlock >= (int)(2 * k.P * k.Q * 8);
+    return !(first && p.opX == 2) && dev.ldsPerBlock >= (int)(2 * k.P * k.Q * 8 + 4 * 16 * (k.P + 4) * 8);   // factors and the waves' stages
   }
   // the 32x32 kernel also takes factors of 17x17 ... 31x31, zero-padded to its tile
   const uint32_t P = p.P[hi];

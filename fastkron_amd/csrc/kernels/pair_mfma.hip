@@ -92,6 +92,9 @@ __global__ __launch_bounds__(256, 2) void kron_pair_kernel(const StepArgs a, con
   const int l0 = tid & 63;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const uint32_t bt = blockIdx.y;
+  // exact tiles: a wave's own stage for 16 rows of its tile, 16 bytes of padding per row
+  constexpr int kPitch = P + VE;
+  T* stage = fB + P * Q + w * (16 * kPitch);
 
   const T* inB = (const T*)a.in + (size_t)bt * a.in_batch;
   T* outB = (T*)a.out + (size_t)bt * a.out_batch;
@@ -122,11 +125,15 @@ __global__ __launch_bounds__(256, 2) void kron_pair_kernel(const StepArgs a, con
   const uint32_t stride = gridDim.x * kPairWaves;
   const uint32_t items = a.M << splitShift;         // an item: one row, one share of its q_a blocks
   const int jbPer = QB >> splitShift;
+  // A row arrives in whole 1 KB pieces, lane l the 16 bytes l of a piece (an instruction that gave each lane 16 bytes
+  // of its own tile row, 16 rows to a wave, kept the address path of the CU busy for 40 % of the kernel's time), and is
+  // turned into operands through the stage, 16 tile rows at a time: lane (lo, hi) holds the columns PC*hi .. PC*hi+PC-1
+  // of the rows 16g + lo.  The padded form loads its operands element by element.
   auto loadRow = [&](uint32_t item, T (&x)[PB][PC]) {
     const uint32_t row = item >> splitShift;
-    const int lo = l0 & 15, hi = l0 >> 4;
-    const T* xp = inB + (size_t)row * a.in_ldm + lo * R + PC * hi;
     if (!EXACT) {
+      const int lo = l0 & 15, hi = l0 >> 4;
+      const T* xp = inB + (size_t)row * a.in_ldm + lo * R + PC * hi;
 #pragma unroll
       for (int g = 0; g < PB; g++)
 #pragma unroll
@@ -134,14 +141,44 @@ __global__ __launch_bounds__(256, 2) void kron_pair_kernel(const StepArgs a, con
           x[g][c] = (16 * g + lo < R && PC * hi + c < R) ? xp[g * 16 * R + c] : (T)0;
       return;
     }
+    const VT* src = (const VT*)(inB + (size_t)row * a.in_ldm) + l0;
 #pragma unroll
     for (int g = 0; g < PB; g++)
 #pragma unroll
       for (int c = 0; c < PC; c += VE) {
-        const VT v = *(const VT*)(xp + g * 16 * P + c);
+        const VT v = src[64 * (g * (PC / VE) + c / VE)];
 #pragma unroll
         for (int e = 0; e < VE; e++) x[g][c + e] = v[e];
       }
+  };
+  auto toOperands = [&](const T (&raw)[PB][PC], T (&x)[PB][PC]) {
+    if (!EXACT) {
+#pragma unroll
+      for (int g = 0; g < PB; g++)
+#pragma unroll
+        for (int c = 0; c < PC; c++) x[g][c] = raw[g][c];
+      return;
+    }
+    constexpr int CPR = P / VE;                     // 16-byte pieces of a tile row
+    const int lo = l0 & 15, hi = l0 >> 4;
+    T* wr = stage + (l0 / CPR) * kPitch + (l0 % CPR) * VE;
+    const T* rd = stage + lo * kPitch + PC * hi;
+#pragma unroll
+    for (int g = 0; g < PB; g++) {
+#pragma unroll
+      for (int c = 0; c < PC; c += VE) {
+        VT v;
+#pragma unroll
+        for (int e = 0; e < VE; e++) v[e] = raw[g][c + e];
+        *(VT*)(wr + (c / VE) * (64 / CPR) * kPitch) = v;
+      }
+#pragma unroll
+      for (int c = 0; c < PC; c += VE) {
+        const VT v = *(const VT*)(rd + c);
+#pragma unroll
+        for (int e = 0; e < VE; e++) x[g][c + e] = v[e];
+      }
+    }
   };
 
   auto computeRow = [&](uint32_t item, const T (&x)[PB][PC]) {
@@ -155,33 +192,89 @@ __global__ __launch_bounds__(256, 2) void kron_pair_kernel(const StepArgs a, con
     T* out = outB + (size_t)row * a.out_ldm;
     const T* Y = HAS_Y ? YB + (size_t)row * a.y_ldm : nullptr;
 
-#pragma unroll 1
+    // Factor operands come from LDS one group of products ahead: those of group n+1 are requested before the
+    // products of group n are issued (left to itself the compiler requests an operand right in front of the two
+    // products that take it, and the wave sits out an LDS round trip per 64 cycles of matrix work).
+    auto readA = [&](int jb, int cg, T (&b)[4]) {        // product 1: F_a rows PC*hi + 4cg .. +3, column 16jb + lo
+#pragma unroll
+      for (int cc = 0; cc < 4; cc++) b[cc] = fA[(PC * hi + 4 * cg + cc) * Q + 16 * jb + lo];
+    };
+    auto readB = [&](int step, T (&f)[4][2]) {           // product 2: step = (pair of column blocks, row block g)
+      const int jb2 = 2 * (step / PB), g = step % PB;
+#pragma unroll
+      for (int r = 0; r < 4; r++)
+#pragma unroll
+        for (int u = 0; u < 2; u++) f[r][u] = fB[(16 * g + MF::row(r, hi)) * Q + 16 * (jb2 + u) + lo];
+    };
+    constexpr int CG = PC / 4, STEPS = (QB / 2) * PB;
+    // fp32: the operands of product 2 change places, which leaves the result transposed in the accumulators, a lane's
+    // four registers four neighbouring columns q_a: 16-byte stores, a quarter of the store instructions (the fp64
+    // instruction spreads a lane's registers over rows 4 apart either way)
+    constexpr bool kTransposed = sizeof(T) == 4 && EXACT;
+    T bn[4], fn[4][2];
+    readA(jb0, 0, bn);
+    // whole rows: unrolled, so that the stores of a row are counted and the wait for the next row's loads, which are
+    // older, does not drain them (loads and stores share one in-order counter; behind a loop the wait is for all)
+#pragma unroll
     for (int jb = jb0; jb < jb0 + jbPer; jb++) {
-      int ofs = 16 * jb + lo;
-      asm volatile("" : "+v"(ofs));
+      const int ofs = 16 * jb + lo;
       Acc d1[PB];
 #pragma unroll
       for (int g = 0; g < PB; g++) d1[g] = (Acc){0, 0, 0, 0};
 #pragma unroll
-      for (int c = 0; c < PC; c++) {
-        const T b = fA[(PC * hi + c) * Q + ofs];
+      for (int cg = 0; cg < CG; cg++) {
+        T bc[4];
 #pragma unroll
-        for (int g = 0; g < PB; g++) d1[g] = MF::mma(x[g][c], b, d1[g]);
+        for (int cc = 0; cc < 4; cc++) bc[cc] = bn[cc];
+        if (cg + 1 < CG) readA(jb, cg + 1, bn); else readB(0, fn);
+        asm volatile("" ::: "memory");
+#pragma unroll
+        for (int cc = 0; cc < 4; cc++)
+#pragma unroll
+          for (int g = 0; g < PB; g++) d1[g] = MF::mma(x[g][4 * cg + cc], bc[cc], d1[g]);
       }
       // register r of d1[g] holds the rows k_b = 16g + row(r, hi): the B operand of product 2 for them;
       // two independent accumulator chains at a time
+      Acc acc[2];
 #pragma unroll
-      for (int jb2 = 0; jb2 < QB; jb2 += 2) {
-        Acc acc[2] = {(Acc){0, 0, 0, 0}, (Acc){0, 0, 0, 0}};
+      for (int step = 0; step < STEPS; step++) {
+        const int jb2 = 2 * (step / PB), g = step % PB;
+        if (g == 0) { acc[0] = (Acc){0, 0, 0, 0}; acc[1] = (Acc){0, 0, 0, 0}; }
+        T fc[4][2];
 #pragma unroll
-        for (int g = 0; g < PB; g++)
+        for (int r = 0; r < 4; r++)
 #pragma unroll
-          for (int r = 0; r < 4; r++)
+          for (int u = 0; u < 2; u++) fc[r][u] = fn[r][u];
+        // (behind the last block of columns the request runs into the rows of F_b: inside LDS, never used)
+        if (step + 1 < STEPS) readB(step + 1, fn); else readA(jb + 1, 0, bn);
+        asm volatile("" ::: "memory");
 #pragma unroll
-            for (int u = 0; u < 2; u++) {
-              const T fa = fB[(16 * g + MF::row(r, hi)) * Q + 16 * (jb2 + u) + lo];
-              acc[u] = MF::mma(fa, d1[g][r], acc[u]);
+        for (int r = 0; r < 4; r++)
+#pragma unroll
+          for (int u = 0; u < 2; u++)
+            acc[u] = kTransposed ? MF::mma(d1[g][r], fc[r][u], acc[u]) : MF::mma(fc[r][u], d1[g][r], acc[u]);
+        if (g != PB - 1) continue;
+        if constexpr (kTransposed) {
+          // lane (lo, hi), register e: Z[q_b = 16*(jb2+u) + lo][q_a = 16*jb + 4*hi + e], four neighbours per lane
+#pragma unroll
+          for (int u = 0; u < 2; u++) {
+            const int qb = 16 * (jb2 + u) + lo, qa = 16 * jb + 4 * hi;
+            if (EXACT) {
+              Acc v = acc[u] * alpha;
+              if (HAS_Y) v += beta * *(const Acc*)(Y + qb * RO + qa);
+              *(Acc*)(out + qb * RO + qa) = v;
+            } else {
+#pragma unroll
+              for (int e = 0; e < 4; e++)
+                if (qb < R && qa + e < R) {
+                  T v = acc[u][e] * alpha;
+                  if (HAS_Y) v += beta * Y[qb * RO + qa + e];
+                  out[qb * RO + qa + e] = v;
+                }
             }
+          }
+          continue;
+        }
         T yv[2][4];
         if (HAS_Y) {
 #pragma unroll
@@ -204,24 +297,24 @@ __global__ __launch_bounds__(256, 2) void kron_pair_kernel(const StepArgs a, con
     }
   };
 
-  // register double buffer over rows: the next row streams in under the products of the current one
-  // (the last row of a wave requests itself again rather than branching around the loads: a register that
-  // keeps its old value on one path would stay live on every path)
+  // the next row streams into registers under the products of the current one (the last row of a wave requests
+  // itself again rather than branching around the loads)
   uint32_t row = blockIdx.x * kPairWaves + w;
   if (row >= items) return;
   auto nextOf = [&](uint32_t r) { return r + stride < items ? r + stride : r; };
-  T xa[PB][PC], xb[PB][PC];
-  loadRow(row, xa);
-  while (true) {
-    loadRow(nextOf(row), xb);
-    computeRow(row, xa);
-    row += stride;
-    if (row >= items) break;
-    loadRow(nextOf(row), xa);
-    computeRow(row, xb);
-    row += stride;
-    if (row >= items) break;
-  }
+  T raw[PB][PC];
+  loadRow(row, raw);
+  auto oneRow = [&](uint32_t r) {
+    T x[PB][PC];
+    toOperands(raw, x);
+    loadRow(nextOf(r), raw);
+    computeRow(r, x);
+  };
+  // The first row is peeled off the loop.  Loads and stores retire through one in-order counter and the wait for the
+  // prefetched row is counted in younger operations: entering the loop only behind a complete row lets that count
+  // include the row's stores (otherwise the loop's wait is the first row's, which drains every store).
+  oneRow(row);
+  for (row += stride; row < items; row += stride) oneRow(row);
 }
 
 
@@ -458,9 +551,9 @@ bool pairMfmaSupported(const StepArgs& a, DType dt) {
   if (P < 32) return a.batch <= 65535;                                                // padded form: element-wise accesses
   const uint64_t vmask = 16 / dtypeSize(dt) - 1;                                      // 128-bit loads
   if (((uintptr_t)a.in & 15) || ((uint64_t)a.in_ldm & vmask) || (a.in_batch & vmask)) return false;
-  if (dt == DType::F64 && P == 64 && Q == 64) {                                       // and 128-bit stores / Y loads
-    if (((uintptr_t)a.out & 15) || ((uint64_t)a.out_ldm & 1) || (a.out_batch & 1)) return false;
-    if (a.y && (((uintptr_t)a.y & 15) || ((uint64_t)a.y_ldm & 1) || (a.y_batch & 1))) return false;
+  if (dt == DType::F32 || (P == 64 && Q == 64)) {                                     // and 128-bit stores / Y loads
+    if (((uintptr_t)a.out & 15) || ((uint64_t)a.out_ldm & vmask) || (a.out_batch & vmask)) return false;
+    if (a.y && (((uintptr_t)a.y & 15) || ((uint64_t)a.y_ldm & vmask) || (a.y_batch & vmask))) return false;
   }
   return a.batch <= 65535;
 }
@@ -468,7 +561,7 @@ bool pairMfmaSupported(const StepArgs& a, DType dt) {
 template <typename T, int P, bool EXACT = true, int Q = P>
 static hipError_t launchPairT(const StepArgs& a, hipStream_t stream) {
   const int cus = deviceCUs();
-  const size_t ldsBytes = 2 * P * Q * sizeof(T);
+  const size_t ldsBytes = (2 * P * Q + (EXACT ? kPairWaves * 16 * (P + 16 / sizeof(T)) : 0)) * sizeof(T);
   uint32_t wgs = (uint32_t)cus * (P == 32 && Q == 32 ? 4 : 2);   // persistent; the 32x32 kernels need few registers
   if (a.batch > 1) wgs = (wgs + a.batch - 1) / a.batch;
   // fewer rows than the waves of one workgroup per CU: the rows are shared out by blocks of output columns (a second
