@@ -110,17 +110,29 @@ __global__ __launch_bounds__(256, 2) void kron_kmm16x2_kernel(const StepArgs a, 
     if (!EXACT) xp += sliceFix;
   };
 
-  for (uint32_t t = blockIdx.x * kK2Waves + w; t < totalTiles; t += nWaves) {
+  // first row of tile t that this lane reads
+  auto tileRows = [&](uint32_t t) {
+    const uint64_t s = t / mTiles;
+    const uint32_t m0 = (uint32_t)(t - s * mTiles) * (16 * JW);
+    const uint32_t m = (JW == 2 || m0 + lo < M) ? m0 + JW * lo : m0;
+    return inB + m + (s * (uint64_t)(P * P) + hi) * (uint64_t)a.in_ldc;
+  };
+  // The first slices of a tile are requested while the tile before it is still in its vector-ALU and store phase
+  // (the window's registers are free from the last matrix product on): a tile that requested them at its own start
+  // sat out a memory round trip, behind the stores of the tile before, with nothing else in flight.
+  T xw[kK2Win][JW][4];
+  uint32_t t = blockIdx.x * kK2Waves + w;
+  if (t >= totalTiles) return;
+  const T* xp = tileRows(t);
+#pragma unroll
+  for (int k = 0; k < kK2Win; k++) loadSlice(xp, xw[k]);
+  for (; t < totalTiles; t += nWaves) {
     const uint64_t s = t / mTiles;
     const uint32_t m0 = (uint32_t)(t - s * mTiles) * (16 * JW);
     const bool mOk = JW == 2 || m0 + lo < M;                      // two columns per lane: whole tiles only
     const uint32_t m = mOk ? m0 + JW * lo : m0;
-    const T* xp = inB + m + (s * (uint64_t)(P * P) + hi) * (uint64_t)a.in_ldc;
 
     T z[JW][16][4];
-    T xw[kK2Win][JW][4];
-#pragma unroll
-    for (int k = 0; k < kK2Win; k++) loadSlice(xp, xw[k]);
 #pragma unroll
     for (int k0 = 0; k0 < 16; k0++) {
       T x[JW][4];
@@ -141,6 +153,10 @@ __global__ __launch_bounds__(256, 2) void kron_kmm16x2_kernel(const StepArgs a, 
       }
       __builtin_amdgcn_sched_barrier(0);             // keeps the loads of later slices from being hoisted up here
     }
+    // (behind the last tile of a wave the requests go to that tile's own rows again and are dropped)
+    xp = tileRows(t + nWaves < totalTiles ? t + nWaves : t);
+#pragma unroll
+    for (int k = 0; k < kK2Win; k++) loadSlice(xp, xw[k]);
 
     // ---- k0 on the vector ALU, one q0 at a time, and the stores ----
     // output row (q0, q1 = row(r, hi)): a running pointer per lane, 16 rows further with every q0
